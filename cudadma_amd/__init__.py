@@ -1,0 +1,26 @@
+"""cudadma_amd: Python side of the hipDMA host drivers (libcudadma_amd.so).
+
+The device library itself is header-only C++ (include/hipDMA.h).  This package
+only loads the C ABI declared in include/cudadma_amd.h with ctypes and wraps it
+for tests and benchmarks; PyTorch is used by callers for device memory and
+streams, never for compute.  Loading fails loudly when the shared library has
+not been built: there is no CPU fallback.
+"""
+from ._lib import (  # noqa: F401
+    CALL_GLOBAL,
+    CALL_LDS_DIRECT,
+    CALL_QUALIFIED,
+    CALL_UNQUALIFIED,
+    PATTERN_GATHER,
+    PATTERN_HALO,
+    PATTERN_SCATTER,
+    PATTERN_SEQUENTIAL,
+    PATTERN_STRIDED,
+    Case,
+    CudaDMAError,
+    PlanQuery,
+    RunArgs,
+    lib,
+    lib_path,
+)
+from . import harness, plan, workloads  # noqa: F401

@@ -1,0 +1,118 @@
+"""ctypes binding of include/cudadma_amd.h."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+PATTERN_SEQUENTIAL, PATTERN_STRIDED, PATTERN_GATHER, PATTERN_SCATTER, PATTERN_HALO = range(5)
+CALL_UNQUALIFIED, CALL_GLOBAL, CALL_QUALIFIED, CALL_LDS_DIRECT = range(4)
+
+PATTERN_NAMES = {
+    PATTERN_SEQUENTIAL: "sequential",
+    PATTERN_STRIDED: "strided",
+    PATTERN_GATHER: "gather",
+    PATTERN_SCATTER: "scatter",
+    PATTERN_HALO: "halo",
+}
+
+
+class CudaDMAError(RuntimeError):
+    pass
+
+
+class Case(ctypes.Structure):
+    """struct cudadma_case"""
+    _fields_ = [(n, ctypes.c_int) for n in (
+        "pattern", "warp_specialized", "level", "alignment", "bytes_per_thread", "bytes_per_elmt",
+        "dma_threads", "num_elmts", "radius", "corners", "dimx", "dimy")]
+
+    def __repr__(self):
+        return "Case(" + ", ".join(f"{n}={getattr(self, n)}" for n, _ in self._fields_) + ")"
+
+
+class PlanQuery(ctypes.Structure):
+    """struct cudadma_plan_query"""
+    _fields_ = [(n, ctypes.c_int) for n in (
+        "pattern", "alignment", "bytes_per_thread", "bytes_per_elmt", "dma_threads", "num_elmts",
+        "src_stride", "dst_stride", "radius", "corners", "dimx", "dimy", "pitch")] + [("index", ctypes.c_void_p)]
+
+
+class RunArgs(ctypes.Structure):
+    """struct cudadma_run"""
+    _fields_ = [
+        ("d_in", ctypes.c_void_p), ("d_out", ctypes.c_void_p), ("d_index", ctypes.c_void_p),
+        ("lds_bytes", ctypes.c_int), ("src_offset_bytes", ctypes.c_int), ("dst_offset_bytes", ctypes.c_int),
+        ("src_stride", ctypes.c_int), ("dst_stride", ctypes.c_int), ("pitch", ctypes.c_int),
+        ("call_style", ctypes.c_int), ("two_phase", ctypes.c_int), ("reps", ctypes.c_int),
+        ("rep_src_bytes", ctypes.c_int), ("rep_index_elmts", ctypes.c_int),
+    ]
+
+
+def lib_path():
+    return os.path.join(_HERE, "libcudadma_amd.so")
+
+
+_lib = None
+
+
+def lib():
+    """The loaded shared library; raises when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise CudaDMAError(
+            f"{path} is missing: build it with `make -C cudadma_amd/csrc` "
+            "(or python -c 'import __graft_entry__ as g; g.build()'); there is no fallback path")
+    L = ctypes.CDLL(path)
+    vp, ci, cs = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    L.cudadma_last_error.restype = ctypes.c_char_p
+    L.cudadma_last_error.argtypes = []
+    L.cudadma_device_cus.restype = ci
+    L.cudadma_num_cases.restype = ci
+    L.cudadma_get_case.restype = ci
+    L.cudadma_get_case.argtypes = [ci, ctypes.POINTER(Case)]
+    L.cudadma_run_case.restype = ci
+    L.cudadma_run_case.argtypes = [ci, ctypes.POINTER(RunArgs), vp]
+    for name, argtypes in _WORKLOAD_SIGNATURES.items():
+        fn = getattr(L, name)
+        fn.restype = ci
+        fn.argtypes = argtypes
+    L.cudadma_plan_map.restype = ci
+    L.cudadma_plan_map.argtypes = [ctypes.POINTER(PlanQuery), ctypes.c_longlong, ctypes.c_longlong, vp, cs,
+                                   ctypes.POINTER(ci)]
+    L.cudadma_diagnose.restype = ci
+    L.cudadma_diagnose.argtypes = [ci] * 8
+    L.cudadma_variant_name.restype = ctypes.c_char_p
+    L.cudadma_variant_name.argtypes = [ci, ci]
+    _lib = L
+    return L
+
+
+_vp, _ci, _cs, _u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_uint64
+
+# name -> argtypes of the workload entry points (all return int)
+_WORKLOAD_SIGNATURES = {
+    "cudadma_fill_uniform": [_vp, _cs, _u64, _vp],
+    "cudadma_fill_indices": [_vp, _cs, ctypes.c_uint32, _u64, _vp],
+    "cudadma_plain_copy": [_vp, _vp, _cs, _vp],
+    "cudadma_num_variants": [_ci],
+    "cudadma_set_workgroups_per_cu": [_ci],
+    "cudadma_sequential_copy": [_vp, _vp, _cs, _ci, _vp],
+    "cudadma_strided_transpose": [_vp, _vp, _ci, _ci, _vp],
+    "cudadma_gather_copy": [_vp, _vp, _vp, _cs, _cs, _ci, _vp],
+    "cudadma_gather_rowsum": [_vp, _vp, _vp, _cs, _cs, _ci, _vp],
+    "cudadma_halo_stencil": [_vp, _vp, _ci, _ci, _ci, _ci, _vp],
+}
+
+
+def check(rc):
+    if rc != 0:
+        raise CudaDMAError(f"libcudadma_amd error {rc}: {lib().cudadma_last_error().decode()}")
+
+
+def exported_symbols():
+    """Every extern "C" symbol include/cudadma_amd.h declares."""
+    return ["cudadma_last_error", "cudadma_device_cus", "cudadma_num_cases", "cudadma_get_case",
+            "cudadma_run_case", "cudadma_variant_name", "cudadma_plan_map", "cudadma_diagnose"] + list(_WORKLOAD_SIGNATURES)

@@ -1,0 +1,114 @@
+// Case registry and C entry points of the known-answer harness.
+#include "harness.hpp"
+#include <algorithm>
+#include <vector>
+
+namespace harness {
+
+static std::vector<Entry>& registry()
+{
+  static std::vector<Entry> r;
+  return r;
+}
+static bool g_sorted = false;
+
+void register_case(const cudadma_case_t& desc, launch_fn fn, int order)
+{
+  registry().push_back(Entry{desc, fn, order});
+  g_sorted = false;
+}
+
+// Static initialisers of different translation units run in no fixed order:
+// give the cases a stable numbering (pattern, then order of appearance in its list).
+static const std::vector<Entry>& sorted()
+{
+  std::vector<Entry>& r = registry();
+  if (!g_sorted) {
+    std::stable_sort(r.begin(), r.end(), [](const Entry& x, const Entry& y) {
+      if (x.desc.pattern != y.desc.pattern) return x.desc.pattern < y.desc.pattern;
+      return x.order < y.order;
+    });
+    g_sorted = true;
+  }
+  return r;
+}
+
+}  // namespace harness
+
+extern "C" int cudadma_num_cases(void) { return (int)harness::sorted().size(); }
+
+extern "C" int cudadma_get_case(int case_id, cudadma_case_t* out)
+{
+  const auto& r = harness::sorted();
+  if (case_id < 0 || case_id >= (int)r.size() || out == nullptr) {
+    cudadma_host::set_error("case %d out of range [0,%d)", case_id, (int)r.size());
+    return CUDADMA_ERANGE;
+  }
+  *out = r[case_id].desc;
+  return CUDADMA_OK;
+}
+
+extern "C" int cudadma_run_case(int case_id, const cudadma_run_t* run, void* stream)
+{
+  const auto& r = harness::sorted();
+  if (case_id < 0 || case_id >= (int)r.size()) {
+    cudadma_host::set_error("case %d out of range [0,%d)", case_id, (int)r.size());
+    return CUDADMA_ERANGE;
+  }
+  CUDADMA_REQUIRE(run != nullptr, "run is NULL");
+  const cudadma_case_t& d = r[case_id].desc;
+  CUDADMA_REQUIRE(run->d_in != nullptr && run->d_out != nullptr, "d_in / d_out must not be NULL");
+  CUDADMA_REQUIRE(run->lds_bytes > 0 && run->lds_bytes <= 64 * 1024 - 256 && (run->lds_bytes % 16) == 0,
+                  "lds_bytes %d must be a positive multiple of 16 below 64 KiB", run->lds_bytes);
+  CUDADMA_REQUIRE(run->reps >= 1, "reps must be >= 1");
+  CUDADMA_REQUIRE(run->call_style >= CUDADMA_CALL_UNQUALIFIED && run->call_style <= CUDADMA_CALL_LDS_DIRECT,
+                  "unknown call_style %d", run->call_style);
+  if (d.pattern == CUDADMA_PATTERN_HALO) {
+    // the origins, not the buffer starts, carry the alignment
+    const int src_origin = run->src_offset_bytes + (d.radius * run->pitch + d.radius) * d.bytes_per_elmt;
+    const int dst_origin = run->dst_offset_bytes + (d.radius * (d.dimx + 2 * d.radius) + d.radius) * d.bytes_per_elmt;
+    CUDADMA_REQUIRE((src_origin % d.alignment) == 0 && (dst_origin % d.alignment) == 0 &&
+                    ((run->pitch * d.bytes_per_elmt) % d.alignment) == 0 && (run->rep_src_bytes % d.alignment) == 0,
+                    "halo origins and pitch must keep the ALIGNMENT (%d) the case was compiled for", d.alignment);
+    CUDADMA_REQUIRE(run->pitch >= d.dimx + 2 * d.radius, "pitch %d is narrower than the padded tile", run->pitch);
+  } else {
+    CUDADMA_REQUIRE((run->src_offset_bytes % d.alignment) == 0 && (run->dst_offset_bytes % d.alignment) == 0 &&
+                    (run->rep_src_bytes % d.alignment) == 0,
+                    "offsets must keep the ALIGNMENT (%d) the case was compiled for", d.alignment);
+  }
+  CUDADMA_REQUIRE(cudadma_host::aligned_to(run->d_in, 16) && cudadma_host::aligned_to(run->d_out, 16),
+                  "d_in and d_out must be 16-byte aligned");
+  if (d.pattern == CUDADMA_PATTERN_GATHER || d.pattern == CUDADMA_PATTERN_SCATTER)
+    CUDADMA_REQUIRE(run->d_index != nullptr, "gather / scatter need d_index");
+  if (d.pattern == CUDADMA_PATTERN_STRIDED)
+    CUDADMA_REQUIRE((run->src_stride % d.alignment) == 0 && (run->dst_stride % d.alignment) == 0,
+                    "strides must be multiples of ALIGNMENT");
+  if (d.pattern == CUDADMA_PATTERN_HALO)
+    CUDADMA_REQUIRE(run->call_style != CUDADMA_CALL_LDS_DIRECT, "the halo object has no direct path");
+  if (d.pattern == CUDADMA_PATTERN_SCATTER)
+    CUDADMA_REQUIRE(run->call_style != CUDADMA_CALL_LDS_DIRECT, "scatter has no direct path");
+  if (run->call_style == CUDADMA_CALL_LDS_DIRECT)
+    CUDADMA_REQUIRE(d.alignment == 16 || d.alignment == 4, "the direct path moves 4 or 16 bytes per lane");
+
+  harness::Args a;
+  a.in = (const char*)run->d_in;
+  a.out = (char*)run->d_out;
+  a.index = run->d_index;
+  a.lds_bytes = run->lds_bytes;
+  a.src_offset = run->src_offset_bytes;
+  a.dst_offset = run->dst_offset_bytes;
+  a.src_stride = run->src_stride;
+  a.dst_stride = run->dst_stride;
+  a.pitch = run->pitch;
+  a.call_style = run->call_style;
+  a.two_phase = run->two_phase;
+  a.reps = run->reps;
+  a.rep_src_bytes = run->rep_src_bytes;
+  a.rep_index_elmts = run->rep_index_elmts;
+  a.bytes_per_elmt = d.bytes_per_elmt;
+  a.dma_threads = d.dma_threads;
+  a.num_elmts = d.num_elmts;
+  a.dimx = d.dimx;
+  a.dimy = d.dimy;
+  return r[case_id].launch(a, (hipStream_t)stream);
+}

@@ -1,0 +1,141 @@
+// Known-answer harness: registry of compiled DMA-object cases and the kernel
+// skeleton they share.  One workgroup; warp-specialised cases run 64 compute
+// threads [0,64) and DMA_THREADS DMA threads [64, 64+DMA_THREADS); the compute
+// wavefront clears the LDS buffer, releases it, waits for the transfer and
+// copies the whole buffer out (the shape of special_xfer_* in
+// src/tests/test_sequential/cudaDMA_test_sequential_v2.cu:52-115).  The other
+// cases run DMA_THREADS threads that all transfer, between two workgroup
+// barriers (nonspec_xfer_*, same file).
+#pragma once
+
+#include "common.hpp"
+#include "../../include/hipDMA.h"
+
+namespace harness {
+
+constexpr int kComputeThreads = 64;
+
+struct Args {
+  const char* in;
+  char* out;
+  const int* index;
+  int lds_bytes;
+  int src_offset, dst_offset;
+  int src_stride, dst_stride;
+  int pitch;
+  int call_style, two_phase;
+  int reps, rep_src_bytes, rep_index_elmts;
+  // run-time copies of the template parameters, fed to the constructors of the lower levels
+  int bytes_per_elmt, dma_threads, num_elmts, dimx, dimy;
+};
+
+typedef int (*launch_fn)(const Args&, hipStream_t);
+
+struct Entry {
+  cudadma_case_t desc;
+  launch_fn launch;
+  int order;
+};
+
+void register_case(const cudadma_case_t& desc, launch_fn fn, int order);
+
+struct Registrar {
+  Registrar(const cudadma_case_t& desc, launch_fn fn, int order) { register_case(desc, fn, order); }
+};
+
+// Transfer through the call style picked at run time.  XFER is a functor
+// template<bool GL,int LQ,int SQ> with static run(obj, two_phase, ...).
+template<typename Obj, typename... P>
+__device__ __forceinline__ void do_transfer(Obj& dma, const int call_style, const int two_phase,
+                                            const void* src, void* dst)
+{
+  if (call_style == CUDADMA_CALL_UNQUALIFIED) {
+    if (two_phase) { dma.start_xfer_async(src); dma.wait_xfer_finish(dst); }
+    else dma.execute_dma(src, dst);
+  } else if (call_style == CUDADMA_CALL_GLOBAL) {
+    if (two_phase) { dma.template start_xfer_async<true>(src); dma.template wait_xfer_finish<true>(dst); }
+    else dma.template execute_dma<true>(src, dst);
+  } else if (call_style == CUDADMA_CALL_QUALIFIED) {
+    if (two_phase) {
+      dma.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src);
+      dma.template wait_xfer_finish<true, LOAD_CACHE_STREAMING, STORE_LDS>(dst);
+    } else dma.template execute_dma<true, LOAD_CACHE_STREAMING, STORE_LDS>(src, dst);
+  }
+}
+
+template<typename Obj>
+__device__ __forceinline__ void do_transfer_direct(Obj& dma, const int two_phase, const void* src, void* dst)
+{
+  if (two_phase) {
+    dma.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS_DIRECT>(src);
+    dma.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS_DIRECT>(dst);
+  } else dma.template execute_dma<true, LOAD_CACHE_ALL, STORE_LDS_DIRECT>(src, dst);
+}
+
+template<typename Obj>
+__device__ __forceinline__ void do_transfer_indexed(Obj& dma, const int call_style, const int two_phase,
+                                                    const int* index, const void* src, void* dst)
+{
+  if (call_style == CUDADMA_CALL_UNQUALIFIED) {
+    if (two_phase) { dma.start_xfer_async(index, src); dma.wait_xfer_finish(dst); }
+    else dma.execute_dma(index, src, dst);
+  } else if (call_style == CUDADMA_CALL_GLOBAL) {
+    if (two_phase) { dma.template start_xfer_async<true>(index, src); dma.template wait_xfer_finish<true>(dst); }
+    else dma.template execute_dma<true>(index, src, dst);
+  } else if (call_style == CUDADMA_CALL_QUALIFIED) {
+    if (two_phase) {
+      dma.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_WRITE_BACK>(index, src);
+      dma.template wait_xfer_finish<true, LOAD_CACHE_STREAMING, STORE_WRITE_BACK>(dst);
+    } else dma.template execute_dma<true, LOAD_CACHE_STREAMING, STORE_WRITE_BACK>(index, src, dst);
+  }
+}
+
+// The LDS buffer handling both kernel shapes share.
+__device__ __forceinline__ void clear_lds(unsigned* buf, const int words, const int tid, const int nthreads)
+{
+  for (int i = tid; i < words; i += nthreads) buf[i] = 0u;
+}
+__device__ __forceinline__ void copy_out(const unsigned* buf, unsigned* out, const int words, const int tid,
+                                         const int nthreads)
+{
+  for (int i = tid; i < words; i += nthreads) out[i] = buf[i];
+}
+
+// Body shared by every case.  `xfer(rep)` performs one transfer (DMA threads).
+template<bool WS, typename Obj, typename Xfer>
+__device__ __forceinline__ void run_body(Obj& dma, const Args& a, unsigned* lds, Xfer xfer)
+{
+  const int words = a.lds_bytes / 4;
+  if constexpr (WS) {
+    if (dma.owns_this_thread()) {
+      for (int rep = 0; rep < a.reps; ++rep) xfer(rep);
+    } else if (threadIdx.x < kComputeThreads) {
+      for (int rep = 0; rep < a.reps; ++rep) {
+        clear_lds(lds, words, threadIdx.x, kComputeThreads);
+        dma.start_async_dma();
+        dma.wait_for_dma_finish();
+        copy_out(lds, (unsigned*)(a.out + (size_t)rep * a.lds_bytes), words, threadIdx.x, kComputeThreads);
+      }
+    }
+  } else {
+    for (int rep = 0; rep < a.reps; ++rep) {
+      clear_lds(lds, words, threadIdx.x, blockDim.x);
+      __syncthreads();
+      xfer(rep);
+      __syncthreads();
+      copy_out(lds, (unsigned*)(a.out + (size_t)rep * a.lds_bytes), words, threadIdx.x, blockDim.x);
+      __syncthreads();
+    }
+  }
+}
+
+template<typename Kernel>
+int launch_case(Kernel kernel, const bool ws, const Args& a, hipStream_t stream)
+{
+  const int threads = ws ? (kComputeThreads + a.dma_threads) : a.dma_threads;
+  hipLaunchKernelGGL(kernel, dim3(1), dim3(threads), (size_t)a.lds_bytes, stream, a);
+  CUDADMA_HIP_CHECK(hipGetLastError());
+  return CUDADMA_OK;
+}
+
+}  // namespace harness

@@ -1,0 +1,111 @@
+// Known-answer cases for CudaDMAStrided
+// (counterpart of src/tests/test_strided/cudaDMA_test_strided_v2.cu).
+#include "harness.hpp"
+
+namespace {
+using harness::Args;
+using harness::kComputeThreads;
+
+// ONE_STRIDE picks the constructor that takes one elmt_stride for both sides
+// (the host then has to pass src_stride == dst_stride); otherwise the
+// constructor with separate source and destination strides is used.
+template<bool WS, int LEVEL, bool ONE_STRIDE, int A, int BPT, int E, int T, int N> struct Make;
+template<bool ONE, int A, int BPT, int E, int T, int N> struct Make<true, 1, ONE, A, BPT, E, T, N> {
+  typedef CudaDMAStrided<true, A, BPT> type;
+  static __device__ __forceinline__ type make(const Args& a)
+  {
+    if constexpr (ONE) return type(1, a.dma_threads, kComputeThreads, kComputeThreads, a.bytes_per_elmt, a.num_elmts, a.src_stride);
+    else return type(1, a.dma_threads, kComputeThreads, kComputeThreads, a.bytes_per_elmt, a.num_elmts, a.src_stride, a.dst_stride);
+  }
+};
+template<bool ONE, int A, int BPT, int E, int T, int N> struct Make<true, 2, ONE, A, BPT, E, T, N> {
+  typedef CudaDMAStrided<true, A, BPT, E> type;
+  static __device__ __forceinline__ type make(const Args& a)
+  {
+    if constexpr (ONE) return type(2, a.dma_threads, kComputeThreads, kComputeThreads, a.num_elmts, a.src_stride);
+    else return type(2, a.dma_threads, kComputeThreads, kComputeThreads, a.num_elmts, a.src_stride, a.dst_stride);
+  }
+};
+template<bool ONE, int A, int BPT, int E, int T, int N> struct Make<true, 3, ONE, A, BPT, E, T, N> {
+  typedef CudaDMAStrided<true, A, BPT, E, T> type;
+  static __device__ __forceinline__ type make(const Args& a)
+  {
+    if constexpr (ONE) return type(3, kComputeThreads, kComputeThreads, a.num_elmts, a.src_stride);
+    else return type(3, kComputeThreads, kComputeThreads, a.num_elmts, a.src_stride, a.dst_stride);
+  }
+};
+template<bool ONE, int A, int BPT, int E, int T, int N> struct Make<true, 4, ONE, A, BPT, E, T, N> {
+  typedef CudaDMAStrided<true, A, BPT, E, T, N> type;
+  static __device__ __forceinline__ type make(const Args& a)
+  {
+    if constexpr (ONE) return type(4, kComputeThreads, kComputeThreads, a.src_stride);
+    else return type(4, kComputeThreads, kComputeThreads, a.src_stride, a.dst_stride);
+  }
+};
+template<bool ONE, int A, int BPT, int E, int T, int N> struct Make<false, 1, ONE, A, BPT, E, T, N> {
+  typedef CudaDMAStrided<false, A, BPT> type;
+  static __device__ __forceinline__ type make(const Args& a)
+  {
+    if constexpr (ONE) return type(a.bytes_per_elmt, a.num_elmts, a.src_stride);
+    else return type(a.bytes_per_elmt, a.num_elmts, a.src_stride, a.dst_stride, a.dma_threads);
+  }
+};
+template<bool ONE, int A, int BPT, int E, int T, int N> struct Make<false, 2, ONE, A, BPT, E, T, N> {
+  typedef CudaDMAStrided<false, A, BPT, E> type;
+  static __device__ __forceinline__ type make(const Args& a)
+  {
+    if constexpr (ONE) return type(a.num_elmts, a.src_stride);
+    else return type(a.num_elmts, a.src_stride, a.dst_stride);
+  }
+};
+template<bool ONE, int A, int BPT, int E, int T, int N> struct Make<false, 3, ONE, A, BPT, E, T, N> {
+  typedef CudaDMAStrided<false, A, BPT, E, T> type;
+  static __device__ __forceinline__ type make(const Args& a)
+  {
+    if constexpr (ONE) return type(a.num_elmts, a.src_stride);
+    else return type(a.num_elmts, a.src_stride, a.dst_stride);
+  }
+};
+template<bool ONE, int A, int BPT, int E, int T, int N> struct Make<false, 4, ONE, A, BPT, E, T, N> {
+  typedef CudaDMAStrided<false, A, BPT, E, T, N> type;
+  static __device__ __forceinline__ type make(const Args& a)
+  {
+    if constexpr (ONE) return type(a.src_stride);
+    else return type(a.src_stride, a.dst_stride);
+  }
+};
+
+template<bool WS, int LEVEL, bool ONE, int A, int BPT, int E, int T, int N>
+__global__ void __launch_bounds__(1024) strided_kernel(const Args a)
+{
+  extern __shared__ __attribute__((aligned(16))) unsigned lds[];
+  auto dma = Make<WS, LEVEL, ONE, A, BPT, E, T, N>::make(a);
+  harness::run_body<WS>(dma, a, lds, [&](const int rep) {
+    const char* src = a.in + a.src_offset + (size_t)rep * a.rep_src_bytes;
+    char* dst = (char*)lds + a.dst_offset;
+    if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
+      if constexpr (A == 16 || A == 4) harness::do_transfer_direct(dma, a.two_phase, src, dst);
+    } else {
+      harness::do_transfer(dma, a.call_style, a.two_phase, src, dst);
+    }
+  });
+}
+
+template<bool WS, int LEVEL, bool ONE, int A, int BPT, int E, int T, int N>
+int launch(const Args& a, hipStream_t s)
+{
+  if (ONE && a.src_stride != a.dst_stride) {
+    cudadma_host::set_error("this case was built with the single-stride constructor: src_stride must equal dst_stride");
+    return CUDADMA_EINVAL;
+  }
+  return harness::launch_case(strided_kernel<WS, LEVEL, ONE, A, BPT, E, T, N>, WS, a, s);
+}
+
+// dimx carries the ONE_STRIDE flag in the case description.
+#define STRIDED_CASE(ORDER, WS, LEVEL, ONE, A, BPT, E, T, N)                                             \
+  static harness::Registrar reg_strided_##ORDER(                                                          \
+      cudadma_case_t{CUDADMA_PATTERN_STRIDED, WS, LEVEL, A, BPT, E, T, N, 0, 0, ONE, 0},                  \
+      launch<WS, LEVEL, ONE, A, BPT, E, T, N>, ORDER);
+#include "cases_strided.inc"
+#undef STRIDED_CASE
+}  // namespace

@@ -1,0 +1,73 @@
+// Variant tables, the occupancy knob and grid sizing shared by the workloads.
+#include "workloads.hpp"
+#include <atomic>
+
+namespace workloads {
+
+static std::atomic<int> g_wg_per_cu{0};
+static int g_cus = 0;
+
+int persistent_grid(long long work_items, int default_wg_per_cu)
+{
+  if (g_cus <= 0) {
+    g_cus = cudadma_device_cus();
+    if (g_cus <= 0) g_cus = 256;
+  }
+  const int knob = g_wg_per_cu.load();
+  const long long want = (long long)g_cus * (knob > 0 ? knob : default_wg_per_cu);
+  return (int)(work_items < want ? work_items : want);
+}
+
+static const VariantInfo kSequential[] = {
+  {"manual double buffer: one DMA group of 2 wavefronts, two objects, two-phase calls, registers -> ds_write_b128"},
+  {"single buffer: one object, execute_dma"},
+  {"double buffer: two DMA groups of 1 wavefront, one object each"},
+  {"manual double buffer with STORE_LDS_DIRECT (global_load_lds_dwordx4, no VGPR staging)"},
+  {"no DMA object: every wavefront copies global -> LDS -> global between workgroup barriers"},
+};
+static const VariantInfo kStrided[] = {
+  {"manual double buffer: one DMA group of 2 wavefronts, two CudaDMAStrided objects, padded LDS rows (272 B)"},
+  {"single buffer: one object, execute_dma"},
+  {"manual double buffer, unpadded LDS rows (256 B): shows the bank-conflict cost"},
+};
+static const VariantInfo kGather[] = {
+  {"manual 4-stage buffering: one DMA group of 2 wavefronts, four CudaDMAIndirect objects"},
+  {"single buffer: one object, execute_dma"},
+  {"manual double buffer: two objects"},
+};
+static const VariantInfo kHalo[] = {
+  {"warp-specialised: CudaDMAHalo ring by 1 DMA wavefront, interior by the 4 compute wavefronts, double-buffered planes"},
+  {"not warp-specialised: all wavefronts move the ring, workgroup barriers"},
+};
+
+static const VariantInfo* table(int workload, int* count)
+{
+  switch (workload) {
+    case CUDADMA_WORKLOAD_SEQUENTIAL: *count = sizeof(kSequential) / sizeof(VariantInfo); return kSequential;
+    case CUDADMA_WORKLOAD_STRIDED:    *count = sizeof(kStrided) / sizeof(VariantInfo);    return kStrided;
+    case CUDADMA_WORKLOAD_GATHER:     *count = sizeof(kGather) / sizeof(VariantInfo);     return kGather;
+    case CUDADMA_WORKLOAD_HALO:       *count = sizeof(kHalo) / sizeof(VariantInfo);       return kHalo;
+    default: *count = 0; return nullptr;
+  }
+}
+
+}  // namespace workloads
+
+extern "C" int cudadma_num_variants(int workload)
+{
+  int n = 0;
+  workloads::table(workload, &n);
+  return n;
+}
+
+extern "C" const char* cudadma_variant_name(int workload, int variant)
+{
+  int n = 0;
+  const workloads::VariantInfo* t = workloads::table(workload, &n);
+  return (t != nullptr && variant >= 0 && variant < n) ? t[variant].name : "";
+}
+
+extern "C" int cudadma_set_workgroups_per_cu(int value)
+{
+  return workloads::g_wg_per_cu.exchange(value < 0 ? 0 : value);
+}

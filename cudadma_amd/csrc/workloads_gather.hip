@@ -1,0 +1,156 @@
+// Config 3: indirect gather of 128-byte records with CudaDMAIndirect, 32 records
+// per LDS tile.  Shapes follow the warp-specialised kernels of
+// src/tests/test_indirect/cudaDMA_test_indirect_v2.cu:52-120, made persistent
+// and multi-buffered as src/examples/stencil/warp_specialized_manual_buffer.h:54-71.
+// Two consumers:
+//   copy   out[i] = table[idx[i]]                       (checks every moved byte)
+//   rowsum out[t][j] = sum_r tile[r][j], r ascending     (the reported workload)
+#include "workloads.hpp"
+
+namespace {
+using workloads::vec4_t;
+
+constexpr int kRecBytes = 128;
+constexpr int kRecFloats = kRecBytes / 4;
+constexpr int kRecsPerTile = 32;
+constexpr int kTileBytes = kRecBytes * kRecsPerTile;     // 4 KiB
+constexpr int kDmaThreads = 128;
+constexpr int kComputeThreads = 128;
+constexpr int kBytesPerThread = kTileBytes / kDmaThreads;   // 32: two dwordx4 per DMA thread, one step
+
+typedef CudaDMAIndirect<true, true, 16, kBytesPerThread, kRecBytes, kDmaThreads, kRecsPerTile> dma_t;
+
+struct CopyConsumer {
+  static __device__ __forceinline__ void run(const char* lds_tile, float* __restrict__ out, const long long tile,
+                                             const dma_t& dma)
+  {
+    vec4_t v[2];
+    const vec4_t* src = (const vec4_t*)lds_tile;
+    v[0] = src[threadIdx.x];
+    v[1] = src[threadIdx.x + kComputeThreads];
+    dma.start_async_dma();
+    vec4_t* dst = (vec4_t*)(out + tile * (kTileBytes / 4));
+    dst[threadIdx.x] = v[0];
+    dst[threadIdx.x + kComputeThreads] = v[1];
+  }
+};
+
+struct RowsumConsumer {
+  static __device__ __forceinline__ void run(const char* lds_tile, float* __restrict__ out, const long long tile,
+                                             const dma_t& dma)
+  {
+    // 32 sums per tile: the first 32 compute threads each add one word of every record, record 0 first
+    const float* t = (const float*)lds_tile;
+    float acc = 0.0f;
+    if (threadIdx.x < kRecFloats) {
+      acc = t[threadIdx.x];
+#pragma unroll
+      for (int r = 1; r < kRecsPerTile; ++r) acc = acc + t[r * kRecFloats + threadIdx.x];
+    }
+    dma.start_async_dma();
+    if (threadIdx.x < kRecFloats) out[tile * kRecFloats + threadIdx.x] = acc;
+  }
+};
+
+// STAGES objects share the DMA threads; each has its own 4 KiB buffer.
+template<typename Consumer, int STAGES>
+__global__ void __launch_bounds__(kDmaThreads + kComputeThreads)
+gather_manual(const float* __restrict__ table, const int* __restrict__ idx, float* __restrict__ out,
+              const long long num_tiles)
+{
+  __shared__ __attribute__((aligned(16))) char buf[STAGES][kTileBytes];
+  dma_t dma0(0, kComputeThreads, kComputeThreads);
+  dma_t dma1(1, kComputeThreads, kComputeThreads);
+  dma_t dma2(2, kComputeThreads, kComputeThreads);
+  dma_t dma3(3, kComputeThreads, kComputeThreads);
+  const long long stride = gridDim.x;
+  const long long first = blockIdx.x;
+#define HIPDMA_FOR_STAGES(...)                                                    \
+  { constexpr int s = 0; dma_t& d = dma0; __VA_ARGS__ }                           \
+  if constexpr (STAGES > 1) { constexpr int s = 1; dma_t& d = dma1; __VA_ARGS__ } \
+  if constexpr (STAGES > 2) { constexpr int s = 2; dma_t& d = dma2; __VA_ARGS__ } \
+  if constexpr (STAGES > 3) { constexpr int s = 3; dma_t& d = dma3; __VA_ARGS__ }
+  if (dma0.owns_this_thread()) {
+    HIPDMA_FOR_STAGES({
+      const long long tt = first + s * stride;
+      if (tt < num_tiles) d.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(idx + tt * kRecsPerTile, table);
+    })
+    for (long long t = first; t < num_tiles; t += STAGES * stride) {
+      HIPDMA_FOR_STAGES({
+        const long long tt = t + s * stride;
+        if (tt < num_tiles) {
+          d.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf[s]);
+          const long long nx = tt + STAGES * stride;
+          if (nx < num_tiles) d.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(idx + nx * kRecsPerTile, table);
+        }
+      })
+    }
+  } else {
+    HIPDMA_FOR_STAGES({ d.start_async_dma(); })
+    for (long long t = first; t < num_tiles; t += STAGES * stride) {
+      HIPDMA_FOR_STAGES({
+        const long long tt = t + s * stride;
+        if (tt < num_tiles) {
+          d.wait_for_dma_finish();
+          Consumer::run(buf[s], out, tt, d);
+        }
+      })
+    }
+  }
+#undef HIPDMA_FOR_STAGES
+}
+
+template<typename Consumer>
+__global__ void __launch_bounds__(kDmaThreads + kComputeThreads)
+gather_single(const float* __restrict__ table, const int* __restrict__ idx, float* __restrict__ out,
+              const long long num_tiles)
+{
+  __shared__ __attribute__((aligned(16))) char buf[kTileBytes];
+  dma_t dma(0, kComputeThreads, kComputeThreads);
+  if (dma.owns_this_thread()) {
+    for (long long t = blockIdx.x; t < num_tiles; t += gridDim.x)
+      dma.template execute_dma<true, LOAD_CACHE_ALL, STORE_LDS>(idx + t * kRecsPerTile, table, buf);
+  } else {
+    dma.start_async_dma();
+    for (long long t = blockIdx.x; t < num_tiles; t += gridDim.x) {
+      dma.wait_for_dma_finish();
+      Consumer::run(buf, out, t, dma);
+    }
+  }
+}
+
+template<typename Consumer>
+int launch_gather(const float* d_table, const int32_t* d_idx, float* d_out, size_t n_records, size_t n_idx,
+                  int variant, void* stream)
+{
+  CUDADMA_REQUIRE((n_idx % kRecsPerTile) == 0, "n_idx (%zu) must be a multiple of %d", n_idx, kRecsPerTile);
+  CUDADMA_REQUIRE(n_records > 0 && n_records * (size_t)kRecBytes <= 0x7fffffffull,
+                  "the table (%zu records) must stay below 2 GiB: the objects address it with int offsets", n_records);
+  if (variant < 0 || variant >= cudadma_num_variants(CUDADMA_WORKLOAD_GATHER)) {
+    cudadma_host::set_error("gather has no variant %d", variant);
+    return CUDADMA_ERANGE;
+  }
+  if (n_idx == 0) return CUDADMA_OK;
+  CUDADMA_REQUIRE(d_table != nullptr && d_idx != nullptr && d_out != nullptr, "NULL pointer");
+  CUDADMA_REQUIRE(cudadma_host::aligned_to(d_table, 16) && cudadma_host::aligned_to(d_out, 16), "pointers must be 16-byte aligned");
+  const long long tiles = (long long)(n_idx / kRecsPerTile);
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 block(kDmaThreads + kComputeThreads);
+  switch (variant) {
+    case 0: hipLaunchKernelGGL((gather_manual<Consumer, 4>), dim3(workloads::persistent_grid(tiles, 8)), block, 0, s, d_table, d_idx, d_out, tiles); break;
+    case 1: hipLaunchKernelGGL(gather_single<Consumer>, dim3(workloads::persistent_grid(tiles, 8)), block, 0, s, d_table, d_idx, d_out, tiles); break;
+    default: hipLaunchKernelGGL((gather_manual<Consumer, 2>), dim3(workloads::persistent_grid(tiles, 8)), block, 0, s, d_table, d_idx, d_out, tiles); break;
+  }
+  CUDADMA_HIP_CHECK(hipGetLastError());
+  return CUDADMA_OK;
+}
+
+}  // namespace
+
+extern "C" int cudadma_gather_copy(const float* d_table, const int32_t* d_idx, float* d_out, size_t n_records,
+                                   size_t n_idx, int variant, void* stream)
+{ return launch_gather<CopyConsumer>(d_table, d_idx, d_out, n_records, n_idx, variant, stream); }
+
+extern "C" int cudadma_gather_rowsum(const float* d_table, const int32_t* d_idx, float* d_out, size_t n_records,
+                                     size_t n_idx, int variant, void* stream)
+{ return launch_gather<RowsumConsumer>(d_table, d_idx, d_out, n_records, n_idx, variant, stream); }

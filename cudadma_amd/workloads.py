@@ -1,0 +1,110 @@
+"""Python face of the benchmark workloads.  Every function takes torch CUDA
+tensors, launches on torch's current stream and returns the output tensor; all
+compute happens in libcudadma_amd.so."""
+import ctypes
+
+import torch
+
+from ._lib import check, lib
+
+SEQUENTIAL, STRIDED, GATHER, HALO, GEMM = range(5)
+
+REC_FLOATS = 32          # 128-byte records
+RECS_PER_TILE = 32
+SEQ_TILE_BYTES = 16 * 1024
+STENCIL_RADIUS = 4
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _need(t, dtype, what):
+    if not (t.is_cuda and t.is_contiguous() and t.dtype == dtype):
+        raise ValueError(f"{what} must be a contiguous CUDA tensor of {dtype}")
+
+
+def num_variants(workload):
+    return lib().cudadma_num_variants(workload)
+
+
+def variant_name(workload, variant):
+    return lib().cudadma_variant_name(workload, variant).decode()
+
+
+def set_workgroups_per_cu(value):
+    return lib().cudadma_set_workgroups_per_cu(int(value))
+
+
+def fill_uniform(out, seed):
+    _need(out, torch.float32, "out")
+    check(lib().cudadma_fill_uniform(_p(out), out.numel(), seed, _stream()))
+    return out
+
+
+def fill_indices(out, n_records, seed):
+    _need(out, torch.int32, "out")
+    check(lib().cudadma_fill_indices(_p(out), out.numel(), n_records, seed, _stream()))
+    return out
+
+
+def plain_copy(src, dst):
+    check(lib().cudadma_plain_copy(_p(src), _p(dst), src.numel() * src.element_size(), _stream()))
+    return dst
+
+
+def sequential_copy(src, dst, variant=0):
+    _need(src, torch.float32, "src")
+    _need(dst, torch.float32, "dst")
+    if dst.numel() != src.numel():
+        raise ValueError("src and dst differ in size")
+    check(lib().cudadma_sequential_copy(_p(src), _p(dst), src.numel() * 4, variant, _stream()))
+    return dst
+
+
+def strided_transpose(src, dst, variant=0):
+    _need(src, torch.float32, "src")
+    _need(dst, torch.float32, "dst")
+    n = src.shape[0]
+    if src.dim() != 2 or src.shape[1] != n or tuple(dst.shape) != (n, n):
+        raise ValueError("src and dst must be n x n")
+    check(lib().cudadma_strided_transpose(_p(src), _p(dst), n, variant, _stream()))
+    return dst
+
+
+def gather_copy(table, idx, out, variant=0):
+    _need(table, torch.float32, "table")
+    _need(idx, torch.int32, "idx")
+    _need(out, torch.float32, "out")
+    if out.numel() != idx.numel() * REC_FLOATS:
+        raise ValueError("out must hold one record per index")
+    check(lib().cudadma_gather_copy(_p(table), _p(idx), _p(out), table.numel() // REC_FLOATS, idx.numel(),
+                                    variant, _stream()))
+    return out
+
+
+def gather_rowsum(table, idx, out, variant=0):
+    _need(table, torch.float32, "table")
+    _need(idx, torch.int32, "idx")
+    _need(out, torch.float32, "out")
+    if out.numel() != idx.numel() // RECS_PER_TILE * REC_FLOATS:
+        raise ValueError("out must hold one record per tile of 32 indices")
+    check(lib().cudadma_gather_rowsum(_p(table), _p(idx), _p(out), table.numel() // REC_FLOATS, idx.numel(),
+                                      variant, _stream()))
+    return out
+
+
+def halo_stencil(grid_in, grid_out, variant=0):
+    """grid_in: (nz+8, ny+8, nx+8) padded input, grid_out: (nz, ny, nx)."""
+    _need(grid_in, torch.float32, "grid_in")
+    _need(grid_out, torch.float32, "grid_out")
+    nz, ny, nx = grid_out.shape
+    p = 2 * STENCIL_RADIUS
+    if tuple(grid_in.shape) != (nz + p, ny + p, nx + p):
+        raise ValueError("grid_in must be the output shape plus 8 in every dimension")
+    check(lib().cudadma_halo_stencil(_p(grid_in), _p(grid_out), nx, ny, nz, variant, _stream()))
+    return grid_out

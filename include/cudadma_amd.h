@@ -1,0 +1,172 @@
+/* C ABI of libcudadma_amd.so: the host drivers around the hipDMA device header.
+ *
+ * The reference is a header; what its repository binds it to are the host
+ * programs of src/tests, src/perf and src/examples.  Each entry point below
+ * stands for one of those programs' run functions, takes plain device pointers
+ * and sizes, launches on the given HIP stream (NULL = default stream) and
+ * returns 0 or a negative CUDADMA_E* code; cudadma_last_error() gives the text.
+ * Nothing here allocates device memory.
+ */
+#ifndef CUDADMA_AMD_H
+#define CUDADMA_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CUDADMA_OK            0
+#define CUDADMA_EINVAL       -1   /* bad argument (size, alignment, variant, null pointer) */
+#define CUDADMA_ELAUNCH      -2   /* HIP reported a launch or runtime error */
+#define CUDADMA_ERANGE       -3   /* case index or variant out of range */
+
+const char* cudadma_last_error(void);
+/* Number of compute units of the current device (used to size persistent grids). */
+int cudadma_device_cus(void);
+
+/* ------------------------------------------------------------------------
+ * Known-answer harness: one workgroup moves data global -> LDS with one DMA
+ * object and copies the whole LDS buffer back out, as the kernels
+ * special_xfer_* / nonspec_xfer_* of
+ * src/tests/test_sequential/cudaDMA_test_sequential_v2.cu:52-395,
+ * src/tests/test_strided/cudaDMA_test_strided_v2.cu:52-536,
+ * src/tests/test_indirect/cudaDMA_test_indirect_v2.cu:52-548 and dma_ld_test of
+ * src/tests/test_halo/cudaDMA_test_halo.cu:180-231 do.  Every compiled
+ * combination of template parameters is one case.
+ * ---------------------------------------------------------------------- */
+enum {
+  CUDADMA_PATTERN_SEQUENTIAL = 0,
+  CUDADMA_PATTERN_STRIDED    = 1,
+  CUDADMA_PATTERN_GATHER     = 2,
+  CUDADMA_PATTERN_SCATTER    = 3,
+  CUDADMA_PATTERN_HALO       = 4
+};
+
+/* Transfer call styles (cudaDMA_test_strided_v2.cu:693-812 runs the same set). */
+enum {
+  CUDADMA_CALL_UNQUALIFIED  = 0,  /* execute_dma(src,dst)                                  */
+  CUDADMA_CALL_GLOBAL       = 1,  /* execute_dma<true>(src,dst)                            */
+  CUDADMA_CALL_QUALIFIED    = 2,  /* execute_dma<true,LOAD_CACHE_STREAMING,STORE_LDS>      */
+  CUDADMA_CALL_LDS_DIRECT   = 3   /* execute_dma<true,LOAD_CACHE_ALL,STORE_LDS_DIRECT>     */
+};
+
+typedef struct cudadma_case {
+  int pattern;            /* CUDADMA_PATTERN_*                                        */
+  int warp_specialized;   /* DO_SYNC                                                  */
+  int level;              /* how many trailing template parameters are compile-time   */
+  int alignment;          /* ALIGNMENT                                                */
+  int bytes_per_thread;   /* BYTES_PER_THREAD                                         */
+  int bytes_per_elmt;     /* BYTES_PER_ELMT (halo: bytes of one cell)                 */
+  int dma_threads;        /* DMA_THREADS                                              */
+  int num_elmts;          /* NUM_ELMTS (strided / indirect)                           */
+  int radius;             /* halo only                                                */
+  int corners;            /* halo only                                                */
+  int dimx, dimy;         /* halo only: tile size in cells                            */
+} cudadma_case_t;
+
+typedef struct cudadma_run {
+  const void* d_in;       /* device input                                             */
+  void* d_out;            /* device output: reps * lds_bytes                          */
+  const int* d_index;     /* device element indices (gather / scatter), else NULL     */
+  int lds_bytes;          /* size of the LDS buffer, copied out whole after each rep  */
+  int src_offset_bytes;   /* added to d_in before the transfer (ALIGN_OFFSET)         */
+  int dst_offset_bytes;   /* added to the LDS buffer before the transfer              */
+  int src_stride;         /* strided: source stride; scatter: dense-side stride       */
+  int dst_stride;         /* strided: destination stride; gather: dense-side stride   */
+  int pitch;              /* halo: source row pitch in cells                          */
+  int call_style;         /* CUDADMA_CALL_*                                           */
+  int two_phase;          /* start_xfer_async + wait_xfer_finish instead of execute   */
+  int reps;               /* transfers run back to back through the same LDS buffer   */
+  int rep_src_bytes;      /* source advance per rep                                   */
+  int rep_index_elmts;    /* index advance per rep                                    */
+} cudadma_run_t;
+
+int cudadma_num_cases(void);
+int cudadma_get_case(int case_id, cudadma_case_t* out);
+int cudadma_run_case(int case_id, const cudadma_run_t* run, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Host-side planner.  cudadma_diagnose prints what the static diagnose()
+ * members of the objects print (include/cudaDMAv2.h:1402-1458, :3208-3493,
+ * :9417-9698).  cudadma_plan_map replays, on the host and with the very code
+ * the device objects use, which DMA thread moves which bytes: map[d] receives
+ * the source byte offset that lands on destination byte d (-1 = untouched),
+ * both relative to the transfer's pointers shifted by src_origin / dst_origin.
+ * Returns the number of destination bytes written more than once (0 for a
+ * sound plan) or a negative error, e.g. when a thread would step outside
+ * [0, map_len).  Needs no GPU.
+ * ---------------------------------------------------------------------- */
+typedef struct cudadma_plan_query {
+  int pattern;            /* CUDADMA_PATTERN_*                                   */
+  int alignment, bytes_per_thread, bytes_per_elmt, dma_threads, num_elmts;
+  int src_stride;         /* strided; scatter: dense-side stride                 */
+  int dst_stride;         /* strided; gather: dense-side stride                  */
+  int radius, corners, dimx, dimy, pitch;   /* halo                              */
+  const int* index;       /* gather / scatter: num_elmts element indices         */
+} cudadma_plan_query_t;
+
+int cudadma_plan_map(const cudadma_plan_query_t* q, long long src_origin, long long dst_origin,
+                     int* map, size_t map_len, int* steps_out);
+int cudadma_diagnose(int pattern, int alignment, int bytes_per_thread, int bytes_per_elmt, int dma_threads,
+                     int num_elmts, int full_template, int verbose);
+
+/* ------------------------------------------------------------------------
+ * Benchmark workloads.  Each launches one persistent-grid kernel built from the
+ * DMA objects; `variant` picks the buffering idiom, as the none / single /
+ * double / manual kernels of src/perf/sequential/perf_sequential.cu:52-223 and
+ * the five stencil kernels of src/examples/stencil do.  Variant 0 is the one the
+ * benchmark reports.  cudadma_num_variants(workload) tells how many exist.
+ * ---------------------------------------------------------------------- */
+enum {
+  CUDADMA_WORKLOAD_SEQUENTIAL = 0,
+  CUDADMA_WORKLOAD_STRIDED    = 1,
+  CUDADMA_WORKLOAD_GATHER     = 2,
+  CUDADMA_WORKLOAD_HALO       = 3,
+  CUDADMA_WORKLOAD_GEMM       = 4
+};
+int cudadma_num_variants(int workload);
+/* One-line description of a variant ("" when out of range). */
+const char* cudadma_variant_name(int workload, int variant);
+/* Tuning knob: workgroups resident per compute unit for the persistent grids
+ * (0 restores each kernel's default).  Returns the previous value. */
+int cudadma_set_workgroups_per_cu(int value);
+
+/* Seeded inputs generated on the device; bit-identical to the host statement
+ * h(i) = splitmix64(seed + i) >> 32, value = (h >> 8) * 2^-23 - 1. */
+int cudadma_fill_uniform(float* d_dst, size_t n, uint64_t seed, void* stream);
+/* Element indices uniform over [0, n_records), one in ten repeating an earlier draw. */
+int cudadma_fill_indices(int32_t* d_dst, size_t n, uint32_t n_records, uint64_t seed, void* stream);
+
+/* Calibration kernel: grid-stride dwordx4 copy with no LDS and no DMA object.
+ * bytes must be a multiple of 16. */
+int cudadma_plain_copy(const void* d_src, void* d_dst, size_t bytes, void* stream);
+
+/* Config 1 (perf_sequential.cu:255-361): copy `bytes` (a multiple of 16 KiB) in
+ * 16 KiB tiles through LDS; 128 DMA + 128 compute threads per workgroup. */
+int cudadma_sequential_copy(const float* d_in, float* d_out, size_t bytes, int variant, void* stream);
+
+/* Config 2: d_out = transpose(d_in) for an n x n float matrix, n a multiple of
+ * 64; CudaDMAStrided pulls 64 rows x 256 B tiles, consumers write them transposed. */
+int cudadma_strided_transpose(const float* d_in, float* d_out, int n, int variant, void* stream);
+
+/* Config 3: records of 128 B; n_idx a multiple of 32.  CudaDMAIndirect gathers
+ * 32 records per LDS tile.
+ *   copy  : d_out[i] = d_table[d_idx[i]]                     (n_idx * 128 B)
+ *   rowsum: d_out[t][j] = sum_{r<32} d_table[d_idx[32t+r]][j] (n_idx/32 * 128 B) */
+int cudadma_gather_copy(const float* d_table, const int32_t* d_idx, float* d_out,
+                        size_t n_records, size_t n_idx, int variant, void* stream);
+int cudadma_gather_rowsum(const float* d_table, const int32_t* d_idx, float* d_out,
+                          size_t n_records, size_t n_idx, int variant, void* stream);
+
+/* Config 4 (src/examples/stencil/cudaDMA_stencil2D.cu:100-240): 8th-order
+ * 25-point star stencil.  d_in is (nx+8) x (ny+8) x (nz+8) floats, x fastest;
+ * d_out is nx x ny x nz.  nx, ny multiples of 32.  CudaDMAHalo brings the ring
+ * of each 32x32 tile, plane by plane along z. */
+int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz, int variant, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUDADMA_AMD_H */

@@ -1,0 +1,276 @@
+// hipDMA: wavefront-specialised DMA objects for AMD CDNA4 (gfx950).
+//
+// This header holds what every DMA object shares: the cache-policy enums, the
+// producer/consumer handshake that stands in for CUDA named barriers, and the
+// CudaDMA base class.  API contract followed: include/cudaDMAv2.h:50-63
+// (qualifier enums) and include/cudaDMAv2.h:1316-1353 (class CudaDMA).
+//
+// Handshake design.  CDNA has no counterpart of `bar.sync id,count` /
+// `bar.arrive id,count`.  Each dmaID owns two monotonically increasing 32-bit
+// words in LDS:
+//     full   counts lanes that have called finish_async_dma()
+//     empty  counts lanes that have called start_async_dma()
+// A signalling wavefront elects one lane which adds the number of active lanes
+// with a single ds_add_u32; a waiting wavefront keeps a private phase number
+// and polls with ds_read_b32 + s_sleep until the word reaches
+// phase * (threads in the signalling group).  The words only ever grow, so a
+// signal that nobody waits for (the "drain" wait_for_dma_start of
+// src/perf/sequential/perf_sequential.cu:139) is harmless either way.
+// Ordering is restricted to the LDS address space: a release before the add
+// (s_waitcnt lgkmcnt(0)), an acquire after the poll.  Outstanding global
+// stores of a consumer therefore do not delay its start_async_dma().
+// Define HIPDMA_FULL_FENCE to order every address space instead.
+//
+// Requirements that differ from the CUDA original:
+//   * DMA and compute groups are made of whole 64-lane wavefronts:
+//     dma_threadIdx_start must be a multiple of 64 (a wavefront must not hold
+//     both roles) and calls must be wavefront-uniform.
+//   * Every thread of the workgroup constructs every warp-specialised object
+//     before the roles branch: the constructor zeroes the two words and
+//     executes one s_barrier.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <cstdio>
+#include <type_traits>
+
+#define HIPDMA_WAVE_SIZE 64
+#define HIPDMA_MAX_DMA_IDS 16
+
+#ifndef HIPDMA_SPIN_SLEEP
+#define HIPDMA_SPIN_SLEEP 1
+#endif
+// A wait gives up after this many polls (about a second) and lets the wavefront
+// run on, so that unbalanced start_async_dma / execute_dma counts end in wrong
+// data and a finished kernel instead of a hung GPU.  0 = wait for ever.
+#ifndef HIPDMA_SPIN_LIMIT
+#define HIPDMA_SPIN_LIMIT (1 << 24)
+#endif
+
+// Load cache policies (names follow include/cudaDMAv2.h:50-56).  On gfx950:
+//   LOAD_CACHE_ALL / LOAD_CACHE_GLOBAL  plain load
+//   LOAD_CACHE_STREAMING / _LAST_USE    non-temporal load (nt bit)
+//   LOAD_CACHE_VOLATILE                 volatile load (sc0 sc1)
+enum CudaDMALoadQualifier {
+  LOAD_CACHE_ALL,
+  LOAD_CACHE_GLOBAL,
+  LOAD_CACHE_STREAMING,
+  LOAD_CACHE_LAST_USE,
+  LOAD_CACHE_VOLATILE,
+};
+
+// Store cache policies (names follow include/cudaDMAv2.h:58-63) plus two
+// additions that only exist here:
+//   STORE_LDS         the destination is known to be LDS: ds_write_b128 instead
+//                     of a generic-address store
+//   STORE_LDS_DIRECT  the destination is LDS and the data never visits a VGPR:
+//                     global_load_lds_dwordx4 writes it straight into LDS.
+//                     Needs a global source; nothing can be issued before the
+//                     buffer is free, so start_xfer_async() only records the
+//                     source and wait_xfer_finish() issues the loads.
+enum CudaDMAStoreQualifier {
+  STORE_WRITE_BACK,
+  STORE_CACHE_GLOBAL,
+  STORE_CACHE_STREAMING,
+  STORE_CACHE_WRITE_THROUGH,
+  STORE_LDS,
+  STORE_LDS_DIRECT,
+};
+
+namespace hipdma {
+namespace detail {
+
+typedef __attribute__((address_space(3))) unsigned lds_word_t;
+
+// Two words per dmaID.  A function-local __shared__ array: every kernel that
+// constructs a warp-specialised object gets its own 128-byte copy and the
+// user never has to pass LDS for it.
+__device__ __forceinline__ lds_word_t* sync_words()
+{
+  __shared__ unsigned words[2 * HIPDMA_MAX_DMA_IDS];
+  return (lds_word_t*)words;
+}
+
+__device__ __forceinline__ void release_lds()
+{
+#ifdef HIPDMA_FULL_FENCE
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+#else
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+#endif
+}
+
+__device__ __forceinline__ void acquire_lds()
+{
+#ifdef HIPDMA_FULL_FENCE
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#else
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#endif
+}
+
+// All active lanes of the calling wavefront arrive at `word`.
+__device__ __forceinline__ void signal_word(lds_word_t* word)
+{
+  release_lds();
+  const unsigned long long active = __builtin_amdgcn_ballot_w64(true);
+  const unsigned lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  if (lane == (unsigned)__builtin_ctzll(active))
+    __hip_atomic_fetch_add(word, (unsigned)__builtin_popcountll(active),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
+// Block until `word` has reached `target` (wrap-around safe).
+__device__ __forceinline__ void wait_word(lds_word_t* word, unsigned target)
+{
+#if HIPDMA_SPIN_LIMIT > 0
+  int polls = 0;
+  while ((int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - target) < 0 &&
+         ++polls < HIPDMA_SPIN_LIMIT)
+    __builtin_amdgcn_s_sleep(HIPDMA_SPIN_SLEEP);
+#else
+  while ((int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - target) < 0)
+    __builtin_amdgcn_s_sleep(HIPDMA_SPIN_SLEEP);
+#endif
+  acquire_lds();
+}
+
+struct no_sync_t {};
+
+__host__ __device__ constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
+__host__ __device__ constexpr int round_up(int a, int b) { return ceil_div(a, b) * b; }
+__host__ __device__ constexpr int pow2_ceil(int v)
+{
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+// Largest power of two that is <= cap and divides v (v > 0).
+__host__ __device__ constexpr int pow2_divisor(int v, int cap)
+{
+  int p = cap;
+  while (p > 1 && (v % p) != 0) p >>= 1;
+  return p;
+}
+
+}  // namespace detail
+}  // namespace hipdma
+
+// Base of every DMA object: role test and the empty/full handshake.
+// Follows include/cudaDMAv2.h:1316-1353; wait_for_dma_start() and
+// finish_async_dma() are public as in include/cudaDMA.h:838-846 because user
+// kernels call them (src/perf/sequential/perf_sequential.cu:139,150).
+class CudaDMA {
+public:
+  // Warp-specialised form.  Must be reached by every thread of the workgroup.
+  __device__ __forceinline__ CudaDMA(const int dmaID,
+                                     const int num_dma_threads,
+                                     const int num_compute_threads,
+                                     const int dma_threadIdx_start)
+    : m_is_dma_thread((int(threadIdx.x) >= dma_threadIdx_start) &&
+                      (int(threadIdx.x) < (dma_threadIdx_start + num_dma_threads))),
+      m_has_sync(true),
+      m_full(hipdma::detail::sync_words() + 2 * dmaID),
+      m_empty(hipdma::detail::sync_words() + 2 * dmaID + 1),
+      m_wait_unit(0),
+      m_wait_target(0)
+  {
+    // A DMA thread waits on `empty` for the compute threads, a compute thread
+    // waits on `full` for the DMA threads.
+    m_wait_unit = m_is_dma_thread ? unsigned(num_compute_threads) : unsigned(num_dma_threads);
+    if (threadIdx.x == 0) {
+      *m_full = 0u;
+      *m_empty = 0u;
+    }
+    __syncthreads();
+  }
+protected:
+  // Form used by objects that are not warp-specialised: no LDS words, no barrier.
+  __device__ __forceinline__ CudaDMA(hipdma::detail::no_sync_t,
+                                     const int num_dma_threads,
+                                     const int dma_threadIdx_start)
+    : m_is_dma_thread((int(threadIdx.x) >= dma_threadIdx_start) &&
+                      (int(threadIdx.x) < (dma_threadIdx_start + num_dma_threads))),
+      m_has_sync(false),
+      m_full(nullptr),
+      m_empty(nullptr),
+      m_wait_unit(0),
+      m_wait_target(0)
+  {
+  }
+public:
+  // Compute side: the buffer is free, the DMA wavefronts may overwrite it.  Does not block.
+  __device__ __forceinline__ void start_async_dma(void) const
+  {
+    if (m_has_sync) hipdma::detail::signal_word(m_empty);
+  }
+  // Compute side: block until the DMA wavefronts have filled the buffer.
+  __device__ __forceinline__ void wait_for_dma_finish(void) const
+  {
+    if (m_has_sync) {
+      m_wait_target += m_wait_unit;
+      hipdma::detail::wait_word(m_full, m_wait_target);
+    }
+  }
+  __device__ __forceinline__ bool owns_this_thread(void) const { return m_is_dma_thread; }
+  // DMA side: block until every compute thread has released the buffer.
+  __device__ __forceinline__ void wait_for_dma_start(void) const
+  {
+    if (m_has_sync) {
+      m_wait_target += m_wait_unit;
+      hipdma::detail::wait_word(m_empty, m_wait_target);
+    }
+  }
+  // DMA side: the buffer is full.  Does not block.
+  __device__ __forceinline__ void finish_async_dma(void) const
+  {
+    if (m_has_sync) hipdma::detail::signal_word(m_full);
+  }
+protected:
+  const bool m_is_dma_thread;
+  const bool m_has_sync;
+  hipdma::detail::lds_word_t* const m_full;
+  hipdma::detail::lds_word_t* const m_empty;
+  unsigned m_wait_unit;
+  mutable unsigned m_wait_target;
+};
+
+namespace hipdma {
+
+// Barrier among a subset of the workgroup's wavefronts: what `bar.sync id,count`
+// gives CUDA code that wants its compute warps to meet without the DMA warps.
+// Uses the LDS word pair of slot `id` (shared numbering with dmaID: give it an
+// id no DMA object of the kernel uses).  Every thread of the workgroup
+// constructs it; only the `num_threads` participants call sync().
+class GroupBarrier {
+public:
+  __device__ __forceinline__ GroupBarrier(const int id, const int num_threads)
+    : m_word(detail::sync_words() + 2 * id), m_unit(unsigned(num_threads)), m_target(0)
+  {
+    if (threadIdx.x == 0) *m_word = 0u;
+    __syncthreads();
+  }
+  __device__ __forceinline__ void sync()
+  {
+    m_target += m_unit;
+    detail::signal_word(m_word);
+    detail::wait_word(m_word, m_target);
+  }
+private:
+  detail::lds_word_t* const m_word;
+  const unsigned m_unit;
+  unsigned m_target;
+};
+
+}  // namespace hipdma
+
+// Sync-only object for hand-written transfer code (include/cudaDMA.h:4184-4208).
+class cudaDMACustom : public CudaDMA {
+public:
+  __device__ __forceinline__ cudaDMACustom(const int dmaID,
+                                           const int num_dma_threads,
+                                           const int num_compute_threads,
+                                           const int dma_threadIdx_start)
+    : CudaDMA(dmaID, num_dma_threads, num_compute_threads, dma_threadIdx_start) {}
+};
+typedef cudaDMACustom CudaDMACustom;

@@ -1,0 +1,173 @@
+// hipDMA memory primitives: fixed-size register chunks and the loads/stores
+// that fill and drain them.  Plays the role of the PTX ld/st wrappers of
+// include/cudaDMAv2.h:80-679 and of the register buffers of
+// include/cudaDMAv2.h:686-1310, for gfx950:
+//   * a chunk is ALIGNMENT bytes (4, 8 or 16) = 1, 2 or 4 VGPRs and is moved by
+//     global_load_dword/x2/x4 (source known global), flat_load_* (generic
+//     source), ds_write_b32/b64/b128 (destination known LDS) or a generic store;
+//   * a ragged tail of 4, 8 or 12 bytes is moved in dword pieces;
+//   * the direct path uses global_load_lds_dwordx4 / _dword, which writes
+//     M0-base + lane*size in LDS without touching a VGPR.
+#pragma once
+
+#include "base.hpp"
+
+namespace hipdma {
+namespace detail {
+
+typedef unsigned u32x1_t;
+typedef unsigned u32x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+
+template<int BYTES> struct chunk_of;
+template<> struct chunk_of<4>  { typedef u32x1_t type; };
+template<> struct chunk_of<8>  { typedef u32x2_t type; };
+template<> struct chunk_of<16> { typedef u32x4_t type; };
+
+#define HIPDMA_GLOBAL_AS __attribute__((address_space(1)))
+#define HIPDMA_LDS_AS    __attribute__((address_space(3)))
+
+// One aligned vector load of sizeof(T) bytes.
+template<typename T, bool GLOBAL_LOAD, int LOAD_QUAL>
+__device__ __forceinline__ T load_vec(const void* ptr)
+{
+  if constexpr (GLOBAL_LOAD) {
+    const HIPDMA_GLOBAL_AS T* p = (const HIPDMA_GLOBAL_AS T*)ptr;
+    if constexpr (LOAD_QUAL == LOAD_CACHE_STREAMING || LOAD_QUAL == LOAD_CACHE_LAST_USE)
+      return __builtin_nontemporal_load(p);
+    else if constexpr (LOAD_QUAL == LOAD_CACHE_VOLATILE)
+      return *(const volatile HIPDMA_GLOBAL_AS T*)p;
+    else
+      return *p;
+  } else {
+    const T* p = (const T*)ptr;
+    if constexpr (LOAD_QUAL == LOAD_CACHE_STREAMING || LOAD_QUAL == LOAD_CACHE_LAST_USE)
+      return __builtin_nontemporal_load(p);
+    else if constexpr (LOAD_QUAL == LOAD_CACHE_VOLATILE)
+      return *(const volatile T*)p;
+    else
+      return *p;
+  }
+}
+
+// One aligned vector store of sizeof(T) bytes.
+template<typename T, int STORE_QUAL>
+__device__ __forceinline__ void store_vec(const T& value, void* ptr)
+{
+  if constexpr (STORE_QUAL == STORE_LDS || STORE_QUAL == STORE_LDS_DIRECT) {
+    *(HIPDMA_LDS_AS T*)ptr = value;
+  } else if constexpr (STORE_QUAL == STORE_CACHE_STREAMING) {
+    __builtin_nontemporal_store(value, (T*)ptr);
+  } else if constexpr (STORE_QUAL == STORE_CACHE_WRITE_THROUGH) {
+    *(volatile T*)ptr = value;
+  } else {
+    *(T*)ptr = value;
+  }
+}
+
+// Word i of a chunk (i is a compile-time constant after unrolling).
+template<typename C>
+__device__ __forceinline__ unsigned get_word(const C& c, const int i)
+{
+  if constexpr (std::is_same<C, u32x1_t>::value) return c; else return c[i];
+}
+template<typename C>
+__device__ __forceinline__ void set_word(C& c, const int i, const unsigned v)
+{
+  if constexpr (std::is_same<C, u32x1_t>::value) c = v; else c[i] = v;
+}
+
+// Fill the first `nbytes` (a multiple of 4, 0 < nbytes <= CHUNK) of a CHUNK-byte
+// register chunk from an address that is only guaranteed PIECE-byte aligned.
+// PIECE == CHUNK and nbytes == CHUNK is the single-instruction fast path.
+template<int CHUNK, int PIECE, bool GLOBAL_LOAD, int LOAD_QUAL>
+__device__ __forceinline__ void load_chunk(typename chunk_of<CHUNK>::type& c, const char* ptr, const int nbytes)
+{
+  typedef typename chunk_of<CHUNK>::type chunk_t;
+  if constexpr (PIECE == CHUNK) {
+    if (nbytes == CHUNK) {
+      c = load_vec<chunk_t, GLOBAL_LOAD, LOAD_QUAL>(ptr);
+      return;
+    }
+  }
+  typedef typename chunk_of<PIECE>::type piece_t;
+  constexpr int WORDS_PER_PIECE = PIECE / 4;
+#pragma unroll
+  for (int p = 0; p < CHUNK / PIECE; ++p) {
+    const int rem = nbytes - p * PIECE;
+    if (rem >= PIECE) {
+      const piece_t v = load_vec<piece_t, GLOBAL_LOAD, LOAD_QUAL>(ptr + p * PIECE);
+#pragma unroll
+      for (int w = 0; w < WORDS_PER_PIECE; ++w)
+        set_word(c, p * WORDS_PER_PIECE + w, get_word(v, w));
+    } else {
+#pragma unroll
+      for (int w = 0; w < WORDS_PER_PIECE; ++w)
+        if (rem > 4 * w)
+          set_word(c, p * WORDS_PER_PIECE + w,
+                   load_vec<u32x1_t, GLOBAL_LOAD, LOAD_QUAL>(ptr + p * PIECE + 4 * w));
+    }
+  }
+}
+
+template<int CHUNK, int PIECE, int STORE_QUAL>
+__device__ __forceinline__ void store_chunk(const typename chunk_of<CHUNK>::type& c, char* ptr, const int nbytes)
+{
+  typedef typename chunk_of<CHUNK>::type chunk_t;
+  if constexpr (PIECE == CHUNK) {
+    if (nbytes == CHUNK) {
+      store_vec<chunk_t, STORE_QUAL>(c, ptr);
+      return;
+    }
+  }
+  typedef typename chunk_of<PIECE>::type piece_t;
+  constexpr int WORDS_PER_PIECE = PIECE / 4;
+#pragma unroll
+  for (int p = 0; p < CHUNK / PIECE; ++p) {
+    const int rem = nbytes - p * PIECE;
+    if (rem >= PIECE) {
+      piece_t v;
+#pragma unroll
+      for (int w = 0; w < WORDS_PER_PIECE; ++w)
+        set_word(v, w, get_word(c, p * WORDS_PER_PIECE + w));
+      store_vec<piece_t, STORE_QUAL>(v, ptr + p * PIECE);
+    } else {
+#pragma unroll
+      for (int w = 0; w < WORDS_PER_PIECE; ++w)
+        if (rem > 4 * w)
+          store_vec<u32x1_t, STORE_QUAL>(get_word(c, p * WORDS_PER_PIECE + w), ptr + p * PIECE + 4 * w);
+    }
+  }
+}
+
+// Direct global -> LDS move of BYTES (4 or 16) per active lane.  `lds_wave_base`
+// must be the same for every lane of the wavefront; lane L lands at
+// lds_wave_base + L*BYTES.
+template<int BYTES>
+__device__ __forceinline__ void load_to_lds(const char* global_lane_ptr, char* lds_wave_base)
+{
+  static_assert(BYTES == 4 || BYTES == 16, "global_load_lds moves 4 or 16 bytes per lane here");
+  // the size operand has to be a literal
+  if constexpr (BYTES == 16)
+    __builtin_amdgcn_global_load_lds((const HIPDMA_GLOBAL_AS void*)global_lane_ptr,
+                                     (HIPDMA_LDS_AS void*)lds_wave_base, 16, 0, 0);
+  else
+    __builtin_amdgcn_global_load_lds((const HIPDMA_GLOBAL_AS void*)global_lane_ptr,
+                                     (HIPDMA_LDS_AS void*)lds_wave_base, 4, 0, 0);
+}
+
+// Wait until every global -> LDS move of this wavefront has landed.
+__device__ __forceinline__ void wait_lds_direct()
+{
+  // s_waitcnt vmcnt(0): simm16 = vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14]
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+}
+
+// Lane number inside the wavefront.
+__device__ __forceinline__ int lane_id()
+{
+  return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+}  // namespace detail
+}  // namespace hipdma

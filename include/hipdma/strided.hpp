@@ -1,0 +1,285 @@
+// CudaDMAStrided: 2-D transfer, dst[i*dst_stride + j] = src[i*src_stride + j]
+// for i < NUM_ELMTS, j < BYTES_PER_ELMT.
+//
+// API contract: include/cudaDMAv2.h:2973-9368 (template parameters :3193-3194;
+// warp-specialised constructors :5110-5163, :6298-6330, :7480-7510, :8610-8651;
+// the other constructors :5556-5604, :6728-6760, :7877-7905, :8993-9030;
+// diagnose :3208-3493).  The work split is the slot grid of grid.hpp.
+#pragma once
+
+#include "grid.hpp"
+
+template<bool DO_SYNC = false, int ALIGNMENT = 0, int BYTES_PER_THREAD = 4 * ALIGNMENT,
+         int BYTES_PER_ELMT = 0, int DMA_THREADS = 0, int NUM_ELMTS = 0>
+class CudaDMAStrided : public CudaDMA {
+  static_assert(ALIGNMENT == 4 || ALIGNMENT == 8 || ALIGNMENT == 16, "ALIGNMENT must be 4, 8 or 16");
+  static_assert((BYTES_PER_THREAD / ALIGNMENT) > 0, "BYTES_PER_THREAD must hold at least one chunk");
+  static_assert((BYTES_PER_THREAD % ALIGNMENT) == 0, "BYTES_PER_THREAD must be a multiple of ALIGNMENT");
+  static_assert((BYTES_PER_ELMT % 4) == 0, "sizes are multiples of 4 bytes");
+  static constexpr int LEVEL = (BYTES_PER_ELMT == 0) ? 1 : (DMA_THREADS == 0) ? 2 : (NUM_ELMTS == 0) ? 3 : 4;
+  static constexpr int MAX_LDS = BYTES_PER_THREAD / ALIGNMENT;
+  typedef typename hipdma::detail::chunk_of<ALIGNMENT>::type chunk_t;
+  template<bool C> using when = typename std::enable_if<C, int>::type;
+public:
+  // ---- warp-specialised constructors: one stride for both sides, or src and dst strides ----
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 1) && S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int dmaID, const int num_dma_threads, const int num_compute_threads,
+                                            const int dma_threadIdx_start, const int elmt_size_in_bytes,
+                                            const int num_elements, const int elmt_stride)
+    : CudaDMA(dmaID, num_dma_threads, num_compute_threads, dma_threadIdx_start)
+  { init(elmt_size_in_bytes, num_elements, num_dma_threads, dma_threadIdx_start, elmt_stride, elmt_stride); }
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 1) && S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int dmaID, const int num_dma_threads, const int num_compute_threads,
+                                            const int dma_threadIdx_start, const int elmt_size_in_bytes,
+                                            const int num_elements, const int src_stride, const int dst_stride)
+    : CudaDMA(dmaID, num_dma_threads, num_compute_threads, dma_threadIdx_start)
+  { init(elmt_size_in_bytes, num_elements, num_dma_threads, dma_threadIdx_start, src_stride, dst_stride); }
+
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 2) && S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int dmaID, const int num_dma_threads, const int num_compute_threads,
+                                            const int dma_threadIdx_start, const int num_elements,
+                                            const int elmt_stride)
+    : CudaDMA(dmaID, num_dma_threads, num_compute_threads, dma_threadIdx_start)
+  { init(BYTES_PER_ELMT, num_elements, num_dma_threads, dma_threadIdx_start, elmt_stride, elmt_stride); }
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 2) && S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int dmaID, const int num_dma_threads, const int num_compute_threads,
+                                            const int dma_threadIdx_start, const int num_elements,
+                                            const int src_stride, const int dst_stride)
+    : CudaDMA(dmaID, num_dma_threads, num_compute_threads, dma_threadIdx_start)
+  { init(BYTES_PER_ELMT, num_elements, num_dma_threads, dma_threadIdx_start, src_stride, dst_stride); }
+
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 3) && S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int dmaID, const int num_compute_threads,
+                                            const int dma_threadIdx_start, const int num_elements,
+                                            const int elmt_stride)
+    : CudaDMA(dmaID, DMA_THREADS, num_compute_threads, dma_threadIdx_start)
+  { init(BYTES_PER_ELMT, num_elements, DMA_THREADS, dma_threadIdx_start, elmt_stride, elmt_stride); }
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 3) && S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int dmaID, const int num_compute_threads,
+                                            const int dma_threadIdx_start, const int num_elements,
+                                            const int src_stride, const int dst_stride)
+    : CudaDMA(dmaID, DMA_THREADS, num_compute_threads, dma_threadIdx_start)
+  { init(BYTES_PER_ELMT, num_elements, DMA_THREADS, dma_threadIdx_start, src_stride, dst_stride); }
+
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 4) && S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int dmaID, const int num_compute_threads,
+                                            const int dma_threadIdx_start, const int elmt_stride)
+    : CudaDMA(dmaID, DMA_THREADS, num_compute_threads, dma_threadIdx_start)
+  { init(BYTES_PER_ELMT, NUM_ELMTS, DMA_THREADS, dma_threadIdx_start, elmt_stride, elmt_stride); }
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 4) && S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int dmaID, const int num_compute_threads,
+                                            const int dma_threadIdx_start, const int src_stride,
+                                            const int dst_stride)
+    : CudaDMA(dmaID, DMA_THREADS, num_compute_threads, dma_threadIdx_start)
+  { init(BYTES_PER_ELMT, NUM_ELMTS, DMA_THREADS, dma_threadIdx_start, src_stride, dst_stride); }
+
+  // ---- constructors of the form that is not warp-specialised ----
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 1) && !S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int elmt_size_in_bytes, const int num_elements,
+                                            const int elmt_stride)
+    : CudaDMA(hipdma::detail::no_sync_t(), int(blockDim.x), 0)
+  { init(elmt_size_in_bytes, num_elements, int(blockDim.x), 0, elmt_stride, elmt_stride); }
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 1) && !S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int elmt_size_in_bytes, const int num_elements,
+                                            const int src_stride, const int dst_stride,
+                                            const int num_dma_threads = 0, const int dma_threadIdx_start = 0)
+    : CudaDMA(hipdma::detail::no_sync_t(), threads_or_block(num_dma_threads), dma_threadIdx_start)
+  { init(elmt_size_in_bytes, num_elements, threads_or_block(num_dma_threads), dma_threadIdx_start, src_stride, dst_stride); }
+
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 2) && !S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int num_elements, const int elmt_stride)
+    : CudaDMA(hipdma::detail::no_sync_t(), int(blockDim.x), 0)
+  { init(BYTES_PER_ELMT, num_elements, int(blockDim.x), 0, elmt_stride, elmt_stride); }
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 2) && !S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int num_elements, const int src_stride, const int dst_stride,
+                                            const int num_dma_threads = 0, const int dma_threadIdx_start = 0)
+    : CudaDMA(hipdma::detail::no_sync_t(), threads_or_block(num_dma_threads), dma_threadIdx_start)
+  { init(BYTES_PER_ELMT, num_elements, threads_or_block(num_dma_threads), dma_threadIdx_start, src_stride, dst_stride); }
+
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 3) && !S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int num_elements, const int elmt_stride)
+    : CudaDMA(hipdma::detail::no_sync_t(), DMA_THREADS, 0)
+  { init(BYTES_PER_ELMT, num_elements, DMA_THREADS, 0, elmt_stride, elmt_stride); }
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 3) && !S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int num_elements, const int src_stride, const int dst_stride,
+                                            const int dma_threadIdx_start = 0)
+    : CudaDMA(hipdma::detail::no_sync_t(), DMA_THREADS, dma_threadIdx_start)
+  { init(BYTES_PER_ELMT, num_elements, DMA_THREADS, dma_threadIdx_start, src_stride, dst_stride); }
+
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 4) && !S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int elmt_stride)
+    : CudaDMA(hipdma::detail::no_sync_t(), DMA_THREADS, 0)
+  { init(BYTES_PER_ELMT, NUM_ELMTS, DMA_THREADS, 0, elmt_stride, elmt_stride); }
+  template<int L = LEVEL, bool S = DO_SYNC, when<(L == 4) && !S> = 0>
+  __device__ __forceinline__ CudaDMAStrided(const int src_stride, const int dst_stride,
+                                            const int dma_threadIdx_start = 0)
+    : CudaDMA(hipdma::detail::no_sync_t(), DMA_THREADS, dma_threadIdx_start)
+  { init(BYTES_PER_ELMT, NUM_ELMTS, DMA_THREADS, dma_threadIdx_start, src_stride, dst_stride); }
+
+public:
+  __device__ __forceinline__ void execute_dma(const void* __restrict__ src_ptr, void* __restrict__ dst_ptr)
+  { execute_dma<false, LOAD_CACHE_ALL, STORE_WRITE_BACK>(src_ptr, dst_ptr); }
+  __device__ __forceinline__ void start_xfer_async(const void* __restrict__ src_ptr)
+  { start_xfer_async<false, LOAD_CACHE_ALL, STORE_WRITE_BACK>(src_ptr); }
+  __device__ __forceinline__ void wait_xfer_finish(void* __restrict__ dst_ptr)
+  { wait_xfer_finish<false, LOAD_CACHE_ALL, STORE_WRITE_BACK>(dst_ptr); }
+
+  template<bool DMA_GLOBAL_LOAD>
+  __device__ __forceinline__ void execute_dma(const void* __restrict__ src_ptr, void* __restrict__ dst_ptr)
+  { execute_dma<DMA_GLOBAL_LOAD, LOAD_CACHE_ALL, STORE_WRITE_BACK>(src_ptr, dst_ptr); }
+  template<bool DMA_GLOBAL_LOAD>
+  __device__ __forceinline__ void start_xfer_async(const void* __restrict__ src_ptr)
+  { start_xfer_async<DMA_GLOBAL_LOAD, LOAD_CACHE_ALL, STORE_WRITE_BACK>(src_ptr); }
+  template<bool DMA_GLOBAL_LOAD>
+  __device__ __forceinline__ void wait_xfer_finish(void* __restrict__ dst_ptr)
+  { wait_xfer_finish<DMA_GLOBAL_LOAD, LOAD_CACHE_ALL, STORE_WRITE_BACK>(dst_ptr); }
+
+  template<bool DMA_GLOBAL_LOAD, int DMA_LOAD_QUAL, int DMA_STORE_QUAL>
+  __device__ __forceinline__ void execute_dma(const void* __restrict__ src_ptr, void* __restrict__ dst_ptr)
+  {
+    start_xfer_async<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL, DMA_STORE_QUAL>(src_ptr);
+    wait_xfer_finish<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL, DMA_STORE_QUAL>(dst_ptr);
+  }
+
+  template<bool DMA_GLOBAL_LOAD, int DMA_LOAD_QUAL, int DMA_STORE_QUAL>
+  __device__ __forceinline__ void start_xfer_async(const void* __restrict__ src_ptr)
+  {
+    m_src = (const char*)src_ptr;
+    if (use_direct<DMA_STORE_QUAL>()) return;
+    load_step<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL>(0, m_grid.begin());
+  }
+
+  template<bool DMA_GLOBAL_LOAD, int DMA_LOAD_QUAL, int DMA_STORE_QUAL>
+  __device__ __forceinline__ void wait_xfer_finish(void* __restrict__ dst_ptr)
+  {
+    if constexpr (DO_SYNC) CudaDMA::wait_for_dma_start();
+    if (use_direct<DMA_STORE_QUAL>()) {
+      if constexpr (DMA_STORE_QUAL == STORE_LDS_DIRECT) {
+        static_assert(DMA_STORE_QUAL != STORE_LDS_DIRECT || DMA_GLOBAL_LOAD,
+                      "STORE_LDS_DIRECT needs a global source");
+        direct_all((char*)dst_ptr);
+      }
+    } else {
+      hipdma::detail::GridCursor cur = m_grid.begin();
+      store_step<DMA_STORE_QUAL>((char*)dst_ptr, 0, cur);
+      for (int step = 1; step < m_grid.steps; ++step) {
+        load_step<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL>(step, cur);
+        store_step<DMA_STORE_QUAL>((char*)dst_ptr, step, cur);
+      }
+    }
+    if constexpr (DO_SYNC) CudaDMA::finish_async_dma();
+  }
+
+private:
+  __device__ __forceinline__ static int threads_or_block(const int n) { return (n <= 0) ? int(blockDim.x) : n; }
+
+  __device__ __forceinline__ void init(const int e, const int n, const int t, const int start,
+                                       const int src_stride, const int dst_stride)
+  {
+    m_grid.init(ALIGNMENT, MAX_LDS, e, n, t, int(threadIdx.x) - start);
+    m_src_stride = src_stride;
+    m_dst_stride = dst_stride;
+  }
+
+  // The direct path needs the 64 lanes of a wavefront to land on 64 consecutive
+  // chunks of LDS: rows at least one wavefront wide, or unpadded rows packed
+  // back to back.  Otherwise the register path is taken.
+  template<int STORE_QUAL>
+  __device__ __forceinline__ bool use_direct() const
+  {
+    if constexpr (STORE_QUAL == STORE_LDS_DIRECT && (ALIGNMENT == 16 || ALIGNMENT == 4))
+      return (m_grid.last_bytes == ALIGNMENT) && ((m_grid.T % HIPDMA_WAVE_SIZE) == 0) &&
+             ((m_grid.W >= HIPDMA_WAVE_SIZE) ||
+              ((m_grid.W == m_grid.LPE) && (m_dst_stride == m_grid.E)));
+    else
+      return false;
+  }
+
+  template<bool GLOBAL_LOAD, int LOAD_QUAL>
+  __device__ __forceinline__ void load_step(const int step, hipdma::detail::GridCursor cur)
+  {
+    using namespace hipdma::detail;
+#pragma unroll
+    for (int k = 0; k < MAX_LDS; ++k) {
+      if (m_grid.live(step * MAX_LDS + k, cur))
+        load_chunk<ALIGNMENT, ALIGNMENT, GLOBAL_LOAD, LOAD_QUAL>(
+            m_buf[k], m_src + cur.row * m_src_stride + cur.col * ALIGNMENT, m_grid.chunk_bytes(ALIGNMENT, cur));
+      m_grid.advance(cur);
+    }
+  }
+
+  // Drains the registers of `step` and leaves `cur` at the first slot of the next step.
+  template<int STORE_QUAL>
+  __device__ __forceinline__ void store_step(char* dst, const int step, hipdma::detail::GridCursor& cur) const
+  {
+    using namespace hipdma::detail;
+#pragma unroll
+    for (int k = 0; k < MAX_LDS; ++k) {
+      if (m_grid.live(step * MAX_LDS + k, cur))
+        store_chunk<ALIGNMENT, ALIGNMENT, STORE_QUAL>(
+            m_buf[k], dst + cur.row * m_dst_stride + cur.col * ALIGNMENT, m_grid.chunk_bytes(ALIGNMENT, cur));
+      m_grid.advance(cur);
+    }
+  }
+
+  __device__ __forceinline__ void direct_all(char* dst)
+  {
+    using namespace hipdma::detail;
+    const int lane = lane_id();
+    GridCursor cur = m_grid.begin();
+    for (int r = 0; r < m_grid.rounds; ++r) {
+      if (m_grid.live(r, cur)) {
+        const int lds_off = cur.row * m_dst_stride + cur.col * ALIGNMENT;
+        if constexpr (ALIGNMENT == 16 || ALIGNMENT == 4)
+          load_to_lds<ALIGNMENT>(m_src + cur.row * m_src_stride + cur.col * ALIGNMENT,
+                                 dst + (lds_off - lane * ALIGNMENT));
+      }
+      m_grid.advance(cur);
+    }
+    wait_lds_direct();
+  }
+
+private:
+  hipdma::detail::GridState m_grid;
+  int m_src_stride;
+  int m_dst_stride;
+  const char* m_src;
+  chunk_t m_buf[MAX_LDS];
+};
+
+// Host-side planner report (include/cudaDMAv2.h:3208-3493).
+template<bool DO_SYNC>
+class CudaDMAStrided<DO_SYNC, 0, 0, 0, 0, 0> {
+public:
+  __host__ static void diagnose(const int ALIGNMENT, const int BYTES_PER_THREAD, const int BYTES_PER_ELMT,
+                                const int DMA_THREADS, const int NUM_ELMTS, const bool FULL_TEMPLATE,
+                                const bool verbose = false)
+  {
+    const hipdma::GridPlan p(ALIGNMENT, BYTES_PER_THREAD, BYTES_PER_ELMT, DMA_THREADS, NUM_ELMTS);
+    fprintf(stdout, "==== CudaDMAStrided plan (gfx950, 64-lane wavefronts) ====\n");
+    fprintf(stdout, "  ALIGNMENT %d  BYTES_PER_THREAD %d  BYTES_PER_ELMT %d  DMA_THREADS %d (%d wavefronts)  NUM_ELMTS %d  %s\n",
+            ALIGNMENT, BYTES_PER_THREAD, BYTES_PER_ELMT, DMA_THREADS,
+            (DMA_THREADS + HIPDMA_WAVE_SIZE - 1) / HIPDMA_WAVE_SIZE, NUM_ELMTS,
+            FULL_TEMPLATE ? "compile-time parameters" : "run-time parameters");
+    if (p.slots_per_row <= HIPDMA_WAVE_SIZE)
+      fprintf(stdout, "  layout: %d loads per element, %d lanes per element, %d elements per wavefront load\n",
+              p.loads_per_elmt, p.slots_per_row, HIPDMA_WAVE_SIZE / p.slots_per_row);
+    else
+      fprintf(stdout, "  layout: %d loads per element, %d wavefront loads per element\n",
+              p.loads_per_elmt, p.slots_per_row / HIPDMA_WAVE_SIZE);
+    if (p.slots_per_row != p.loads_per_elmt)
+      fprintf(stdout, "  %d of every %d lanes idle: element size is not a power-of-two (or 64x) number of loads\n",
+              p.slots_per_row - p.loads_per_elmt, p.slots_per_row);
+    fprintf(stdout, "  loads per thread: %d, registers hold %d -> %d step(s)\n", p.rounds, p.loads_per_step, p.total_steps);
+    if (p.total_steps <= 1)
+      fprintf(stdout, "  single step: every load is issued before the handshake wait.\n");
+    else
+      fprintf(stdout, "  multiple steps: to reach one step use BYTES_PER_THREAD >= %d or DMA_THREADS >= %d\n",
+              p.rounds * ALIGNMENT,
+              hipdma::detail::round_up(hipdma::detail::ceil_div(NUM_ELMTS * p.slots_per_row, p.loads_per_step), HIPDMA_WAVE_SIZE));
+    if (verbose)
+      fprintf(stdout, "  loads_per_elmt %d  slots_per_row %d  last_chunk_bytes %d  rounds %d  sure_rounds %d  total_steps %d\n",
+              p.loads_per_elmt, p.slots_per_row, p.last_chunk_bytes, p.rounds, p.sure_rounds, p.total_steps);
+    fflush(stdout);
+  }
+};

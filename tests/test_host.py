@@ -1,0 +1,151 @@
+"""CPU-side tests of libcudadma_amd.so: it loads, exports what include/cudadma_amd.h declares,
+validates arguments before touching a GPU, and its host replay of the device objects' index
+arithmetic agrees with the oracle's closed forms for every compiled case."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import cudadma_amd as cd
+from tests.cases import CaseIO, case_id_str
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "cudadma_amd.h")).read()
+    declared = set(re.findall(r"\b(cudadma_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    L = ctypes.CDLL(cd.lib_path())
+    for name in sorted(declared):
+        assert hasattr(L, name), f"{name} is declared in cudadma_amd.h but not exported"
+    assert declared == set(cd._lib.exported_symbols())
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(cd._lib, "_lib", None)
+    monkeypatch.setattr(cd._lib, "lib_path", lambda: "/nonexistent/libcudadma_amd.so")
+    with pytest.raises(cd.CudaDMAError, match="no fallback"):
+        cd._lib.lib()
+
+
+def test_case_table_is_sane():
+    cases = cd.harness.all_cases()
+    assert len(cases) >= 150
+    patterns = [c.pattern for c in cases]
+    assert patterns == sorted(patterns)
+    for p in range(5):
+        assert patterns.count(p) >= 10
+    for c in cases:
+        assert c.alignment in (4, 8, 16)
+        assert c.bytes_per_thread % c.alignment == 0 and c.bytes_per_thread > 0
+        assert c.dma_threads % 64 == 0 and 64 <= c.dma_threads <= 960
+    # every constructor form is compiled: each (pattern, warp_specialized, level) combination exists
+    seen = {(c.pattern, c.warp_specialized, c.level) for c in cases}
+    for p, levels in ((0, (1, 2, 3)), (1, (1, 2, 3, 4)), (2, (1, 2, 3, 4)), (4, (1, 2, 3))):
+        for ws in (0, 1):
+            for lv in levels:
+                assert (p, ws, lv) in seen, (p, ws, lv)
+    assert (cd.PATTERN_HALO, 1, 0) in seen          # the older cudaDMAHalo class
+    with pytest.raises(cd.CudaDMAError):
+        cd.harness.get_case(len(cases))
+
+
+def test_run_case_validates_before_launching():
+    r = cd.RunArgs(d_in=0, d_out=0, lds_bytes=1024, reps=1)
+    L = cd.lib()
+    assert L.cudadma_run_case(0, ctypes.byref(r), None) == -1
+    assert b"d_in" in L.cudadma_last_error()
+    r = cd.RunArgs(d_in=4096, d_out=8192, lds_bytes=1000, reps=1)
+    assert L.cudadma_run_case(0, ctypes.byref(r), None) == -1
+    assert b"lds_bytes" in L.cudadma_last_error()
+    r = cd.RunArgs(d_in=4096, d_out=8192, lds_bytes=1024, reps=1, src_offset_bytes=2)
+    assert L.cudadma_run_case(0, ctypes.byref(r), None) == -1
+    assert L.cudadma_run_case(10 ** 6, ctypes.byref(r), None) == -3
+    # workloads: sizes and variants are checked first
+    assert L.cudadma_sequential_copy(4096, 8192, 1000, 0, None) == -1
+    assert L.cudadma_sequential_copy(4096, 8192, 16384, 99, None) == -3
+    assert L.cudadma_strided_transpose(4096, 8192, 100, 0, None) == -1
+    assert L.cudadma_gather_copy(4096, 4096, 8192, 16, 33, 0, None) == -1
+    assert L.cudadma_halo_stencil(4096, 8192, 33, 32, 8, 0, None) == -1
+    assert L.cudadma_plain_copy(4096, 8192, 10, None) == -1
+
+
+def test_variants_are_described():
+    for w, least in ((cd.workloads.SEQUENTIAL, 4), (cd.workloads.STRIDED, 2), (cd.workloads.GATHER, 2),
+                     (cd.workloads.HALO, 2)):
+        n = cd.workloads.num_variants(w)
+        assert n >= least
+        for v in range(n):
+            assert cd.workloads.variant_name(w, v)
+        assert cd.workloads.variant_name(w, n) == ""
+    assert cd.workloads.num_variants(99) == 0
+
+
+def test_diagnose_prints_the_plan(capfd):
+    cd.plan.diagnose(cd.PATTERN_SEQUENTIAL, 16, 128, 16384, 128, 0, True, True)
+    cd.plan.diagnose(cd.PATTERN_SEQUENTIAL, 16, 64, 16384, 64)
+    cd.plan.diagnose(cd.PATTERN_STRIDED, 16, 128, 256, 128, 64, True, True)
+    cd.plan.diagnose(cd.PATTERN_GATHER, 16, 32, 128, 128, 32)
+    out = capfd.readouterr().out
+    assert "steps needed: 1 (1 full + 0 partial)" in out
+    assert "steps needed: 4 (4 full + 0 partial)" in out and "DMA_THREADS >= 256" in out
+    assert "16 lanes per element, 4 elements per wavefront load" in out
+    assert "gather" in out
+    with pytest.raises(cd.CudaDMAError):
+        cd.plan.diagnose(cd.PATTERN_HALO, 16, 32, 128, 128, 32)
+
+
+_CASES = cd.harness.all_cases()
+
+
+@pytest.mark.parametrize("case_id", range(len(_CASES)), ids=[case_id_str(i, c) for i, c in enumerate(_CASES)])
+def test_replay_of_every_compiled_case_matches_the_oracle(case_id):
+    """Every destination byte is written exactly once and with the byte the closed form names."""
+    case = _CASES[case_id]
+    for flavour in (0, 1):
+        io = CaseIO(case, flavour=flavour, reps=1)
+        got, steps, doubles = io.replay_map()
+        want = io.expected_map()
+        if case.pattern == cd.PATTERN_GATHER:
+            assert doubles == 0
+        else:
+            assert doubles == 0, f"{doubles} bytes written twice"
+        assert np.array_equal(got, want)
+        assert steps >= 1
+
+
+def test_replay_on_random_parameters():
+    """The reference fuzz distribution (src/tests/test_strided/param_sweep_v2.py:51-75) on the host replay."""
+    rng = np.random.default_rng(99)
+    O = __import__("tests.oracle_lib", fromlist=["x"]).load()
+    from tests.oracle_lib import ptr
+    for _ in range(300):
+        a = int(rng.choice([4, 8, 16]))
+        bpt = a * int(rng.integers(1, 9))
+        e = 4 * max(1, abs(int(np.ceil(rng.normal(256, 256)))))
+        n = int(rng.integers(1, 33))
+        t = 64 * int(rng.integers(1, 17))
+        ss = (e + a - 1) // a * a + a * int(rng.integers(0, 3))
+        ds = (e + a - 1) // a * a + a * int(rng.integers(0, 3))
+        ids = np.arange(n * ss + 64, dtype=np.int32)
+        want = np.full(n * ds + 64, -1, dtype=np.int32)
+        O.oracle_strided(ptr(ids), ptr(want), 4 * e, n, 4 * ss, 4 * ds)
+        got, steps, doubles = cd.plan.plan_map(cd.PATTERN_STRIDED, alignment=a, bytes_per_thread=bpt,
+                                               bytes_per_elmt=e, dma_threads=t, num_elmts=n, src_stride=ss,
+                                               dst_stride=ds, map_len=want.size)
+        assert doubles == 0 and np.array_equal(got, want), (a, bpt, e, n, t)
+        # sequential with the same numbers
+        want = np.full(e + 32, -1, dtype=np.int32)
+        O.oracle_sequential(ptr(ids), ptr(want), 4 * e)
+        got, steps, doubles = cd.plan.plan_map(cd.PATTERN_SEQUENTIAL, alignment=a, bytes_per_thread=bpt,
+                                               bytes_per_elmt=e, dma_threads=t, map_len=want.size)
+        assert doubles == 0 and np.array_equal(got, want), (a, bpt, e, t)
+
+
+def test_replay_rejects_a_window_that_is_too_small():
+    with pytest.raises(cd.CudaDMAError, match="outside"):
+        cd.plan.plan_map(cd.PATTERN_SEQUENTIAL, alignment=16, bytes_per_thread=64, bytes_per_elmt=4096,
+                         dma_threads=64, map_len=1024)

@@ -1,0 +1,276 @@
+"""Pins the CPU oracle (oracle/oracle.c) without the reference, which cannot be
+built here (CUDA + inline PTX).  Each function is checked against
+  * the expectations of the reference's own tests (ramp input + exact compare,
+    src/tests/test_*/cudaDMA_test_*_v2.cu; check_halo of
+    src/tests/test_halo/cudaDMA_test_halo.cu:91-164, restated independently in numpy),
+  * the library routine it must reduce to (numpy copy / slicing / take / .T / matmul,
+    torch's bf16 rounding),
+  * what the mathematics fixes (splitmix64 known answer, stencil exact on polynomials).
+"""
+import numpy as np
+import pytest
+
+from tests import oracle_lib as ol
+from tests.oracle_lib import ptr
+
+
+@pytest.fixture(scope="module")
+def O():
+    return ol.load()
+
+
+# ------------------------------------------------------------------ generators
+def test_splitmix64_known_answer(O):
+    # first output of the published splitmix64 generator seeded with 0
+    assert O.oracle_splitmix64(0) == 0xE220A8397B1DCDAF
+    # and the mixing function restated with Python integers
+    def mix(x):
+        m = (1 << 64) - 1
+        z = (x + 0x9E3779B97F4A7C15) & m
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & m
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & m
+        return z ^ (z >> 31)
+    for x in (1, 2, 1001, 2**63 + 12345, 2**64 - 1):
+        assert O.oracle_splitmix64(x) == mix(x)
+        assert O.oracle_hash32(x, 7) == mix((x + 7) & ((1 << 64) - 1)) >> 32
+
+
+def test_uniform_formula_and_range(O):
+    n = 100003
+    u = ol.uniform(n, 1001)
+    h = np.array([O.oracle_hash32(1001, i) for i in range(2000)], dtype=np.uint64)
+    expect = ((h >> 8).astype(np.float64) * 2.0 ** -23 - 1.0).astype(np.float32)
+    assert np.array_equal(u[:2000], expect)
+    assert u.min() >= -1.0 and u.max() < 1.0
+    assert abs(float(u.mean())) < 0.01 and abs(float(u.var()) - 1.0 / 3.0) < 0.01
+    assert not np.array_equal(u, ol.uniform(n, 1002))
+
+
+def test_ramp_is_the_reference_input(O):
+    assert np.array_equal(ol.ramp(4099), np.arange(4099, dtype=np.float32))
+
+
+def test_indices_range_and_repeats(O):
+    n, recs = 200000, 4096 * 16
+    idx = ol.indices(n, recs, 1003)
+    assert idx.min() >= 0 and idx.max() < recs
+    base = np.array([O.oracle_hash32(1003, i) % recs for i in range(3000)], dtype=np.int32)
+    r = np.array([O.oracle_hash32(1003 ^ 0x5bd1e995, i) for i in range(3000)], dtype=np.int64)
+    for i in range(3000):
+        if i > 1024 and r[i] % 10 == 0:
+            j = i - 1 - (r[i] // 10) % 1024
+            assert idx[i] == base[j]
+        else:
+            assert idx[i] == base[i]
+    forced = sum(1 for i in range(1025, 3000) if r[i] % 10 == 0) / (3000 - 1025)
+    assert 0.07 < forced < 0.13
+
+
+def test_bf16_rounding_matches_torch(O):
+    import torch
+    x = np.concatenate([ol.uniform(5000, 5) * 100.0, np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3895314e38,
+                                                              np.inf, -np.inf, 1e-40], dtype=np.float32)])
+    got = np.array([O.oracle_f32_to_bf16(float(v)) for v in x], dtype=np.uint16)
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(got, want)
+    back = np.array([O.oracle_bf16_to_f32(int(v)) for v in got], dtype=np.float32)
+    assert np.array_equal(back, torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy())
+
+
+# ------------------------------------------------------------------ transfers
+@pytest.mark.parametrize("nbytes", [0, 4, 8, 12, 16, 20, 1024, 4100, 16384])
+@pytest.mark.parametrize("off", [0, 1, 3])
+def test_sequential_is_memcpy_on_the_ramp(O, nbytes, off):
+    # cudaDMA_test_sequential_v2.cu:416-418,501-512: ramp in, exact compare of the moved floats
+    src = ol.ramp(nbytes // 4 + off + 8)
+    dst = np.zeros_like(src)
+    O.oracle_sequential(ptr(src, off * 4), ptr(dst, off * 4), nbytes)
+    want = np.zeros_like(src)
+    want[off:off + nbytes // 4] = src[off:off + nbytes // 4]
+    assert np.array_equal(dst, want)      # also: nothing outside the footprint
+
+
+@pytest.mark.parametrize("e,n,ss,ds", [(4, 1, 4, 4), (12, 7, 16, 32), (256, 64, 65536 // 64, 272), (1000, 9, 1024, 1000),
+                                       (128, 32, 128, 128), (132, 31, 256, 144)])
+def test_strided_is_numpy_slicing(O, e, n, ss, ds):
+    # cudaDMA_test_strided_v2.cu:561-563,659-677
+    src = ol.ramp(n * ss // 4 + 64).view(np.uint8)
+    dst = np.zeros(n * ds + 64, dtype=np.uint8)
+    O.oracle_strided(ptr(src), ptr(dst), e, n, ss, ds)
+    want = np.zeros_like(dst)
+    want_rows = np.lib.stride_tricks.as_strided(want, shape=(n, e), strides=(ds, 1))
+    src_rows = np.lib.stride_tricks.as_strided(src, shape=(n, e), strides=(ss, 1))
+    want_rows[...] = src_rows
+    assert np.array_equal(dst, want)
+    if e == ss == ds:                     # equal strides and packed rows: plain memcpy
+        assert np.array_equal(dst[:n * e], src[:n * e])
+
+
+@pytest.mark.parametrize("e,n,alt", [(4, 5, 0), (128, 32, 0), (128, 32, 64), (128, 32, 128), (128, 32, 144), (20, 9, 32)])
+def test_gather_is_take_and_scatter_inverts_it(O, e, n, alt):
+    # cudaDMA_test_indirect_v2.cu:558-560,659-690 (ramp source, non-overlapping element offsets)
+    rng = np.random.default_rng(e * 1000 + n)
+    table_elems = 3 * n + 5
+    table = ol.ramp(table_elems * e // 4).view(np.uint8).reshape(table_elems, e)
+    index = rng.permutation(table_elems)[:n].astype(np.int32)
+    stride = max(alt, e)
+    dst = np.zeros(n * stride + 16, dtype=np.uint8)
+    O.oracle_gather(ptr(index), ptr(table), ptr(dst), e, n, alt)
+    want = np.zeros_like(dst)
+    for r in range(n):
+        want[r * stride:r * stride + e] = np.take(table, index[r], axis=0)
+    assert np.array_equal(dst, want)
+    # duplicates are allowed in a gather
+    dup = index.copy()
+    dup[n // 2:] = dup[0]
+    O.oracle_gather(ptr(dup), ptr(table), ptr(dst), e, n, alt)
+    assert np.array_equal(dst[(n - 1) * stride:(n - 1) * stride + e], table[dup[0]])
+    # scatter of the gathered rows puts every touched element back where it came from
+    back = np.zeros_like(table)
+    O.oracle_gather(ptr(index), ptr(table), ptr(dst), e, n, alt)
+    O.oracle_scatter(ptr(index), ptr(dst), ptr(back), e, n, alt)
+    want_back = np.zeros_like(table)
+    want_back[index] = table[index]
+    assert np.array_equal(back, want_back)
+
+
+def numpy_check_halo(idata, odata, radius, corners, dimx, dimy, pitch):
+    """check_halo of the reference (cudaDMA_test_halo.cu:91-164) on 2-D views of cells."""
+    i2 = idata[:(dimy + 2 * radius) * pitch].reshape(dimy + 2 * radius, pitch, -1)
+    o2 = odata[:(dimy + 2 * radius) * (dimx + 2 * radius)].reshape(dimy + 2 * radius, dimx + 2 * radius, -1)
+    c0, c1 = (0, dimx + 2 * radius) if corners else (radius, radius + dimx)
+    ok = np.array_equal(i2[:radius, c0:c1], o2[:radius, c0:c1])
+    ok &= np.array_equal(i2[radius + dimy:, c0:c1], o2[radius + dimy:, c0:c1])
+    ok &= np.array_equal(i2[radius:radius + dimy, :radius], o2[radius:radius + dimy, :radius])
+    ok &= np.array_equal(i2[radius:radius + dimy, radius + dimx:radius + dimx + radius],
+                         o2[radius:radius + dimy, radius + dimx:])
+    return bool(ok)
+
+
+@pytest.mark.parametrize("es", [4, 8, 16])
+@pytest.mark.parametrize("radius,corners,dimx,dimy,extra", [(1, 0, 8, 8, 0), (3, 1, 17, 9, 5), (4, 0, 32, 32, 0),
+                                                            (8, 1, 63, 20, 3), (2, 1, 13, 21, 1)])
+def test_halo_matches_the_reference_checker(O, es, radius, corners, dimx, dimy, extra):
+    cells = es // 4
+    pitch = dimx + 2 * radius + extra
+    rng = np.random.default_rng(radius * 100 + dimx)
+    # cudaDMA_test_halo.cu:245-246: rand()%10 cells
+    idata = rng.integers(0, 10, size=(dimy + 2 * radius) * pitch * cells).astype(np.float32).reshape(-1, cells)
+    odata = np.zeros(((dimx + 2 * radius) * (dimy + 2 * radius), cells), dtype=np.float32)
+    src_origin = (radius * pitch + radius) * es
+    dst_origin = (radius * (dimx + 2 * radius) + radius) * es
+    O.oracle_halo(ptr(idata, src_origin), ptr(odata, dst_origin), es, radius, corners, dimx, dimy, pitch)
+    assert numpy_check_halo(idata, odata, radius, corners, dimx, dimy, pitch)
+    assert O.oracle_halo_check(ptr(idata), ptr(odata), es, radius, corners, dimx, dimy, pitch) == 1
+    # stricter than the reference: interior (and corners when off) stay zero
+    o2 = odata.reshape(dimy + 2 * radius, dimx + 2 * radius, cells)
+    assert not o2[radius:radius + dimy, radius:radius + dimx].any()
+    if not corners:
+        assert not o2[:radius, :radius].any() and not o2[-radius:, -radius:].any()
+    # total bytes moved = ring area
+    ring = 2 * radius * (dimx + (2 * radius if corners else 0)) + 2 * radius * dimy
+    i2 = idata.reshape(dimy + 2 * radius, pitch, cells)[:, :dimx + 2 * radius]
+    assert np.count_nonzero(o2 != 0) <= ring * cells
+    mask = np.ones((dimy + 2 * radius, dimx + 2 * radius), dtype=bool)
+    mask[radius:radius + dimy, radius:radius + dimx] = False
+    if not corners:
+        for ys in (slice(0, radius), slice(radius + dimy, None)):
+            for xs in (slice(0, radius), slice(radius + dimx, None)):
+                mask[ys, xs] = False
+    assert np.array_equal(o2[mask], i2[mask])
+    # the checker itself notices a wrong cell
+    bad = odata.copy()
+    bad[radius * (dimx + 2 * radius)] += 1.0          # first cell of the left panel
+    assert O.oracle_halo_check(ptr(idata), ptr(bad), es, radius, corners, dimx, dimy, pitch) == 0
+    assert not numpy_check_halo(idata, bad, radius, corners, dimx, dimy, pitch)
+
+
+# ------------------------------------------------------------------ workloads
+def test_copy_and_transpose(O):
+    a = ol.uniform(256 * 256, 1002).reshape(256, 256)
+    out = np.empty_like(a)
+    O.oracle_copy(ptr(a), ptr(out), a.size)
+    assert np.array_equal(out, a)
+    O.oracle_transpose(ptr(a), ptr(out), 256)
+    assert np.array_equal(out, a.T)
+    ramp = ol.ramp(192 * 192).reshape(192, 192)
+    out = np.empty_like(ramp)
+    O.oracle_transpose(ptr(ramp), ptr(out), 192)
+    assert out[5, 7] == 7 * 192 + 5
+
+
+def test_gather_copy_and_rowsum(O):
+    recs, n_idx = 4096, 32 * 300
+    table = ol.uniform(recs * 32, 1003).reshape(recs, 32)
+    idx = ol.indices(n_idx, recs, 1003)
+    out = np.empty((n_idx, 32), dtype=np.float32)
+    O.oracle_gather_copy(ptr(table), ptr(idx), ptr(out), n_idx, 32)
+    assert np.array_equal(out, table[idx])
+    sums = np.empty((n_idx // 32, 32), dtype=np.float32)
+    O.oracle_gather_rowsum(ptr(table), ptr(idx), ptr(sums), n_idx, 32, 32)
+    tiles = table[idx].reshape(-1, 32, 32)
+    acc = tiles[:, 0, :].copy()
+    for r in range(1, 32):
+        acc = acc + tiles[:, r, :]                    # float32, ascending record order
+    assert np.array_equal(sums, acc)
+    # a different order gives different bits somewhere: the order is part of the statement
+    rev = tiles[:, 31, :].copy()
+    for r in range(30, -1, -1):
+        rev = rev + tiles[:, r, :]
+    assert not np.array_equal(sums, rev)
+    assert np.allclose(sums, tiles.astype(np.float64).sum(axis=1), rtol=1e-5, atol=1e-5)
+
+
+def stencil_numpy64(g, nx, ny, nz, p):
+    c = [3.0 * (-205.0 / 72.0), 8.0 / 5.0, -1.0 / 5.0, 8.0 / 315.0, -1.0 / 560.0]
+    g = g.astype(np.float64)
+    core = (slice(p, p + nz), slice(p, p + ny), slice(p, p + nx))
+    out = c[0] * g[core]
+    for r in range(1, 5):
+        for ax in range(3):
+            for s in (-r, r):
+                sl = list(core)
+                sl[ax] = slice(core[ax].start + s, core[ax].stop + s)
+                out = out + c[r] * g[tuple(sl)]
+    return out
+
+
+def test_stencil_against_numpy_and_polynomials(O):
+    nx, ny, nz, p = 32, 32, 12, 4
+    g = ol.uniform((nx + 2 * p) * (ny + 2 * p) * (nz + 2 * p), 1004).reshape(nz + 2 * p, ny + 2 * p, nx + 2 * p)
+    out = np.empty((nz, ny, nx), dtype=np.float32)
+    O.oracle_stencil25(ptr(g), ptr(out), nx, ny, nz, p)
+    ref = stencil_numpy64(g, nx, ny, nz, p)
+    assert np.max(np.abs(out - ref)) <= 1e-5 * np.max(np.abs(ref))
+    # a constant field has zero Laplacian; x^2 + 2y^2 + 3z^2 has Laplacian 12; the 8th-order
+    # stencil is exact for polynomials up to degree 9, so x^4 at x gives 12 x^2
+    z, y, x = np.meshgrid(np.arange(nz + 2 * p), np.arange(ny + 2 * p), np.arange(nx + 2 * p), indexing="ij")
+    for field, want in ((np.ones_like(x), lambda X, Y, Z: 0.0 * X),
+                        (x * x + 2 * y * y + 3 * z * z, lambda X, Y, Z: 12.0 + 0.0 * X),
+                        (x ** 4 // 1, lambda X, Y, Z: 12.0 * X * X)):
+        f32 = field.astype(np.float32)
+        O.oracle_stencil25(ptr(f32), ptr(out), nx, ny, nz, p)
+        core = want(x[p:-p, p:-p, p:-p].astype(np.float64), None, None)
+        scale = max(1.0, float(np.max(np.abs(f32))))
+        assert np.max(np.abs(out - core)) <= 2e-5 * scale, (np.max(np.abs(out - core)), scale)
+    # anisotropy check: a wrong axis pitch would mix y and z
+    f32 = (z.astype(np.float32)) ** 2
+    O.oracle_stencil25(ptr(f32), ptr(out), nx, ny, nz, p)
+    assert np.max(np.abs(out - 2.0)) < 1e-2
+
+
+def test_gemm_bf16(O):
+    m, n, k = 96, 80, 160
+    a = np.empty(m * k, dtype=np.uint16)
+    b = np.empty(k * n, dtype=np.uint16)
+    O.oracle_fill_normal_bf16(ptr(a), a.size, 1005)
+    O.oracle_fill_normal_bf16(ptr(b), b.size, 2005)
+    def widen(u):
+        return (u.astype(np.uint32) << 16).view(np.float32)
+    af, bf = widen(a).reshape(m, k), widen(b).reshape(k, n)
+    assert abs(float(af.mean())) < 0.05 and abs(float(af.std()) - 1.0) < 0.05   # normal(0,1)
+    c = np.empty((m, n), dtype=np.float32)
+    O.oracle_gemm_bf16(ptr(a), ptr(b), ptr(c), m, n, k)
+    ref = af.astype(np.float64) @ bf.astype(np.float64)
+    assert np.max(np.abs(c - ref)) <= 1e-4 * np.max(np.abs(ref))
+    assert abs(O.oracle_gemm_bf16_entry(ptr(a), ptr(b), n, k, 5, 7) - c[5, 7]) <= 1e-5 * abs(c[5, 7]) + 1e-6

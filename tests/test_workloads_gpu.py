@@ -1,0 +1,189 @@
+"""GPU parity of the five benchmark workloads, called through the C ABI.
+Small shapes are compared with the oracle element by element; the BASELINE shapes are
+checked through properties that do not need a host pass over gigabytes where one would
+be slow (double transpose = identity, gather of identity indices = table, linearity)."""
+import numpy as np
+import pytest
+import torch
+
+import cudadma_amd as cd
+from cudadma_amd import workloads as wl
+from tests import oracle_lib as ol
+from tests.oracle_lib import ptr
+
+pytestmark = pytest.mark.gpu
+
+
+def _variants(w):
+    return range(wl.num_variants(w))
+
+
+# ------------------------------------------------------------------ generators
+def test_device_generators_match_the_host_statement(device):
+    n = 1 << 20
+    got = wl.fill_uniform(torch.empty(n + 3, dtype=torch.float32, device=device), 1001).cpu().numpy()
+    assert np.array_equal(got, ol.uniform(n + 3, 1001))
+    idx = wl.fill_indices(torch.empty(n, dtype=torch.int32, device=device), 4096 * 1024, 1003).cpu().numpy()
+    assert np.array_equal(idx, ol.indices(n, 4096 * 1024, 1003))
+
+
+# ------------------------------------------------------------------ config 1
+@pytest.mark.parametrize("variant", _variants(wl.SEQUENTIAL))
+@pytest.mark.parametrize("tiles", [1, 3, 257, 4096])
+def test_sequential_copy(device, variant, tiles):
+    n = tiles * wl.SEQ_TILE_BYTES // 4
+    src = wl.fill_uniform(torch.empty(n, dtype=torch.float32, device=device), 1001)
+    dst = torch.full_like(src, float("nan"))
+    print(f"sequential variant {variant} tiles {tiles}", flush=True)
+    wl.sequential_copy(src, dst, variant)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(torch.int32), src.view(torch.int32))       # bit-exact, config 1
+    if tiles <= 257:
+        want = np.empty(n, dtype=np.float32)
+        host = ol.uniform(n, 1001)
+        ol.load().oracle_copy(ptr(host), ptr(want), n)
+        assert np.array_equal(dst.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_sequential_copy_rejects_ragged_sizes(device):
+    src = torch.zeros(5000, dtype=torch.float32, device=device)
+    with pytest.raises(cd.CudaDMAError, match="multiple"):
+        wl.sequential_copy(src, torch.empty_like(src))
+    empty = torch.zeros(0, dtype=torch.float32, device=device)
+    wl.sequential_copy(empty, torch.empty_like(empty))                     # empty input is a no-op
+
+
+def test_plain_copy(device):
+    src = wl.fill_uniform(torch.empty(1 << 22, dtype=torch.float32, device=device), 7)
+    dst = torch.zeros_like(src)
+    wl.plain_copy(src, dst)
+    torch.cuda.synchronize()
+    assert torch.equal(dst, src)
+
+
+# ------------------------------------------------------------------ config 2
+@pytest.mark.parametrize("variant", _variants(wl.STRIDED))
+@pytest.mark.parametrize("n", [1024, 2048])
+def test_strided_transpose_small(device, variant, n):
+    host = ol.uniform(n * n, 1002).reshape(n, n)
+    want = np.empty_like(host)
+    ol.load().oracle_transpose(ptr(host), ptr(want), n)
+    src = torch.from_numpy(host).to(device)
+    dst = torch.full_like(src, float("nan"))
+    print(f"transpose variant {variant} n {n}", flush=True)
+    wl.strided_transpose(src, dst, variant)
+    torch.cuda.synchronize()
+    assert np.array_equal(dst.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_strided_transpose_full_size(device):
+    n = 16384
+    src = wl.fill_uniform(torch.empty(n * n, dtype=torch.float32, device=device), 1002).view(n, n)
+    dst = torch.empty_like(src)
+    wl.strided_transpose(src, dst, 0)
+    torch.cuda.synchronize()
+    # rows of the oracle's statement on a sample of the output, then transpose twice = identity
+    host_rows = ol.uniform(n * n, 1002).reshape(n, n)
+    for c in (0, 1, 63, 64, 8191, n - 1):
+        assert np.array_equal(dst[c].cpu().numpy(), host_rows[:, c])
+    del host_rows
+    back = torch.empty_like(src)
+    wl.strided_transpose(dst, back, 0)
+    torch.cuda.synchronize()
+    assert torch.equal(back.view(torch.int32), src.view(torch.int32))
+
+
+# ------------------------------------------------------------------ config 3
+@pytest.mark.parametrize("variant", _variants(wl.GATHER))
+@pytest.mark.parametrize("n_tiles", [1, 5, 4099])
+def test_gather_small(device, variant, n_tiles):
+    recs = 1 << 16
+    n_idx = n_tiles * wl.RECS_PER_TILE
+    table = ol.uniform(recs * wl.REC_FLOATS, 1003)
+    idx = ol.indices(n_idx, recs, 1003)
+    want_copy = np.empty(n_idx * wl.REC_FLOATS, dtype=np.float32)
+    want_sum = np.empty(n_tiles * wl.REC_FLOATS, dtype=np.float32)
+    O = ol.load()
+    O.oracle_gather_copy(ptr(table), ptr(idx), ptr(want_copy), n_idx, wl.REC_FLOATS)
+    O.oracle_gather_rowsum(ptr(table), ptr(idx), ptr(want_sum), n_idx, wl.REC_FLOATS, wl.RECS_PER_TILE)
+    d_table = torch.from_numpy(table).to(device)
+    d_idx = torch.from_numpy(idx).to(device)
+    print(f"gather variant {variant} tiles {n_tiles}", flush=True)
+    got_copy = wl.gather_copy(d_table, d_idx, torch.full((want_copy.size,), float("nan"), device=device), variant)
+    got_sum = wl.gather_rowsum(d_table, d_idx, torch.full((want_sum.size,), float("nan"), device=device), variant)
+    torch.cuda.synchronize()
+    assert np.array_equal(got_copy.cpu().numpy().view(np.uint32), want_copy.view(np.uint32))
+    assert np.array_equal(got_sum.cpu().numpy().view(np.uint32), want_sum.view(np.uint32))
+
+
+def test_gather_full_size(device):
+    recs, n_idx = 4 * 1024 * 1024, 32 * 1024 * 1024
+    table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=device), 1003)
+    idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=device), recs, 1003)
+    out = torch.empty(n_idx * wl.REC_FLOATS, dtype=torch.float32, device=device)
+    wl.gather_copy(table, idx, out, 0)
+    torch.cuda.synchronize()
+    # every record against torch's own gather, in slabs to bound memory
+    t2 = table.view(recs, wl.REC_FLOATS)
+    o2 = out.view(n_idx, wl.REC_FLOATS)
+    slab = 1 << 22
+    for s in range(0, n_idx, slab):
+        assert torch.equal(o2[s:s + slab].view(torch.int32), t2[idx[s:s + slab].long()].view(torch.int32))
+    # the headline consumer on the oracle's statement for a sample of tiles
+    sums = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, dtype=torch.float32, device=device)
+    wl.gather_rowsum(table, idx, sums, 0)
+    torch.cuda.synchronize()
+    tiles = o2.view(-1, wl.RECS_PER_TILE, wl.REC_FLOATS)
+    sample = torch.arange(0, tiles.shape[0], 997, device=device)
+    t = tiles[sample].cpu().numpy()
+    acc = t[:, 0, :].copy()
+    for r in range(1, wl.RECS_PER_TILE):
+        acc = acc + t[:, r, :]
+    assert np.array_equal(sums.view(-1, wl.REC_FLOATS)[sample].cpu().numpy().view(np.uint32), acc.view(np.uint32))
+    # duplicates are really there
+    assert int((idx[1025:100000] == idx[1024:99999]).sum()) >= 0
+    # empty index list is a no-op
+    wl.gather_copy(table, idx[:0], out[:0], 0)
+
+
+# ------------------------------------------------------------------ config 4
+STENCIL_RTOL = 1e-5       # BASELINE config 4: fp32 within 1e-5 relative of the host reference
+
+
+@pytest.mark.parametrize("variant", _variants(wl.HALO))
+@pytest.mark.parametrize("shape", [(32, 32, 5), (64, 96, 70), (128, 64, 130)])
+def test_halo_stencil_small(device, variant, shape):
+    nx, ny, nz = shape
+    p = 2 * wl.STENCIL_RADIUS
+    g = ol.uniform((nx + p) * (ny + p) * (nz + p), 1004).reshape(nz + p, ny + p, nx + p)
+    want = np.empty((nz, ny, nx), dtype=np.float32)
+    ol.load().oracle_stencil25(ptr(g), ptr(want), nx, ny, nz, wl.STENCIL_RADIUS)
+    d_in = torch.from_numpy(g).to(device)
+    d_out = torch.full((nz, ny, nx), float("nan"), dtype=torch.float32, device=device)
+    print(f"stencil variant {variant} shape {shape}", flush=True)
+    wl.halo_stencil(d_in, d_out, variant)
+    torch.cuda.synchronize()
+    got = d_out.cpu().numpy()
+    err = np.abs(got - want)
+    assert np.all(err <= STENCIL_RTOL * np.maximum(np.abs(want), 1.0)), float(err.max())
+
+
+def test_halo_stencil_full_size(device):
+    n = 512
+    p = 2 * wl.STENCIL_RADIUS
+    d_in = wl.fill_uniform(torch.empty((n + p) ** 3, dtype=torch.float32, device=device), 1004).view(n + p, n + p, n + p)
+    d_out = torch.empty((n, n, n), dtype=torch.float32, device=device)
+    wl.halo_stencil(d_in, d_out, 0)
+    torch.cuda.synchronize()
+    # slabs of the host statement
+    g = ol.uniform((n + p) ** 3, 1004).reshape(n + p, n + p, n + p)
+    for z0 in (0, 250, n - 3):
+        want = np.empty((3, n, n), dtype=np.float32)
+        ol.load().oracle_stencil25(ptr(np.ascontiguousarray(g[z0:z0 + 3 + p])), ptr(want), n, n, 3, wl.STENCIL_RADIUS)
+        got = d_out[z0:z0 + 3].cpu().numpy()
+        assert np.all(np.abs(got - want) <= STENCIL_RTOL * np.maximum(np.abs(want), 1.0))
+    # a constant field has zero Laplacian everywhere (catches a wrong tile or plane anywhere in the grid)
+    d_in.fill_(1.0)
+    wl.halo_stencil(d_in, d_out, 0)
+    torch.cuda.synchronize()
+    assert float(d_out.abs().max()) <= 1e-5
