@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Benchmark of the hipDMA transfer patterns on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one launch of the CudaDMAStrided tile-transpose kernel over the whole
+16384 x 16384 float32 matrix (BASELINE config 2, the configuration the metric is
+quoted on); inputs are resident in HBM before the timed region.  The other three
+HBM-bound patterns (sequential copy, indirect gather, halo stencil) and a plain
+copy kernel are timed the same way and reported under "patterns".  One JSON line
+goes to stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0           # MI355X published HBM3E bandwidth
+
+# HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
+# scaled by what the same counters read for the plain copy kernel (see profiles/).
+# None until such a profile has been taken for the current kernel.
+MEASURED_TRAFFIC_BYTES = {"strided": None}
+
+
+def log(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def time_launches(fn, steps, warmup):
+    """Average milliseconds per launch, HIP events on the launch stream around `steps` launches."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return start.elapsed_time(stop) / steps, wall_ms / steps
+
+
+def cpu_baseline_transpose(budget_s=20.0):
+    """The oracle's OpenMP transpose on this machine's host cores, on an 8192 x 8192 sample
+    (a quarter of the matrix: 512 MiB of traffic per repetition)."""
+    import numpy as np
+    from tests import oracle_lib as ol
+    from tests.oracle_lib import ptr
+    O = ol.load()
+    n = 8192
+    a = ol.uniform(n * n, 1002).reshape(n, n)      # parallel first touch
+    out = np.empty_like(a)
+    O.oracle_transpose(ptr(a), ptr(out), n)          # warm-up + first touch of the output
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 5 or (len(times) < 15 and time.perf_counter() - t_all < budget_s):
+        t0 = time.perf_counter()
+        O.oracle_transpose(ptr(a), ptr(out), n)
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_all > budget_s:
+            break
+    med = sorted(times)[len(times) // 2]
+    return {
+        "value": round(2.0 * n * n * 4 / med / 1e9, 2),
+        "unit": "GB/s",
+        "cores": O.oracle_num_threads(),
+        "kind": "port",
+        "sample": f"oracle_transpose (OpenMP, blocked 64x64) of an {n}x{n} float32 sample, "
+                  f"median of {len(times)} repetitions",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-core baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (the DMA objects live inside one kernel on one "
+                 "device; there is no multi-GPU path to time). Use --gpus 1.")
+
+    import torch
+    import cudadma_amd as cd
+    from cudadma_amd import workloads as wl
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the hipDMA kernels have no CPU path")
+    dev = torch.device("cuda:0")
+    cd.lib()
+    steps, warmup = args.steps, args.warmup
+    patterns = {}
+
+    def report(name, ms, nbytes, note):
+        gbs = nbytes / ms / 1e6
+        patterns[name] = {"GB/s": round(gbs, 1), "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4),
+                          "ms": round(ms, 4), "algorithmic_bytes": nbytes, "workload": note}
+        log(f"{name:12s} {ms:9.4f} ms  {gbs:8.1f} GB/s  {100 * gbs / HBM_PEAK_GBS:5.1f}% of peak   {note}")
+
+    # ---- config 2: strided tile transpose (headline) ----
+    n = 16384
+    src = wl.fill_uniform(torch.empty(n * n, dtype=torch.float32, device=dev), 1002).view(n, n)
+    dst = torch.empty_like(src)
+    strided_ms, strided_wall_ms = time_launches(lambda: wl.strided_transpose(src, dst, 0), steps, warmup)
+    strided_bytes = 2 * n * n * 4
+    report("strided", strided_ms, strided_bytes, "CudaDMAStrided 64x256B tiles of a 16384^2 f32 matrix, transposed out")
+    # yardstick on the same buffers: plain dwordx4 copy
+    copy_ms, _ = time_launches(lambda: wl.plain_copy(src, dst), steps, warmup)
+    report("plain_copy", copy_ms, strided_bytes, "grid-stride dwordx4 copy of 1 GiB, no LDS, no DMA object")
+    del src, dst
+
+    # ---- config 1: sequential copy, 64 MiB in 16 KiB tiles ----
+    m = 64 * 1024 * 1024 // 4
+    s_src = wl.fill_uniform(torch.empty(m, dtype=torch.float32, device=dev), 1001)
+    s_dst = torch.empty_like(s_src)
+    ms, _ = time_launches(lambda: wl.sequential_copy(s_src, s_dst, 0), max(steps, 50), warmup)
+    report("sequential", ms, 2 * m * 4, "CudaDMASequential 16 KiB tiles of a 64 MiB f32 buffer (fits the 256 MB Infinity Cache)")
+    del s_src, s_dst
+
+    # ---- config 3: indirect gather, row-sum consumer ----
+    recs, n_idx = 4 * 1024 * 1024, 32 * 1024 * 1024
+    table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev), 1003)
+    idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=dev), recs, 1003)
+    sums = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, dtype=torch.float32, device=dev)
+    ms, _ = time_launches(lambda: wl.gather_rowsum(table, idx, sums, 0), steps, warmup)
+    report("gather", ms, n_idx * 4 + n_idx * 128 + sums.numel() * 4,
+           "CudaDMAIndirect 32 x 128 B records per tile from a 512 MiB table, row-sum consumer")
+    del table, idx, sums
+
+    # ---- config 4: halo stencil ----
+    g = 512
+    p = 2 * wl.STENCIL_RADIUS
+    grid_in = wl.fill_uniform(torch.empty((g + p) ** 3, dtype=torch.float32, device=dev), 1004).view(g + p, g + p, g + p)
+    grid_out = torch.empty((g, g, g), dtype=torch.float32, device=dev)
+    ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 0), steps, warmup)
+    report("halo", ms, 2 * g ** 3 * 4, "CudaDMAHalo radius-4 ring of 32x32 tiles, 25-point stencil on a 512^3 f32 grid")
+    del grid_in, grid_out
+
+    value = patterns["strided"]["GB/s"]
+    result = {
+        "metric": "achieved HBM GB/s (% of MI355X peak) per DMA pattern: seq/strided/gather/halo",
+        "value": value,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(strided_wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "CudaDMAStrided 2D tile extraction: 16384x16384 f32, 64 rows x 256 B tiles, "
+                               "double-buffered, transposed to output (BASELINE configs[1])",
+                   "tile_rows": 64, "tile_row_bytes": 256, "src_stride_bytes": 65536,
+                   "workgroup": "128 DMA + 128 compute threads"},
+        "roofline": {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(value / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES["strided"],
+                     "kernel": "transpose_manual_double<272>", "kernel_ms": round(strided_ms, 4),
+                     "algorithmic_bytes_per_launch": strided_bytes},
+        "patterns": patterns,
+    }
+    if not args.no_cpu_baseline:
+        log("timing the host-core baseline (oracle transpose) ...")
+        result["cpu_baseline"] = cpu_baseline_transpose()
+        log(f"cpu baseline: {result['cpu_baseline']}")
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
