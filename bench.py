@@ -144,7 +144,10 @@ def main():
     grid_in = wl.fill_uniform(torch.empty((g + p) ** 3, dtype=torch.float32, device=dev), 1004).view(g + p, g + p, g + p)
     grid_out = torch.empty((g, g, g), dtype=torch.float32, device=dev)
     ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 0), steps, warmup)
-    report("halo", ms, 2 * g ** 3 * 4, "CudaDMAHalo radius-4 ring of 32x32 tiles, 25-point stencil on a 512^3 f32 grid")
+    report("halo", ms, 2 * g ** 3 * 4, "CudaDMAHalo radius-4 ring of 32x32 tiles, 25-point stencil on a 512^3 f32 grid "
+           "(empty/full handshake + one s_barrier per plane)")
+    ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 2), steps, warmup)
+    report("halo_barrier_only", ms, 2 * g ** 3 * 4, "same kernel with execute_dma_no_sync: ordered by the per-plane s_barrier alone")
     del grid_in, grid_out
 
     value = patterns["strided"]["GB/s"]

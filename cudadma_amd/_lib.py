@@ -84,6 +84,8 @@ def lib():
                                    ctypes.POINTER(ci)]
     L.cudadma_diagnose.restype = ci
     L.cudadma_diagnose.argtypes = [ci] * 8
+    L.cudadma_set_tuning.restype = ci
+    L.cudadma_set_tuning.argtypes = [ctypes.c_char_p, ci]
     L.cudadma_variant_name.restype = ctypes.c_char_p
     L.cudadma_variant_name.argtypes = [ci, ci]
     _lib = L
@@ -115,4 +117,4 @@ def check(rc):
 def exported_symbols():
     """Every extern "C" symbol include/cudadma_amd.h declares."""
     return ["cudadma_last_error", "cudadma_device_cus", "cudadma_num_cases", "cudadma_get_case",
-            "cudadma_run_case", "cudadma_variant_name", "cudadma_plan_map", "cudadma_diagnose"] + list(_WORKLOAD_SIGNATURES)
+            "cudadma_run_case", "cudadma_variant_name", "cudadma_plan_map", "cudadma_diagnose", "cudadma_set_tuning"] + list(_WORKLOAD_SIGNATURES)

@@ -1,6 +1,7 @@
 // Variant tables, the occupancy knob and grid sizing shared by the workloads.
 #include "workloads.hpp"
 #include <atomic>
+#include <cstring>
 
 namespace workloads {
 
@@ -16,6 +17,26 @@ int persistent_grid(long long work_items, int default_wg_per_cu)
   const int knob = g_wg_per_cu.load();
   const long long want = (long long)g_cus * (knob > 0 ? knob : default_wg_per_cu);
   return (int)(work_items < want ? work_items : want);
+}
+
+struct Knob {
+  const char* name;
+  std::atomic<int> value;
+};
+static Knob g_knobs[] = {{"transpose_band", {0}}, {"stencil_zchunk", {0}}, {"stencil_xcd_remap", {0}}};
+
+static Knob* find_knob(const char* name)
+{
+  for (Knob& k : g_knobs)
+    if (name != nullptr && std::strcmp(k.name, name) == 0) return &k;
+  return nullptr;
+}
+
+int tuning(const char* name, int fallback)
+{
+  Knob* k = find_knob(name);
+  const int v = k != nullptr ? k->value.load() : 0;
+  return v > 0 ? v : fallback;
 }
 
 static const VariantInfo kSequential[] = {
@@ -36,8 +57,14 @@ static const VariantInfo kGather[] = {
   {"manual double buffer: two objects"},
 };
 static const VariantInfo kHalo[] = {
-  {"warp-specialised: CudaDMAHalo ring by 1 DMA wavefront, interior by the 4 compute wavefronts, double-buffered planes"},
-  {"not warp-specialised: all wavefronts move the ring, workgroup barriers"},
+  {"warp-specialised, 4 cells per thread as one dwordx4: CudaDMAHalo ring by 1 DMA wavefront with the empty/full "
+   "handshake, one s_barrier per plane for the interior exchange"},
+  {"as variant 0 but the compute wavefronts meet in an LDS-counter GroupBarrier and the DMA wavefront runs free"},
+  {"as variant 0 without the handshake: execute_dma_no_sync, ordered by the per-plane s_barrier alone"},
+  {"not warp-specialised, dwordx4 cells: every thread computes, half of them also carry a ring chunk requested one "
+   "plane ahead; one LDS plane, two s_barriers per plane"},
+  {"warp-specialised, one cell per dword load (first version kept for comparison)"},
+  {"not warp-specialised, one cell per dword load"},
 };
 
 static const VariantInfo* table(int workload, int* count)
@@ -65,6 +92,16 @@ extern "C" const char* cudadma_variant_name(int workload, int variant)
   int n = 0;
   const workloads::VariantInfo* t = workloads::table(workload, &n);
   return (t != nullptr && variant >= 0 && variant < n) ? t[variant].name : "";
+}
+
+extern "C" int cudadma_set_tuning(const char* name, int value)
+{
+  workloads::Knob* k = workloads::find_knob(name);
+  if (k == nullptr) {
+    cudadma_host::set_error("unknown tuning knob '%s'", name != nullptr ? name : "(null)");
+    return CUDADMA_EINVAL;
+  }
+  return k->value.exchange(value < 0 ? 0 : value);
 }
 
 extern "C" int cudadma_set_workgroups_per_cu(int value)

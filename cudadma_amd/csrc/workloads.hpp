@@ -11,6 +11,9 @@ namespace workloads {
 // default), never more than there are work items.
 int persistent_grid(long long work_items, int default_wg_per_cu);
 
+// Value of a named knob, or `fallback` while it is unset (0).
+int tuning(const char* name, int fallback);
+
 struct VariantInfo {
   const char* name;
 };

@@ -32,7 +32,7 @@ struct Coeffs {
   float c0, c1, c2, c3, c4;
 };
 
-// One cell: same operations in the same order as the host statement, no fused multiply-add.
+// One cell: same operations in the same order as the host statement.
 __device__ __forceinline__ float stencil_cell(const float* __restrict__ plane, const int lx, const int ly,
                                               const float (&q)[2 * kR + 1], const Coeffs& k)
 {
@@ -45,7 +45,7 @@ __device__ __forceinline__ float stencil_cell(const float* __restrict__ plane, c
     const float sx = c[-r] + c[r];
     const float sy = c[-r * kPitch] + c[r * kPitch];
     const float sz = q[kR - r] + q[kR + r];
-    acc += cr[r] * ((sx + sy) + sz);
+    acc = __builtin_fmaf(cr[r], (sx + sy) + sz, acc);
   }
   return acc;
 }
@@ -56,11 +56,21 @@ struct TileWork {
   int planes;               // output planes in this chunk
 };
 
+// `zchunk` carries the chunk length in its low 24 bits; bit 24 asks for the
+// XCD-aware numbering: workgroup b runs on XCD b % 8 (8 XCDs, round-robin
+// dispatch), so giving XCD k the k-th eighth of the tile list keeps tiles that
+// share ghost cells behind the same L2.
+constexpr int kXcdFlag = 1 << 24;
+constexpr int kXcds = 8;
+
 __device__ __forceinline__ TileWork tile_work(const float* in, float* out, const int nx, const int ny, const int nz,
-                                              const int zchunk)
+                                              const int zchunk_and_flags)
 {
+  const int zchunk = zchunk_and_flags & (kXcdFlag - 1);
   const int tiles_x = nx / kTX, tiles_y = ny / kTY;
   int b = blockIdx.x;
+  if ((zchunk_and_flags & kXcdFlag) && (gridDim.x % kXcds) == 0)
+    b = (b % kXcds) * (gridDim.x / kXcds) + b / kXcds;
   const int tx = b % tiles_x; b /= tiles_x;
   const int ty = b % tiles_y; b /= tiles_y;
   const int z0 = b * zchunk;
@@ -186,6 +196,256 @@ stencil_not_specialized(const float* __restrict__ in, float* __restrict__ out, c
   }
 }
 
+// ---------------------------------------------------------------------------
+// dwordx4 version: a compute thread owns four consecutive cells of one tile row
+// and moves them as one 16-byte access everywhere (global load of the newest
+// plane, LDS write of the centre plane, LDS reads of the x/y neighbours, global
+// store of the result).  PREFETCH planes beyond the nine of the stencil are
+// kept in flight per thread so that a workgroup has (1 + PREFETCH) x 4 KiB of
+// loads outstanding.
+// ---------------------------------------------------------------------------
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kXQ = kTX / 4;                          // 8 threads per tile row
+constexpr int kPrefetch = 3;
+constexpr int kQueue = 2 * kR + 1 + kPrefetch;        // planes held in registers: 12
+// The z column is a ring of registers: plane z + p of the chunk sits in slot
+// (z + p) % kQueue, and the z loop is unrolled kQueue times so that every slot
+// number is a compile-time constant and no plane is ever moved between registers.
+#define HIPDMA_QSLOT(ROT, P) (((ROT) + (P)) % kQueue)
+
+enum SyncMode {
+  kHandshakeAndBarrier = 0,   // empty/full handshake + one s_barrier per plane (DMA wavefront joins it)
+  kHandshakeAndGroupBarrier,  // empty/full handshake + LDS-counter barrier of the compute wavefronts
+  kBarrierOnly,               // execute_dma_no_sync + one s_barrier per plane
+};
+
+// Four cells of row ly starting at column lx; plane p of the z column is q[HIPDMA_QSLOT(ROT, p)].
+// Same operations in the same order as the host statement: one multiply, then per
+// radius five additions and one fused multiply-add.
+template<int ROT>
+__device__ __forceinline__ f32x4_t stencil_cells4(const float* __restrict__ plane, const int lx, const int ly,
+                                                  const f32x4_t (&q)[kQueue], const Coeffs& k)
+{
+#pragma clang fp contract(off)
+  const float* c = plane + (ly + kR) * kPitch + (lx + kR);
+  const float cr[5] = {0.0f, k.c1, k.c2, k.c3, k.c4};
+  // x neighbourhood: 4 cells left, the centre cells, 4 cells right
+  const f32x4_t xl = *(const f32x4_t*)(c - 4);
+  const f32x4_t xc = q[HIPDMA_QSLOT(ROT, kR)];
+  const f32x4_t xr = *(const f32x4_t*)(c + 4);
+  const float xs[12] = {xl[0], xl[1], xl[2], xl[3], xc[0], xc[1], xc[2], xc[3], xr[0], xr[1], xr[2], xr[3]};
+  f32x4_t up[kR], dn[kR];
+#pragma unroll
+  for (int r = 1; r <= kR; ++r) {
+    up[r - 1] = *(const f32x4_t*)(c - r * kPitch);
+    dn[r - 1] = *(const f32x4_t*)(c + r * kPitch);
+  }
+  f32x4_t out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float acc = k.c0 * xc[i];
+#pragma unroll
+    for (int r = 1; r <= kR; ++r) {
+      const float sx = xs[4 + i - r] + xs[4 + i + r];
+      const float sy = up[r - 1][i] + dn[r - 1][i];
+      const float sz = q[HIPDMA_QSLOT(ROT, kR - r)][i] + q[HIPDMA_QSLOT(ROT, kR + r)][i];
+      acc = __builtin_fmaf(cr[r], (sx + sy) + sz, acc);
+    }
+    out[i] = acc;
+  }
+  return out;
+}
+
+// Runs the body for z = 0 .. planes-1 with ROT = z % kQueue as a constant.  Whole
+// groups of kQueue planes run without a single branch, so the compiler's
+// s_waitcnt placement can count exactly how many younger loads and stores may
+// stay in flight; only the last, partial group checks the plane count.
+#define HIPDMA_Z_STEP(J, CHECK, ...) if (!(CHECK) || z0 + (J) < planes) { constexpr int ROT = (J); const int z = z0 + (J); __VA_ARGS__ }
+#define HIPDMA_Z_GROUP(CHECK, ...)                                                                       \
+  HIPDMA_Z_STEP(0, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(1, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(2, CHECK, __VA_ARGS__)   \
+  HIPDMA_Z_STEP(3, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(4, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(5, CHECK, __VA_ARGS__)   \
+  HIPDMA_Z_STEP(6, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(7, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(8, CHECK, __VA_ARGS__)   \
+  HIPDMA_Z_STEP(9, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(10, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(11, CHECK, __VA_ARGS__)
+#define HIPDMA_FOR_Z(planes_expr, ...)                                       \
+  {                                                                          \
+    const int planes = (planes_expr);                                        \
+    int z0 = 0;                                                              \
+    for (; z0 + kQueue <= planes; z0 += kQueue) { HIPDMA_Z_GROUP(false, __VA_ARGS__) } \
+    if (z0 < planes) { HIPDMA_Z_GROUP(true, __VA_ARGS__) }                   \
+  }
+static_assert(kQueue == 12 && kQueue % 4 == 0, "HIPDMA_FOR_Z unrolls twelve steps; the LDS planes rotate with period 4");
+
+// The DMA wavefront keeps the rings of the next kRingAhead planes in flight,
+// each in the registers of its own CudaDMAHalo object (manual buffering with
+// two-phase calls, as src/examples/stencil/warp_specialized_manual_buffer.h:54-71,
+// eight objects deep), and lands them one per plane in one of four LDS planes.
+// kRingAhead matches the distance at which the compute threads fetch the
+// interior, so a ring is requested while the neighbouring tiles are pulling the
+// same cache lines as their interior.  The objects that hold the registers
+// carry no handshake; the four LDS planes are guarded by cudaDMACustom objects,
+// the sync-only class of include/cudaDMA.h:4184-4208.
+constexpr int kBufs = 4;
+constexpr int kRingObjs = 8;
+constexpr int kRingAhead = kRingObjs - 1;
+typedef CudaDMAHalo<false, 16, 32, 4, kDmaThreads, kR, false, kTX, kTY> halo_reg_t;
+
+template<typename T>
+struct Eight {
+  T a0, a1, a2, a3, a4, a5, a6, a7;
+  template<int I> __device__ __forceinline__ T& get()
+  {
+    if constexpr (I == 0) return a0; else if constexpr (I == 1) return a1; else if constexpr (I == 2) return a2;
+    else if constexpr (I == 3) return a3; else if constexpr (I == 4) return a4; else if constexpr (I == 5) return a5;
+    else if constexpr (I == 6) return a6; else return a7;
+  }
+};
+template<typename T>
+struct Four {
+  T a0, a1, a2, a3;
+  template<int I> __device__ __forceinline__ T& get()
+  {
+    if constexpr (I == 0) return a0; else if constexpr (I == 1) return a1; else if constexpr (I == 2) return a2;
+    else return a3;
+  }
+};
+
+#define HIPDMA_RING_STEP(J, CHECK, ...) if (!(CHECK) || z0 + (J) < planes) { constexpr int S = (J); const int z = z0 + (J); __VA_ARGS__ }
+#define HIPDMA_RING_GROUP(CHECK, ...)                                                                            \
+  HIPDMA_RING_STEP(0, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(1, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(2, CHECK, __VA_ARGS__) \
+  HIPDMA_RING_STEP(3, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(4, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(5, CHECK, __VA_ARGS__) \
+  HIPDMA_RING_STEP(6, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(7, CHECK, __VA_ARGS__)
+#define HIPDMA_FOR_RING(planes_expr, ...)                                        \
+  {                                                                              \
+    const int planes = (planes_expr);                                            \
+    int z0 = 0;                                                                  \
+    for (; z0 + kRingObjs <= planes; z0 += kRingObjs) { HIPDMA_RING_GROUP(false, __VA_ARGS__) } \
+    if (z0 < planes) { HIPDMA_RING_GROUP(true, __VA_ARGS__) }                    \
+  }
+static_assert(kRingObjs == 8 && kRingObjs % kBufs == 0, "HIPDMA_FOR_RING unrolls eight steps");
+
+template<int SYNC>
+__global__ void __launch_bounds__(kComputeThreads + kDmaThreads)
+stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int nx, const int ny, const int nz,
+                const int zchunk, const Coeffs k)
+{
+  __shared__ __attribute__((aligned(16))) float plane[kBufs][kPlaneFloats];
+  const int px = nx + 2 * kR;
+  const size_t in_plane = (size_t)px * (size_t)(ny + 2 * kR);
+  const size_t out_plane = (size_t)nx * ny;
+  // guards of the four LDS planes: empty/full handshake between the compute and the DMA wavefronts
+  Four<cudaDMACustom> guard{cudaDMACustom(0, kDmaThreads, kComputeThreads, kComputeThreads),
+                            cudaDMACustom(1, kDmaThreads, kComputeThreads, kComputeThreads),
+                            cudaDMACustom(2, kDmaThreads, kComputeThreads, kComputeThreads),
+                            cudaDMACustom(3, kDmaThreads, kComputeThreads, kComputeThreads)};
+  hipdma::GroupBarrier compute_barrier(4, kComputeThreads);
+  const TileWork w = tile_work(in, out, nx, ny, nz, zchunk);
+  constexpr int kOrigin = kR * kPitch + kR;
+
+  if (guard.a0.owns_this_thread()) {
+    Eight<halo_reg_t> ring{halo_reg_t(px, kComputeThreads), halo_reg_t(px, kComputeThreads),
+                           halo_reg_t(px, kComputeThreads), halo_reg_t(px, kComputeThreads),
+                           halo_reg_t(px, kComputeThreads), halo_reg_t(px, kComputeThreads),
+                           halo_reg_t(px, kComputeThreads), halo_reg_t(px, kComputeThreads)};
+    // ring of the centre plane of output plane z: padded plane z + kR
+    const float* ring0 = w.in_origin + (size_t)kR * in_plane;
+    // a request past the last plane re-reads the last one: the loads stay unconditional, nothing lands from them
+    const int last = w.planes - 1;
+#define HIPDMA_ISSUE(I, ZP) \
+    ring.get<(I)>().template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(ring0 + (size_t)((ZP) < last ? (ZP) : last) * in_plane);
+#define HIPDMA_LAND(I, ZP)                                                                                   \
+    if ((ZP) < w.planes) {                                                                                   \
+      if constexpr (SYNC != kBarrierOnly) guard.get<(I) % kBufs>().wait_for_dma_start();                     \
+      ring.get<(I)>().template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(&plane[(I) % kBufs][kOrigin]); \
+      if constexpr (SYNC != kBarrierOnly) guard.get<(I) % kBufs>().finish_async_dma();                       \
+    }
+    // planes 0 .. kRingAhead-1 are requested up front; plane 0 lands before the first barrier
+    HIPDMA_ISSUE(0, 0) HIPDMA_ISSUE(1, 1) HIPDMA_ISSUE(2, 2) HIPDMA_ISSUE(3, 3)
+    HIPDMA_ISSUE(4, 4) HIPDMA_ISSUE(5, 5) HIPDMA_ISSUE(6, 6)
+    HIPDMA_LAND(0, 0)
+    // iteration z: request plane z + kRingAhead, meet the compute wavefronts, land plane z + 1
+    HIPDMA_FOR_RING(w.planes, {
+      HIPDMA_ISSUE((S + kRingAhead) % kRingObjs, z + kRingAhead)
+      if constexpr (SYNC != kHandshakeAndGroupBarrier) __syncthreads();
+      HIPDMA_LAND((S + 1) % kRingObjs, z + 1)
+    })
+#undef HIPDMA_ISSUE
+#undef HIPDMA_LAND
+  } else {
+    const int lx = 4 * (threadIdx.x % kXQ);
+    const int ly = threadIdx.x / kXQ;
+    f32x4_t q[kQueue];
+    const float* col = w.in_origin + (size_t)ly * px + lx;
+    // planes 0 .. kQueue-2 of the chunk; every iteration fetches one more
+    const int avail = w.planes + 2 * kR;                  // padded planes this chunk may touch
+#pragma unroll
+    for (int p = 0; p < kQueue - 1; ++p)
+      q[p] = (p < avail) ? *(const f32x4_t*)(col + (size_t)p * in_plane) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if constexpr (SYNC != kBarrierOnly) {
+      guard.a0.start_async_dma();
+      guard.a1.start_async_dma();
+      guard.a2.start_async_dma();
+      guard.a3.start_async_dma();
+    }
+    *(f32x4_t*)(&plane[0][kOrigin] + ly * kPitch + lx) = q[kR];
+    float* o = w.out_origin + (size_t)ly * nx + lx;
+    HIPDMA_FOR_Z(w.planes, {
+      constexpr int B = ROT % kBufs;
+      const cudaDMACustom& cur_halo = guard.get<B>();
+      // past the end of the chunk the last plane is fetched again: unconditional loads keep the wait counts exact
+      const int zf = (z + kQueue - 1 < avail) ? (z + kQueue - 1) : (avail - 1);
+      q[HIPDMA_QSLOT(ROT, kQueue - 1)] = *(const f32x4_t*)(col + (size_t)zf * in_plane);
+      if constexpr (SYNC != kBarrierOnly) cur_halo.wait_for_dma_finish();
+      if constexpr (SYNC == kHandshakeAndGroupBarrier) compute_barrier.sync();
+      else __syncthreads();
+      const f32x4_t r = stencil_cells4<ROT>(plane[B], lx, ly, q, k);
+      if constexpr (SYNC != kBarrierOnly) cur_halo.start_async_dma();
+      *(f32x4_t*)(&plane[(B + 1) % kBufs][kOrigin] + ly * kPitch + lx) = q[HIPDMA_QSLOT(ROT, kR + 1)];
+      *(f32x4_t*)o = r;
+      o += out_plane;
+    })
+  }
+}
+
+// The form that is not warp-specialised (src/examples/stencil/non_warp_specialized_single_buffer.h:34-58):
+// every thread computes and every other thread also carries one chunk of the
+// ring, requested one plane ahead; one LDS plane, two s_barriers per plane.
+__global__ void __launch_bounds__(kComputeThreads)
+stencil_all_vec4(const float* __restrict__ in, float* __restrict__ out, const int nx, const int ny, const int nz,
+                 const int zchunk, const Coeffs k)
+{
+  __shared__ __attribute__((aligned(16))) float plane[kPlaneFloats];
+  const int px = nx + 2 * kR;
+  const size_t in_plane = (size_t)px * (size_t)(ny + 2 * kR);
+  const size_t out_plane = (size_t)nx * ny;
+  halo_all_t halo(px);
+  const TileWork w = tile_work(in, out, nx, ny, nz, zchunk);
+  float* lds_origin = &plane[kR * kPitch + kR];
+  const int lx = 4 * (threadIdx.x % kXQ);
+  const int ly = threadIdx.x / kXQ;
+  f32x4_t q[kQueue];
+  const float* col = w.in_origin + (size_t)ly * px + lx;
+  const int avail = w.planes + 2 * kR;
+#pragma unroll
+  for (int p = 0; p < kQueue - 1; ++p)
+    q[p] = (p < avail) ? *(const f32x4_t*)(col + (size_t)p * in_plane) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const float* ring0 = w.in_origin + (size_t)kR * in_plane;
+  const int last = w.planes - 1;
+  float* o = w.out_origin + (size_t)ly * nx + lx;
+  halo.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(ring0);
+  HIPDMA_FOR_Z(w.planes, {
+    const int zf = (z + kQueue - 1 < avail) ? (z + kQueue - 1) : (avail - 1);
+    q[HIPDMA_QSLOT(ROT, kQueue - 1)] = *(const f32x4_t*)(col + (size_t)zf * in_plane);
+    halo.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(lds_origin);
+    *(f32x4_t*)(lds_origin + ly * kPitch + lx) = q[HIPDMA_QSLOT(ROT, kR)];
+    __syncthreads();
+    halo.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(ring0 + (size_t)(z < last ? z + 1 : last) * in_plane);
+    *(f32x4_t*)o = stencil_cells4<ROT>(plane, lx, ly, q, k);
+    o += out_plane;
+    __syncthreads();
+  })
+}
+
 }  // namespace
 
 extern "C" int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz, int variant, void* stream)
@@ -201,18 +461,29 @@ extern "C" int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int
   const Coeffs k = {(float)(3.0 * (-205.0 / 72.0)), (float)(8.0 / 5.0), (float)(-1.0 / 5.0), (float)(8.0 / 315.0),
                     (float)(-1.0 / 560.0)};
   // z is cut into chunks so that a 512^3 grid yields a few thousand workgroups instead of 256
-  int zchunk = 64;
+  // enough chunks for two workgroups per compute unit, as few as that allows: every chunk
+  // re-reads 2*radius + prefetch planes before it produces output
+  const long long tiles_xy = (long long)(nx / kTX) * (ny / kTY);
+  const int cus = cudadma_device_cus() > 0 ? cudadma_device_cus() : 256;
+  long long want_chunks = (2LL * cus + tiles_xy - 1) / tiles_xy;
+  if (want_chunks < 1) want_chunks = 1;
+  int zchunk = workloads::tuning("stencil_zchunk", (int)((nz + want_chunks - 1) / want_chunks));
+  if (zchunk < 16) zchunk = 16;
   if (zchunk > nz) zchunk = nz;
   const int chunks = (nz + zchunk - 1) / zchunk;
+  if (workloads::tuning("stencil_xcd_remap", 1) != 2) zchunk |= kXcdFlag;    // knob: 2 turns the XCD-aware numbering off
   const long long grid = (long long)(nx / kTX) * (ny / kTY) * chunks;
   CUDADMA_REQUIRE(grid <= 0x7fffffffLL, "grid too large");
   hipStream_t s = (hipStream_t)stream;
-  if (variant == 0)
-    hipLaunchKernelGGL(stencil_warp_specialized, dim3((unsigned)grid), dim3(kComputeThreads + kDmaThreads), 0, s,
-                       d_in, d_out, nx, ny, nz, zchunk, k);
-  else
-    hipLaunchKernelGGL(stencil_not_specialized, dim3((unsigned)grid), dim3(kComputeThreads), 0, s,
-                       d_in, d_out, nx, ny, nz, zchunk, k);
+  const dim3 g((unsigned)grid), ws(kComputeThreads + kDmaThreads), all(kComputeThreads);
+  switch (variant) {
+    case 0: hipLaunchKernelGGL(stencil_ws_vec4<kHandshakeAndBarrier>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+    case 1: hipLaunchKernelGGL(stencil_ws_vec4<kHandshakeAndGroupBarrier>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+    case 2: hipLaunchKernelGGL(stencil_ws_vec4<kBarrierOnly>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+    case 3: hipLaunchKernelGGL(stencil_all_vec4, g, all, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+    case 4: hipLaunchKernelGGL(stencil_warp_specialized, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+    default: hipLaunchKernelGGL(stencil_not_specialized, g, all, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+  }
   CUDADMA_HIP_CHECK(hipGetLastError());
   return CUDADMA_OK;
 }

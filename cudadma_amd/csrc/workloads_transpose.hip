@@ -19,17 +19,18 @@ constexpr int kDmaThreads = 128;
 constexpr int kComputeThreads = 128;
 constexpr int kBytesPerThread = kTile * kRowBytes / kDmaThreads;   // 128: the whole tile in one step
 
-// Tile order: x fastest inside bands of kBand tile rows, so that the workgroups
-// resident at one time read long contiguous runs of the source rows and also
-// write runs of kBand * 256 B of the output rows.
-constexpr int kBand = 16;
+// Tile order: the matrix is cut into bands of `band` tile rows; inside a band
+// the tile row index runs fastest, then the tile column.  The workgroups
+// resident at one time therefore read runs of (resident / band) * 256 B of the
+// source rows and write runs of band * 256 B of the output rows.
+constexpr int kDefaultBand = 16;
 
-__device__ __forceinline__ void tile_coords(const int t, const int tiles_per_side, int& ty, int& tx)
+__device__ __forceinline__ void tile_coords(const int t, const int tiles_per_side, const int band_rows, int& ty, int& tx)
 {
-  const int band = t / (kBand * tiles_per_side);
-  const int in_band = t - band * (kBand * tiles_per_side);
-  tx = in_band / kBand;
-  ty = band * kBand + (in_band - tx * kBand);
+  const int band = t / (band_rows * tiles_per_side);
+  const int in_band = t - band * (band_rows * tiles_per_side);
+  tx = in_band / band_rows;
+  ty = band * band_rows + (in_band - tx * band_rows);
 }
 
 template<int LDS_ROW_BYTES, typename Dma>
@@ -56,7 +57,8 @@ __device__ __forceinline__ void write_tile_transposed(const char* lds_tile, floa
 
 template<int LDS_ROW_BYTES>
 __global__ void __launch_bounds__(kDmaThreads + kComputeThreads)
-transpose_manual_double(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles)
+transpose_manual_double(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles,
+                        const int band)
 {
   __shared__ __attribute__((aligned(16))) char buf0[kTile * LDS_ROW_BYTES];
   __shared__ __attribute__((aligned(16))) char buf1[kTile * LDS_ROW_BYTES];
@@ -67,7 +69,7 @@ transpose_manual_double(const float* __restrict__ in, float* __restrict__ out, c
   const int stride = gridDim.x;
   auto src_of = [&](const int t) {
     int ty, tx;
-    tile_coords(t, tiles_per_side, ty, tx);
+    tile_coords(t, tiles_per_side, band, ty, tx);
     return (const void*)(in + (size_t)ty * kTile * n + (size_t)tx * kTile);
   };
   if (dma0.owns_this_thread()) {
@@ -87,11 +89,11 @@ transpose_manual_double(const float* __restrict__ in, float* __restrict__ out, c
     dma1.start_async_dma();
     for (int t = blockIdx.x; t < num_tiles; t += 2 * stride) {
       int ty, tx;
-      tile_coords(t, tiles_per_side, ty, tx);
+      tile_coords(t, tiles_per_side, band, ty, tx);
       dma0.wait_for_dma_finish();
       write_tile_transposed<LDS_ROW_BYTES>(buf0, out, n, ty, tx, dma0);
       if (t + stride < num_tiles) {
-        tile_coords(t + stride, tiles_per_side, ty, tx);
+        tile_coords(t + stride, tiles_per_side, band, ty, tx);
         dma1.wait_for_dma_finish();
         write_tile_transposed<LDS_ROW_BYTES>(buf1, out, n, ty, tx, dma1);
       }
@@ -100,7 +102,7 @@ transpose_manual_double(const float* __restrict__ in, float* __restrict__ out, c
 }
 
 __global__ void __launch_bounds__(kDmaThreads + kComputeThreads)
-transpose_single(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles)
+transpose_single(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles, const int band)
 {
   constexpr int kLdsRow = 272;
   __shared__ __attribute__((aligned(16))) char buf[kTile * kLdsRow];
@@ -110,14 +112,14 @@ transpose_single(const float* __restrict__ in, float* __restrict__ out, const in
   if (dma.owns_this_thread()) {
     for (int t = blockIdx.x; t < num_tiles; t += gridDim.x) {
       int ty, tx;
-      tile_coords(t, tiles_per_side, ty, tx);
+      tile_coords(t, tiles_per_side, band, ty, tx);
       dma.template execute_dma<true, LOAD_CACHE_ALL, STORE_LDS>(in + (size_t)ty * kTile * n + (size_t)tx * kTile, buf);
     }
   } else {
     dma.start_async_dma();
     for (int t = blockIdx.x; t < num_tiles; t += gridDim.x) {
       int ty, tx;
-      tile_coords(t, tiles_per_side, ty, tx);
+      tile_coords(t, tiles_per_side, band, ty, tx);
       dma.wait_for_dma_finish();
       write_tile_transposed<kLdsRow>(buf, out, n, ty, tx, dma);
     }
@@ -129,7 +131,8 @@ transpose_single(const float* __restrict__ in, float* __restrict__ out, const in
 extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n, int variant, void* stream)
 {
   CUDADMA_REQUIRE(n >= 0 && (n % kTile) == 0, "n (%d) must be a multiple of %d", n, kTile);
-  CUDADMA_REQUIRE((n / kTile) % kBand == 0 || n == 0, "n / 64 (%d) must be a multiple of %d", n / kTile, kBand);
+  int band = workloads::tuning("transpose_band", kDefaultBand);
+  while (band > 1 && (n / kTile) % band != 0) band /= 2;      // bands must tile the matrix
   CUDADMA_REQUIRE((long long)n * 4 <= 0x7fffffffLL, "row pitch must fit an int");
   if (variant < 0 || variant >= cudadma_num_variants(CUDADMA_WORKLOAD_STRIDED)) {
     cudadma_host::set_error("strided transpose has no variant %d", variant);
@@ -142,9 +145,9 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
   hipStream_t s = (hipStream_t)stream;
   const dim3 block(kDmaThreads + kComputeThreads);
   switch (variant) {
-    case 0: hipLaunchKernelGGL(transpose_manual_double<272>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles); break;
-    case 1: hipLaunchKernelGGL(transpose_single, dim3(workloads::persistent_grid(tiles, 8)), block, 0, s, d_in, d_out, n, tiles); break;
-    default: hipLaunchKernelGGL(transpose_manual_double<256>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles); break;
+    case 0: hipLaunchKernelGGL(transpose_manual_double<272>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 1: hipLaunchKernelGGL(transpose_single, dim3(workloads::persistent_grid(tiles, 8)), block, 0, s, d_in, d_out, n, tiles, band); break;
+    default: hipLaunchKernelGGL(transpose_manual_double<256>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
   }
   CUDADMA_HIP_CHECK(hipGetLastError());
   return CUDADMA_OK;

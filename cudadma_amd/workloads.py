@@ -40,6 +40,13 @@ def set_workgroups_per_cu(value):
     return lib().cudadma_set_workgroups_per_cu(int(value))
 
 
+def set_tuning(name, value):
+    rc = lib().cudadma_set_tuning(name.encode(), int(value))
+    if rc < 0:
+        check(rc)
+    return rc
+
+
 def fill_uniform(out, seed):
     _need(out, torch.float32, "out")
     check(lib().cudadma_fill_uniform(_p(out), out.numel(), seed, _stream()))

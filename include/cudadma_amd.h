@@ -132,6 +132,12 @@ const char* cudadma_variant_name(int workload, int variant);
 /* Tuning knob: workgroups resident per compute unit for the persistent grids
  * (0 restores each kernel's default).  Returns the previous value. */
 int cudadma_set_workgroups_per_cu(int value);
+/* Further integer knobs by name (0 restores the default); returns the previous
+ * value or CUDADMA_EINVAL for an unknown name:
+ *   "transpose_band"  tile rows per band of the config 2 tile order
+ *   "stencil_zchunk"     output planes one workgroup marches through in config 4
+ *   "stencil_xcd_remap"  config 4 numbers its workgroups so that each XCD gets a contiguous part of the grid; 2 turns that off */
+int cudadma_set_tuning(const char* name, int value);
 
 /* Seeded inputs generated on the device; bit-identical to the host statement
  * h(i) = splitmix64(seed + i) >> 32, value = (h >> 8) * 2^-23 - 1. */

@@ -60,6 +60,18 @@ struct HaloGeom {
     s1 = round_up(2 * RADIUS * w1, HIPDMA_WAVE_SIZE);
     total = s1 + 2 * dimy * W2;
   }
+  // What the slots [round*threads, (round+1)*threads) of one round are:
+  //   0  all of them live row chunks, 1  all of them live side chunks, 2  a mix, or some idle.
+  // With compile-time tile size and thread count this folds to a constant, which
+  // turns the whole transfer into straight-line code: no per-lane predication,
+  // so loads of later transfers can stay in flight across it.
+  __host__ __device__ __forceinline__ int round_kind(const int round, const int threads) const
+  {
+    const int lo = round * threads, hi = lo + threads;
+    if ((w1 == lpr) && (hi <= 2 * RADIUS * w1)) return 0;
+    if ((W2 == LPS) && (lo >= s1) && (hi <= total)) return 1;
+    return 2;
+  }
   __host__ __device__ __forceinline__ HaloSlot decode(const int s) const
   {
     HaloSlot r;
@@ -182,6 +194,11 @@ public:
     m_src = (const char*)src_origin;
     pass<true, DMA_GLOBAL_LOAD, DMA_LOAD_QUAL, DMA_STORE_QUAL>(0, nullptr);
   }
+  // Second half of a two-phase transfer without the handshake (the two-phase
+  // counterpart of execute_dma_no_sync).
+  template<bool DMA_GLOBAL_LOAD, int DMA_LOAD_QUAL, int DMA_STORE_QUAL>
+  __device__ __forceinline__ void drain_no_sync(void* __restrict__ dst_origin)
+  { drain<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL, DMA_STORE_QUAL>((char*)dst_origin); }
   template<bool DMA_GLOBAL_LOAD, int DMA_LOAD_QUAL, int DMA_STORE_QUAL>
   __device__ __forceinline__ void wait_xfer_finish(void* __restrict__ dst_origin)
   {
@@ -220,21 +237,28 @@ private:
     using namespace hipdma::detail;
 #pragma unroll
     for (int k = 0; k < MAX_LDS; ++k) {
-      const HaloSlot slot = m_geom.decode(m_tid + (step * MAX_LDS + k) * m_threads);
-      if (slot.live) {
-        if (slot.is_row) {
-          if constexpr (IS_LOAD)
-            load_chunk<ALIGNMENT, XR, GLOBAL_LOAD, LOAD_QUAL>(m_buf[k], m_src + slot.src_off, slot.nbytes);
-          else
-            store_chunk<ALIGNMENT, XR, STORE_QUAL>(m_buf[k], dst + slot.dst_off, slot.nbytes);
-        } else {
-          if constexpr (IS_LOAD)
-            load_chunk<ALIGNMENT, XS, GLOBAL_LOAD, LOAD_QUAL>(m_buf[k], m_src + slot.src_off, XS);
-          else
-            store_chunk<ALIGNMENT, XS, STORE_QUAL>(m_buf[k], dst + slot.dst_off, XS);
-        }
+      const int round = step * MAX_LDS + k;
+      const int kind = m_geom.round_kind(round, m_threads);
+      const HaloSlot slot = m_geom.decode(m_tid + round * m_threads);
+      if (kind == 0) {
+        move<IS_LOAD, XR, GLOBAL_LOAD, LOAD_QUAL, STORE_QUAL>(k, slot, dst, slot.nbytes);
+      } else if (kind == 1) {
+        move<IS_LOAD, XS, GLOBAL_LOAD, LOAD_QUAL, STORE_QUAL>(k, slot, dst, XS);
+      } else if (slot.live) {
+        if (slot.is_row) move<IS_LOAD, XR, GLOBAL_LOAD, LOAD_QUAL, STORE_QUAL>(k, slot, dst, slot.nbytes);
+        else move<IS_LOAD, XS, GLOBAL_LOAD, LOAD_QUAL, STORE_QUAL>(k, slot, dst, XS);
       }
     }
+  }
+
+  template<bool IS_LOAD, int PIECE, bool GLOBAL_LOAD, int LOAD_QUAL, int STORE_QUAL>
+  __device__ __forceinline__ void move(const int k, const hipdma::detail::HaloSlot& slot, char* dst, const int nbytes)
+  {
+    using namespace hipdma::detail;
+    if constexpr (IS_LOAD)
+      load_chunk<ALIGNMENT, PIECE, GLOBAL_LOAD, LOAD_QUAL>(m_buf[k], m_src + slot.src_off, nbytes);
+    else
+      store_chunk<ALIGNMENT, PIECE, STORE_QUAL>(m_buf[k], dst + slot.dst_off, nbytes);
   }
 
 private:

@@ -242,7 +242,8 @@ void oracle_gather_rowsum(const float* table, const int32_t* idx, float* out, si
 /* Config 4: 8th-order, 25-point star stencil (second derivative in each axis).
  * `in` is a (nx+2p) x (ny+2p) x (nz+2p) array (x fastest) with p = radius_pad >= 4;
  * `out` is nx x ny x nz.  Fixed evaluation order:
- *   acc = c0 * centre; for r = 1..4: acc += c[r] * (((xm + xp) + (ym + yp)) + (zm + zp)) */
+ *   acc = c0 * centre; for r = 1..4: acc = fma(c[r], ((xm + xp) + (ym + yp)) + (zm + zp), acc)
+ * with every other operation rounded on its own (no contraction). */
 void oracle_stencil25(const float* in, float* out, int nx, int ny, int nz, int radius_pad)
 {
   const float c0 = (float)(3.0 * (-205.0 / 72.0));
@@ -259,7 +260,7 @@ void oracle_stencil25(const float* in, float* out, int nx, int ny, int nz, int r
           const float sx = in[o - r] + in[o + r];
           const float sy = in[o - r * px] + in[o + r * px];
           const float sz = in[o - r * px * py] + in[o + r * px * py];
-          acc += c[r] * ((sx + sy) + sz);
+          acc = fmaf(c[r], (sx + sy) + sz, acc);
         }
         out[((size_t)z * ny + y) * nx + x] = acc;
       }
