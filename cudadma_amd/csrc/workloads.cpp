@@ -50,6 +50,8 @@ static const VariantInfo kStrided[] = {
   {"manual double buffer: one DMA group of 2 wavefronts, two CudaDMAStrided objects, padded LDS rows (272 B)"},
   {"single buffer: one object, execute_dma"},
   {"manual double buffer, unpadded LDS rows (256 B): shows the bank-conflict cost"},
+  {"double buffer: two DMA groups of 1 wavefront, one CudaDMAStrided object and one padded LDS tile each"},
+  {"not warp-specialised: all four wavefronts move the tile and write it out, next tile requested two-phase"},
 };
 static const VariantInfo kGather[] = {
   {"manual 4-stage buffering: one DMA group of 2 wavefronts, four CudaDMAIndirect objects"},

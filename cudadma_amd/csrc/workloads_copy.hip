@@ -39,9 +39,24 @@ copy_manual_double(const char* __restrict__ in, char* __restrict__ out, const in
   const int stride = gridDim.x;
   if (dma0.owns_this_thread()) {
     int t = blockIdx.x;
-    if (t < num_tiles) dma0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_QUAL>(in + (size_t)t * kTileBytes);
-    if (t + stride < num_tiles)
+    if (t + 3 * stride < num_tiles) {
+      // Steady state with no branch around any load, entered from a prologue that has none either:
+      // the wait for one object's tile then leaves the other object's loads in flight.
+      dma0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_QUAL>(in + (size_t)t * kTileBytes);
       dma1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_QUAL>(in + (size_t)(t + stride) * kTileBytes);
+      do {
+        dma0.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_QUAL>(buf0);
+        dma0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_QUAL>(in + (size_t)(t + 2 * stride) * kTileBytes);
+        dma1.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_QUAL>(buf1);
+        dma1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_QUAL>(in + (size_t)(t + 3 * stride) * kTileBytes);
+        t += 2 * stride;
+      } while (t + 3 * stride < num_tiles);
+    } else {
+      if (t < num_tiles) dma0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_QUAL>(in + (size_t)t * kTileBytes);
+      if (t + stride < num_tiles)
+        dma1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_QUAL>(in + (size_t)(t + stride) * kTileBytes);
+    }
+    // the last tiles of this workgroup
     for (; t < num_tiles; t += 2 * stride) {
       dma0.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_QUAL>(buf0);
       if (t + 2 * stride < num_tiles)

@@ -71,11 +71,28 @@ gather_manual(const float* __restrict__ table, const int* __restrict__ idx, floa
   if constexpr (STAGES > 2) { constexpr int s = 2; dma_t& d = dma2; __VA_ARGS__ } \
   if constexpr (STAGES > 3) { constexpr int s = 3; dma_t& d = dma3; __VA_ARGS__ }
   if (dma0.owns_this_thread()) {
-    HIPDMA_FOR_STAGES({
-      const long long tt = first + s * stride;
-      if (tt < num_tiles) d.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(idx + tt * kRecsPerTile, table);
-    })
-    for (long long t = first; t < num_tiles; t += STAGES * stride) {
+    long long t = first;
+    if (t + (2 * STAGES - 1) * stride < num_tiles) {
+      // Steady state with no branch around any load, entered from a prologue that has none either:
+      // waiting for one stage then leaves the loads of the other stages in flight.
+      HIPDMA_FOR_STAGES({
+        d.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(idx + (t + s * stride) * kRecsPerTile, table);
+      })
+      do {
+        HIPDMA_FOR_STAGES({
+          d.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf[s]);
+          d.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(idx + (t + (s + STAGES) * stride) * kRecsPerTile, table);
+        })
+        t += STAGES * stride;
+      } while (t + (2 * STAGES - 1) * stride < num_tiles);
+    } else {
+      HIPDMA_FOR_STAGES({
+        const long long tt = t + s * stride;
+        if (tt < num_tiles) d.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(idx + tt * kRecsPerTile, table);
+      })
+    }
+    // the last tiles of this workgroup
+    for (; t < num_tiles; t += STAGES * stride) {
       HIPDMA_FOR_STAGES({
         const long long tt = t + s * stride;
         if (tt < num_tiles) {

@@ -74,8 +74,24 @@ transpose_manual_double(const float* __restrict__ in, float* __restrict__ out, c
   };
   if (dma0.owns_this_thread()) {
     int t = blockIdx.x;
-    if (t < num_tiles) dma0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t));
-    if (t + stride < num_tiles) dma1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t + stride));
+    if (t + 3 * stride < num_tiles) {
+      // Steady state with no branch around any load, entered from a prologue that has none either:
+      // every path into a wait then carries the same loads, and the wait for one object's tile
+      // leaves the other object's eight loads in flight (s_waitcnt vmcnt(15..8), not vmcnt(7..0)).
+      dma0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t));
+      dma1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t + stride));
+      do {
+        dma0.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf0);
+        dma0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t + 2 * stride));
+        dma1.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf1);
+        dma1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t + 3 * stride));
+        t += 2 * stride;
+      } while (t + 3 * stride < num_tiles);
+    } else {
+      if (t < num_tiles) dma0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t));
+      if (t + stride < num_tiles) dma1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t + stride));
+    }
+    // the last tiles of this workgroup
     for (; t < num_tiles; t += 2 * stride) {
       dma0.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf0);
       if (t + 2 * stride < num_tiles) dma0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t + 2 * stride));
@@ -97,6 +113,105 @@ transpose_manual_double(const float* __restrict__ in, float* __restrict__ out, c
         dma1.wait_for_dma_finish();
         write_tile_transposed<LDS_ROW_BYTES>(buf1, out, n, ty, tx, dma1);
       }
+    }
+  }
+}
+
+// Two DMA groups of one wavefront, one object and one LDS tile each
+// (src/perf/sequential/perf_sequential.cu:116-173).  A wavefront's loads complete in
+// issue order and s_waitcnt counts them in that order, so a wavefront that owns a
+// single object waits for exactly its own tile; the second tile in flight belongs
+// to the other wavefront.  Each DMA thread holds a whole tile share of 16 dwordx4.
+template<int LDS_ROW_BYTES>
+__global__ void __launch_bounds__(kDmaThreads + kComputeThreads)
+transpose_double_groups(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles,
+                        const int band)
+{
+  __shared__ __attribute__((aligned(16))) char buf0[kTile * LDS_ROW_BYTES];
+  __shared__ __attribute__((aligned(16))) char buf1[kTile * LDS_ROW_BYTES];
+  constexpr int kGroup = kDmaThreads / 2;
+  typedef CudaDMAStrided<true, 16, kTile * kRowBytes / kGroup, kRowBytes, kGroup, kTile> dma_t;
+  dma_t dma0(0, kComputeThreads, kComputeThreads, n * 4, LDS_ROW_BYTES);
+  dma_t dma1(1, kComputeThreads, kComputeThreads + kGroup, n * 4, LDS_ROW_BYTES);
+  const int tiles_per_side = n / kTile;
+  const int stride = gridDim.x;
+  auto src_of = [&](const int t) {
+    int ty, tx;
+    tile_coords(t, tiles_per_side, band, ty, tx);
+    return (const void*)(in + (size_t)ty * kTile * n + (size_t)tx * kTile);
+  };
+  auto dma_loop = [&](dma_t& dma, char* buf, int t) {
+    if (t < num_tiles) dma.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t));
+    for (; t + 2 * stride < num_tiles; t += 2 * stride) {
+      dma.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf);
+      dma.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t + 2 * stride));
+    }
+    if (t < num_tiles) dma.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf);
+  };
+  if (dma0.owns_this_thread()) {
+    dma_loop(dma0, buf0, blockIdx.x);
+  } else if (dma1.owns_this_thread()) {
+    dma_loop(dma1, buf1, blockIdx.x + stride);
+  } else {
+    dma0.start_async_dma();
+    dma1.start_async_dma();
+    for (int t = blockIdx.x; t < num_tiles; t += 2 * stride) {
+      int ty, tx;
+      tile_coords(t, tiles_per_side, band, ty, tx);
+      dma0.wait_for_dma_finish();
+      write_tile_transposed<LDS_ROW_BYTES>(buf0, out, n, ty, tx, dma0);
+      if (t + stride < num_tiles) {
+        tile_coords(t + stride, tiles_per_side, band, ty, tx);
+        dma1.wait_for_dma_finish();
+        write_tile_transposed<LDS_ROW_BYTES>(buf1, out, n, ty, tx, dma1);
+      }
+    }
+  }
+}
+
+// The form that is not warp-specialised (src/examples/stencil/non_warp_specialized_double_buffer.h:52-89):
+// all four wavefronts move the tile into LDS, meet, and all four write it out
+// transposed.  The next tile is requested (two-phase call) before the current one
+// is consumed, so its loads are in flight under the LDS reads and the stores.
+__global__ void __launch_bounds__(kDmaThreads + kComputeThreads)
+transpose_not_specialized(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles,
+                          const int band)
+{
+  constexpr int kLdsRow = 272;
+  constexpr int kThreads = kDmaThreads + kComputeThreads;
+  __shared__ __attribute__((aligned(16))) char buf[kTile * kLdsRow];
+  CudaDMAStrided<false, 16, kTile * kRowBytes / kThreads, kRowBytes, kThreads, kTile> dma(n * 4, kLdsRow);
+  const int tiles_per_side = n / kTile;
+  const int stride = gridDim.x;
+  const int last = num_tiles - 1;
+  auto src_of = [&](const int t) {
+    int ty, tx;
+    tile_coords(t, tiles_per_side, band, ty, tx);
+    return (const void*)(in + (size_t)ty * kTile * n + (size_t)tx * kTile);
+  };
+  const int lane = threadIdx.x & 63;
+  const int w = threadIdx.x >> 6;          // wavefront w writes tile columns [16w, 16w+16)
+  int t = blockIdx.x;
+  if (t >= num_tiles) return;
+  dma.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t));
+  for (; t < num_tiles; t += stride) {
+    dma.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf);
+    __syncthreads();
+    // past the last tile the last one is requested again: the loads stay unconditional
+    const int tn = (t + stride < num_tiles) ? (t + stride) : last;
+    dma.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(tn));
+    vec4_t v[4];
+    const vec4_t* row = (const vec4_t*)(buf + lane * kLdsRow) + w * 4;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = row[j];
+    __syncthreads();
+    int ty, tx;
+    tile_coords(t, tiles_per_side, band, ty, tx);
+    float* o = out + (size_t)(tx * kTile + w * 16) * n + (size_t)ty * kTile + lane;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[(size_t)(4 * j + k) * n] = __uint_as_float(v[j][k]);
     }
   }
 }
@@ -147,7 +262,9 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
   switch (variant) {
     case 0: hipLaunchKernelGGL(transpose_manual_double<272>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 1: hipLaunchKernelGGL(transpose_single, dim3(workloads::persistent_grid(tiles, 8)), block, 0, s, d_in, d_out, n, tiles, band); break;
-    default: hipLaunchKernelGGL(transpose_manual_double<256>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 2: hipLaunchKernelGGL(transpose_manual_double<256>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 3: hipLaunchKernelGGL(transpose_double_groups<272>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
+    default: hipLaunchKernelGGL(transpose_not_specialized, dim3(workloads::persistent_grid(tiles, 6)), block, 0, s, d_in, d_out, n, tiles, band); break;
   }
   CUDADMA_HIP_CHECK(hipGetLastError());
   return CUDADMA_OK;
