@@ -24,8 +24,8 @@ HBM_PEAK_GBS = 8000.0           # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # scaled by what the same counters read for the plain copy kernel (see profiles/).
-# None until such a profile has been taken for the current kernel.
-MEASURED_TRAFFIC_BYTES = {"strided": None}
+# profiles/bench_all_patterns_mi355x.md: FETCH_SIZE 524384 KiB x 2.0000 + WRITE_SIZE 1048576 KiB x 1.0000.
+MEASURED_TRAFFIC_BYTES = {"strided": 2147680256}
 
 
 def log(msg):
@@ -145,9 +145,9 @@ def main():
     grid_out = torch.empty((g, g, g), dtype=torch.float32, device=dev)
     ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 0), steps, warmup)
     report("halo", ms, 2 * g ** 3 * 4, "CudaDMAHalo radius-4 ring of 32x32 tiles, 25-point stencil on a 512^3 f32 grid "
-           "(empty/full handshake + one s_barrier per plane)")
-    ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 2), steps, warmup)
-    report("halo_barrier_only", ms, 2 * g ** 3 * 4, "same kernel with execute_dma_no_sync: ordered by the per-plane s_barrier alone")
+           "(ring landed without handshake, one s_barrier per plane)")
+    ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 1), steps, warmup)
+    report("halo_handshake", ms, 2 * g ** 3 * 4, "same kernel with the empty/full handshake on the LDS planes next to the s_barrier")
     del grid_in, grid_out
 
     value = patterns["strided"]["GB/s"]

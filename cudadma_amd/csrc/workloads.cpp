@@ -8,12 +8,18 @@ namespace workloads {
 static std::atomic<int> g_wg_per_cu{0};
 static int g_cus = 0;
 
-int persistent_grid(long long work_items, int default_wg_per_cu)
+int device_cus()
 {
   if (g_cus <= 0) {
     g_cus = cudadma_device_cus();
     if (g_cus <= 0) g_cus = 256;
   }
+  return g_cus;
+}
+
+int persistent_grid(long long work_items, int default_wg_per_cu)
+{
+  device_cus();
   const int knob = g_wg_per_cu.load();
   const long long want = (long long)g_cus * (knob > 0 ? knob : default_wg_per_cu);
   return (int)(work_items < want ? work_items : want);
@@ -59,10 +65,11 @@ static const VariantInfo kGather[] = {
   {"manual double buffer: two objects"},
 };
 static const VariantInfo kHalo[] = {
-  {"warp-specialised, 4 cells per thread as one dwordx4: CudaDMAHalo ring by 1 DMA wavefront with the empty/full "
-   "handshake, one s_barrier per plane for the interior exchange"},
-  {"as variant 0 but the compute wavefronts meet in an LDS-counter GroupBarrier and the DMA wavefront runs free"},
-  {"as variant 0 without the handshake: execute_dma_no_sync, ordered by the per-plane s_barrier alone"},
+  {"warp-specialised, 4 cells per thread as one dwordx4: 1 DMA wavefront keeps the rings of 7 planes in flight in 8 "
+   "CudaDMAHalo objects and lands one per plane (execute_dma_no_sync style); one s_barrier per plane orders the ring, "
+   "the interior exchange and the reuse of the 4 LDS planes"},
+  {"as variant 0 plus the empty/full handshake (cudaDMACustom guards on the 4 LDS planes) next to the s_barrier"},
+  {"as variant 1 but the compute wavefronts meet in an LDS-counter GroupBarrier and the DMA wavefront runs free"},
   {"not warp-specialised, dwordx4 cells: every thread computes, half of them also carry a ring chunk requested one "
    "plane ahead; one LDS plane, two s_barriers per plane"},
   {"warp-specialised, one cell per dword load (first version kept for comparison)"},

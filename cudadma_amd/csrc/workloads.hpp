@@ -10,6 +10,8 @@ namespace workloads {
 // Workgroups to launch for a persistent kernel: CUs x (knob or the kernel's
 // default), never more than there are work items.
 int persistent_grid(long long work_items, int default_wg_per_cu);
+// Compute units of the current device, queried once.
+int device_cus();
 
 // Value of a named knob, or `fallback` while it is unset (0).
 int tuning(const char* name, int fallback);

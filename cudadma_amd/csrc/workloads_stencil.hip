@@ -223,6 +223,17 @@ enum SyncMode {
 // Four cells of row ly starting at column lx; plane p of the z column is q[HIPDMA_QSLOT(ROT, p)].
 // Same operations in the same order as the host statement: one multiply, then per
 // radius five additions and one fused multiply-add.
+// Tile row of a compute thread.  Eight lanes share a row (128 B); ds_read_b128 serves
+// sixteen lanes at a time, and with the 40-float row pitch the second eight must sit
+// four rows further down (4 * 160 B = 640 B = 32 banks off) to stay clear of the
+// banks of the first eight.
+__device__ __forceinline__ int tile_row_of_thread()
+{
+  const int half = (threadIdx.x / kXQ) & 1;
+  const int group = threadIdx.x / (2 * kXQ);          // 0 .. 15
+  return (group / 4) * 8 + (group % 4) + 4 * half;
+}
+
 template<int ROT>
 __device__ __forceinline__ f32x4_t stencil_cells4(const float* __restrict__ plane, const int lx, const int ly,
                                                   const f32x4_t (&q)[kQueue], const Coeffs& k)
@@ -373,7 +384,7 @@ stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int
 #undef HIPDMA_LAND
   } else {
     const int lx = 4 * (threadIdx.x % kXQ);
-    const int ly = threadIdx.x / kXQ;
+    const int ly = tile_row_of_thread();
     f32x4_t q[kQueue];
     const float* col = w.in_origin + (size_t)ly * px + lx;
     // planes 0 .. kQueue-2 of the chunk; every iteration fetches one more
@@ -422,7 +433,7 @@ stencil_all_vec4(const float* __restrict__ in, float* __restrict__ out, const in
   const TileWork w = tile_work(in, out, nx, ny, nz, zchunk);
   float* lds_origin = &plane[kR * kPitch + kR];
   const int lx = 4 * (threadIdx.x % kXQ);
-  const int ly = threadIdx.x / kXQ;
+  const int ly = tile_row_of_thread();
   f32x4_t q[kQueue];
   const float* col = w.in_origin + (size_t)ly * px + lx;
   const int avail = w.planes + 2 * kR;
@@ -461,11 +472,12 @@ extern "C" int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int
   const Coeffs k = {(float)(3.0 * (-205.0 / 72.0)), (float)(8.0 / 5.0), (float)(-1.0 / 5.0), (float)(8.0 / 315.0),
                     (float)(-1.0 / 560.0)};
   // z is cut into chunks so that a 512^3 grid yields a few thousand workgroups instead of 256
-  // enough chunks for two workgroups per compute unit, as few as that allows: every chunk
-  // re-reads 2*radius + prefetch planes before it produces output
+  // z is cut into as few chunks as still give every compute unit work: each chunk re-reads
+  // 2*radius + prefetch planes before it produces output.  The variants that pay for the
+  // handshake want two workgroups per compute unit to hide it, the others run best with one.
   const long long tiles_xy = (long long)(nx / kTX) * (ny / kTY);
-  const int cus = cudadma_device_cus() > 0 ? cudadma_device_cus() : 256;
-  long long want_chunks = (2LL * cus + tiles_xy - 1) / tiles_xy;
+  const int per_cu = (variant == 0 || variant == 3) ? 1 : 2;
+  long long want_chunks = ((long long)per_cu * workloads::device_cus() + tiles_xy - 1) / tiles_xy;
   if (want_chunks < 1) want_chunks = 1;
   int zchunk = workloads::tuning("stencil_zchunk", (int)((nz + want_chunks - 1) / want_chunks));
   if (zchunk < 16) zchunk = 16;
@@ -477,9 +489,9 @@ extern "C" int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int
   hipStream_t s = (hipStream_t)stream;
   const dim3 g((unsigned)grid), ws(kComputeThreads + kDmaThreads), all(kComputeThreads);
   switch (variant) {
-    case 0: hipLaunchKernelGGL(stencil_ws_vec4<kHandshakeAndBarrier>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
-    case 1: hipLaunchKernelGGL(stencil_ws_vec4<kHandshakeAndGroupBarrier>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
-    case 2: hipLaunchKernelGGL(stencil_ws_vec4<kBarrierOnly>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+    case 0: hipLaunchKernelGGL(stencil_ws_vec4<kBarrierOnly>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+    case 1: hipLaunchKernelGGL(stencil_ws_vec4<kHandshakeAndBarrier>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+    case 2: hipLaunchKernelGGL(stencil_ws_vec4<kHandshakeAndGroupBarrier>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
     case 3: hipLaunchKernelGGL(stencil_all_vec4, g, all, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
     case 4: hipLaunchKernelGGL(stencil_warp_specialized, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
     default: hipLaunchKernelGGL(stencil_not_specialized, g, all, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
