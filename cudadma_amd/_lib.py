@@ -106,6 +106,7 @@ _WORKLOAD_SIGNATURES = {
     "cudadma_gather_copy": [_vp, _vp, _vp, _cs, _cs, _ci, _vp],
     "cudadma_gather_rowsum": [_vp, _vp, _vp, _cs, _cs, _ci, _vp],
     "cudadma_halo_stencil": [_vp, _vp, _ci, _ci, _ci, _ci, _vp],
+    "cudadma_gemm_bf16": [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
 }
 
 

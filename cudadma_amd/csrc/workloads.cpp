@@ -76,6 +76,11 @@ static const VariantInfo kHalo[] = {
   {"not warp-specialised, one cell per dword load"},
 };
 
+static const VariantInfo kGemm[] = {
+  {"warp-specialised: one DMA wavefront per operand (CudaDMAStrided, two LDS stages behind one object), four compute "
+   "wavefronts with v_mfma_f32_32x32x16_bf16, B fragments through ds_read_b64_tr_b16"},
+};
+
 static const VariantInfo* table(int workload, int* count)
 {
   switch (workload) {
@@ -83,6 +88,7 @@ static const VariantInfo* table(int workload, int* count)
     case CUDADMA_WORKLOAD_STRIDED:    *count = sizeof(kStrided) / sizeof(VariantInfo);    return kStrided;
     case CUDADMA_WORKLOAD_GATHER:     *count = sizeof(kGather) / sizeof(VariantInfo);     return kGather;
     case CUDADMA_WORKLOAD_HALO:       *count = sizeof(kHalo) / sizeof(VariantInfo);       return kHalo;
+    case CUDADMA_WORKLOAD_GEMM:       *count = sizeof(kGemm) / sizeof(VariantInfo);       return kGemm;
     default: *count = 0; return nullptr;
   }
 }

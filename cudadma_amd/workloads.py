@@ -115,3 +115,16 @@ def halo_stencil(grid_in, grid_out, variant=0):
         raise ValueError("grid_in must be the output shape plus 8 in every dimension")
     check(lib().cudadma_halo_stencil(_p(grid_in), _p(grid_out), nx, ny, nz, variant, _stream()))
     return grid_out
+
+
+def gemm_bf16(a, b, c, variant=0):
+    """a: (m, k) and b: (k, n) torch.bfloat16, c: (m, n) float32; returns c = a @ b with fp32 accumulation."""
+    _need(a, torch.bfloat16, "a")
+    _need(b, torch.bfloat16, "b")
+    _need(c, torch.float32, "c")
+    m, k = a.shape
+    k2, n = b.shape
+    if k2 != k or tuple(c.shape) != (m, n):
+        raise ValueError("shapes do not agree")
+    check(lib().cudadma_gemm_bf16(_p(a), _p(b), _p(c), m, n, k, variant, _stream()))
+    return c

@@ -187,3 +187,63 @@ def test_halo_stencil_full_size(device):
     wl.halo_stencil(d_in, d_out, 0)
     torch.cuda.synchronize()
     assert float(d_out.abs().max()) <= 1e-5
+
+
+# ------------------------------------------------------------------ config 5
+GEMM_RTOL = 1e-2          # BASELINE config 5: within 1e-2 relative of the fp32 host GEMM
+
+
+def _bf16_inputs(m, n, k):
+    a = np.empty(m * k, dtype=np.uint16)
+    b = np.empty(k * n, dtype=np.uint16)
+    O = ol.load()
+    O.oracle_fill_normal_bf16(ptr(a), a.size, 1005)
+    O.oracle_fill_normal_bf16(ptr(b), b.size, 2005)
+    return a.reshape(m, k), b.reshape(k, n)
+
+
+@pytest.mark.parametrize("shape", [(128, 128, 64), (256, 384, 192), (512, 512, 512)])
+def test_gemm_small(device, shape):
+    m, n, k = shape
+    a, b = _bf16_inputs(m, n, k)
+    want = np.empty((m, n), dtype=np.float32)
+    ol.load().oracle_gemm_bf16(ptr(a), ptr(b), ptr(want), m, n, k)
+    d_a = torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
+    d_b = torch.from_numpy(b.view(np.int16)).to(device).view(torch.bfloat16)
+    d_c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
+    print(f"gemm {shape}", flush=True)
+    wl.gemm_bf16(d_a, d_b, d_c)
+    torch.cuda.synchronize()
+    got = d_c.cpu().numpy()
+    scale = np.sqrt(k)                      # typical magnitude of an entry
+    assert np.all(np.abs(got - want) <= GEMM_RTOL * np.maximum(np.abs(want), scale)), \
+        float(np.max(np.abs(got - want)))
+    # much tighter in practice: both sides accumulate the same exact bf16 products in fp32
+    assert float(np.max(np.abs(got - want))) <= 1e-4 * scale * np.sqrt(k)
+
+
+def test_gemm_full_size(device):
+    m = n = k = 4096
+    a, b = _bf16_inputs(m, n, k)
+    d_a = torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
+    d_b = torch.from_numpy(b.view(np.int16)).to(device).view(torch.bfloat16)
+    d_c = torch.empty((m, n), dtype=torch.float32, device=device)
+    wl.gemm_bf16(d_a, d_b, d_c)
+    torch.cuda.synchronize()
+    got = d_c.cpu().numpy()
+    O = ol.load()
+    rng = np.random.default_rng(5)
+    for row, col in zip(rng.integers(0, m, 400), rng.integers(0, n, 400)):
+        want = O.oracle_gemm_bf16_entry(ptr(a), ptr(b), n, k, int(row), int(col))
+        assert abs(got[row, col] - want) <= GEMM_RTOL * max(abs(want), 64.0)
+    # every tile against the matrix cores' own library path on the same bits
+    ref = torch.matmul(d_a.float(), d_b.float())
+    assert float((d_c - ref).abs().max()) <= 1e-2 * 64.0
+
+
+def test_gemm_rejects_ragged_shapes(device):
+    a = torch.zeros((100, 64), dtype=torch.bfloat16, device=device)
+    b = torch.zeros((64, 128), dtype=torch.bfloat16, device=device)
+    c = torch.zeros((100, 128), dtype=torch.float32, device=device)
+    with pytest.raises(cd.CudaDMAError, match="multiples"):
+        wl.gemm_bf16(a, b, c)
