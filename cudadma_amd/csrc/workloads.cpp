@@ -77,8 +77,8 @@ static const VariantInfo kHalo[] = {
 };
 
 static const VariantInfo kGemm[] = {
-  {"warp-specialised: one DMA wavefront per operand (CudaDMAStrided, two LDS stages behind one object), four compute "
-   "wavefronts with v_mfma_f32_32x32x16_bf16, B fragments through ds_read_b64_tr_b16"},
+  {"warp-specialised: one DMA wavefront per operand with two CudaDMAStrided objects (two LDS stages, tile two K steps "
+   "ahead in flight), four compute wavefronts with v_mfma_f32_32x32x16_bf16, B fragments through ds_read_b64_tr_b16"},
 };
 
 static const VariantInfo* table(int workload, int* count)

@@ -174,7 +174,7 @@ int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz
 
 /* Config 5 (no GEMM in the reference; nearest: src/examples/sgemv/sgemv_dma.cu:329-388):
  * C = A * B with A m x k and B k x n row-major bf16 (as uint16 bit patterns), C m x n
- * float, fp32 accumulation on the matrix cores.  m, n multiples of 128, k of 64.
+ * float, fp32 accumulation on the matrix cores.  m, n and k multiples of 128.
  * DMA wavefronts stage 128 x 64 tiles of A and 64 x 128 tiles of B through CudaDMAStrided. */
 int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k,
                       int variant, void* stream);

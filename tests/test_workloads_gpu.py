@@ -202,7 +202,7 @@ def _bf16_inputs(m, n, k):
     return a.reshape(m, k), b.reshape(k, n)
 
 
-@pytest.mark.parametrize("shape", [(128, 128, 64), (256, 384, 192), (512, 512, 512)])
+@pytest.mark.parametrize("shape", [(128, 128, 128), (256, 384, 256), (512, 512, 512)])
 def test_gemm_small(device, shape):
     m, n, k = shape
     a, b = _bf16_inputs(m, n, k)
@@ -242,8 +242,8 @@ def test_gemm_full_size(device):
 
 
 def test_gemm_rejects_ragged_shapes(device):
-    a = torch.zeros((100, 64), dtype=torch.bfloat16, device=device)
-    b = torch.zeros((64, 128), dtype=torch.bfloat16, device=device)
+    a = torch.zeros((100, 128), dtype=torch.bfloat16, device=device)
+    b = torch.zeros((128, 128), dtype=torch.bfloat16, device=device)
     c = torch.zeros((100, 128), dtype=torch.float32, device=device)
     with pytest.raises(cd.CudaDMAError, match="multiples"):
         wl.gemm_bf16(a, b, c)
