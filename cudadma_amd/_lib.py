@@ -45,6 +45,7 @@ class RunArgs(ctypes.Structure):
         ("src_stride", ctypes.c_int), ("dst_stride", ctypes.c_int), ("pitch", ctypes.c_int),
         ("call_style", ctypes.c_int), ("two_phase", ctypes.c_int), ("reps", ctypes.c_int),
         ("rep_src_bytes", ctypes.c_int), ("rep_index_elmts", ctypes.c_int),
+        ("reverse", ctypes.c_int), ("out_bytes", ctypes.c_int),
     ]
 
 
@@ -107,6 +108,7 @@ _WORKLOAD_SIGNATURES = {
     "cudadma_gather_rowsum": [_vp, _vp, _vp, _cs, _cs, _ci, _vp],
     "cudadma_halo_stencil": [_vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cudadma_gemm_bf16": [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
+    "cudadma_selftest_bounded_wait": [_vp, _vp],
 }
 
 

@@ -89,6 +89,12 @@ extern "C" int cudadma_run_case(int case_id, const cudadma_run_t* run, void* str
     CUDADMA_REQUIRE(run->call_style != CUDADMA_CALL_LDS_DIRECT, "scatter has no direct path");
   if (run->call_style == CUDADMA_CALL_LDS_DIRECT)
     CUDADMA_REQUIRE(d.alignment == 16 || d.alignment == 4, "the direct path moves 4 or 16 bytes per lane");
+  if (run->reverse) {
+    CUDADMA_REQUIRE(run->call_style == CUDADMA_CALL_UNQUALIFIED,
+                    "LDS -> global transfers go through the unqualified (generic-pointer) calls");
+    CUDADMA_REQUIRE(run->out_bytes > 0 && (run->out_bytes % 16) == 0, "out_bytes must be a positive multiple of 16");
+    CUDADMA_REQUIRE((run->rep_src_bytes % 4) == 0, "rep_src_bytes must be a multiple of 4");
+  }
 
   harness::Args a;
   a.in = (const char*)run->d_in;
@@ -105,6 +111,8 @@ extern "C" int cudadma_run_case(int case_id, const cudadma_run_t* run, void* str
   a.reps = run->reps;
   a.rep_src_bytes = run->rep_src_bytes;
   a.rep_index_elmts = run->rep_index_elmts;
+  a.reverse = run->reverse ? 1 : 0;
+  a.out_bytes = run->out_bytes;
   a.bytes_per_elmt = d.bytes_per_elmt;
   a.dma_threads = d.dma_threads;
   a.num_elmts = d.num_elmts;

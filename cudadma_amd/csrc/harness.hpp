@@ -25,6 +25,7 @@ struct Args {
   int pitch;
   int call_style, two_phase;
   int reps, rep_src_bytes, rep_index_elmts;
+  int reverse, out_bytes;
   // run-time copies of the template parameters, fed to the constructors of the lower levels
   int bytes_per_elmt, dma_threads, num_elmts, dimx, dimy;
 };
@@ -101,29 +102,54 @@ __device__ __forceinline__ void copy_out(const unsigned* buf, unsigned* out, con
   for (int i = tid; i < words; i += nthreads) out[i] = buf[i];
 }
 
-// Body shared by every case.  `xfer(rep)` performs one transfer (DMA threads).
+__device__ __forceinline__ void fill_lds(unsigned* buf, const unsigned* in, const int words, const int tid,
+                                         const int nthreads)
+{
+  for (int i = tid; i < words; i += nthreads) buf[i] = in[i];
+}
+
+// Body shared by every case.  `xfer(rep)` performs one transfer (DMA threads); it has exactly
+// one call site per kernel shape so that it is inlined and the object stays in registers.
+// Forward: the compute side clears LDS, releases it, waits for the transfer, copies LDS out.
+// Reverse (LDS is the source): the compute side loads the image into LDS and waits until the DMA
+// side has moved it out to global memory.  The objects issue their loads before the handshake
+// wait (the source is assumed ready, as in the reference), so the compute side signals twice:
+// the first signal says "the image is in LDS" and is consumed by an explicit
+// wait_for_dma_start() ahead of the transfer, the second is the one the transfer itself waits for.
 template<bool WS, typename Obj, typename Xfer>
 __device__ __forceinline__ void run_body(Obj& dma, const Args& a, unsigned* lds, Xfer xfer)
 {
   const int words = a.lds_bytes / 4;
   if constexpr (WS) {
     if (dma.owns_this_thread()) {
-      for (int rep = 0; rep < a.reps; ++rep) xfer(rep);
+      for (int rep = 0; rep < a.reps; ++rep) {
+        if (a.reverse) dma.wait_for_dma_start();
+        xfer(rep);
+      }
     } else if (threadIdx.x < kComputeThreads) {
       for (int rep = 0; rep < a.reps; ++rep) {
-        clear_lds(lds, words, threadIdx.x, kComputeThreads);
+        if (a.reverse)
+          fill_lds(lds, (const unsigned*)(a.in + (size_t)rep * a.rep_src_bytes), words, threadIdx.x, kComputeThreads);
+        else
+          clear_lds(lds, words, threadIdx.x, kComputeThreads);
+        if (a.reverse) dma.start_async_dma();
         dma.start_async_dma();
         dma.wait_for_dma_finish();
-        copy_out(lds, (unsigned*)(a.out + (size_t)rep * a.lds_bytes), words, threadIdx.x, kComputeThreads);
+        if (!a.reverse)
+          copy_out(lds, (unsigned*)(a.out + (size_t)rep * a.lds_bytes), words, threadIdx.x, kComputeThreads);
       }
     }
   } else {
     for (int rep = 0; rep < a.reps; ++rep) {
-      clear_lds(lds, words, threadIdx.x, blockDim.x);
+      if (a.reverse)
+        fill_lds(lds, (const unsigned*)(a.in + (size_t)rep * a.rep_src_bytes), words, threadIdx.x, blockDim.x);
+      else
+        clear_lds(lds, words, threadIdx.x, blockDim.x);
       __syncthreads();
       xfer(rep);
       __syncthreads();
-      copy_out(lds, (unsigned*)(a.out + (size_t)rep * a.lds_bytes), words, threadIdx.x, blockDim.x);
+      if (!a.reverse)
+        copy_out(lds, (unsigned*)(a.out + (size_t)rep * a.lds_bytes), words, threadIdx.x, blockDim.x);
       __syncthreads();
     }
   }

@@ -53,9 +53,11 @@ __global__ void __launch_bounds__(1024) halo_kernel(const Args a)
 {
   extern __shared__ __attribute__((aligned(16))) unsigned lds[];
   auto dma = Make<WS, LEVEL, A, BPT, ES, T, R, C, DX, DY>::make(a);
-  harness::run_body<WS>(dma, a, lds, [&](const int rep) {
-    const char* src = a.in + a.src_offset + (size_t)rep * a.rep_src_bytes + (size_t)(R * a.pitch + R) * ES;
-    char* dst = (char*)lds + a.dst_offset + (size_t)(R * (a.dimx + 2 * R) + R) * ES;
+  harness::run_body<WS>(dma, a, lds, [&](const int rep) __attribute__((always_inline)) {
+    const char* src = (a.reverse ? (const char*)lds + a.src_offset : a.in + a.src_offset + (size_t)rep * a.rep_src_bytes) +
+                      (size_t)(R * a.pitch + R) * ES;
+    char* dst = (a.reverse ? a.out + (size_t)rep * a.out_bytes + a.dst_offset : (char*)lds + a.dst_offset) +
+                (size_t)(R * (a.dimx + 2 * R) + R) * ES;
     harness::do_transfer(dma, a.call_style, a.two_phase, src, dst);
   });
 }

@@ -54,10 +54,10 @@ __global__ void __launch_bounds__(1024) indirect_kernel(const Args a)
 {
   extern __shared__ __attribute__((aligned(16))) unsigned lds[];
   auto dma = Make<G, WS, LEVEL, A, BPT, E, T, N>::make(a);
-  harness::run_body<WS>(dma, a, lds, [&](const int rep) {
-    const char* src = a.in + a.src_offset + (size_t)rep * a.rep_src_bytes;
+  harness::run_body<WS>(dma, a, lds, [&](const int rep) __attribute__((always_inline)) {
+    const char* src = a.reverse ? (const char*)lds + a.src_offset : a.in + a.src_offset + (size_t)rep * a.rep_src_bytes;
     const int* index = a.index + (size_t)rep * a.rep_index_elmts;
-    char* dst = (char*)lds + a.dst_offset;
+    char* dst = a.reverse ? a.out + (size_t)rep * a.out_bytes + a.dst_offset : (char*)lds + a.dst_offset;
     if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
       if constexpr (G && (A == 16 || A == 4)) {
         if (a.two_phase) {

@@ -80,9 +80,9 @@ __global__ void __launch_bounds__(1024) strided_kernel(const Args a)
 {
   extern __shared__ __attribute__((aligned(16))) unsigned lds[];
   auto dma = Make<WS, LEVEL, ONE, A, BPT, E, T, N>::make(a);
-  harness::run_body<WS>(dma, a, lds, [&](const int rep) {
-    const char* src = a.in + a.src_offset + (size_t)rep * a.rep_src_bytes;
-    char* dst = (char*)lds + a.dst_offset;
+  harness::run_body<WS>(dma, a, lds, [&](const int rep) __attribute__((always_inline)) {
+    const char* src = a.reverse ? (const char*)lds + a.src_offset : a.in + a.src_offset + (size_t)rep * a.rep_src_bytes;
+    char* dst = a.reverse ? a.out + (size_t)rep * a.out_bytes + a.dst_offset : (char*)lds + a.dst_offset;
     if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
       if constexpr (A == 16 || A == 4) harness::do_transfer_direct(dma, a.two_phase, src, dst);
     } else {

@@ -1,0 +1,102 @@
+"""Parameter sweep over the benchmark workloads: every buffering variant x workgroups per
+compute unit, timed with HIP events.  The counterpart of the reference's
+src/perf/sequential/param_sweep.py:27-58, which rewrites params_directed.h and recompiles per
+point; here the variants are compiled in and the occupancy is a run-time knob.
+
+    python -m cudadma_amd.sweep [sequential] [strided] [gather] [halo] [gemm] [--wg 0,2,4,8] [--steps 20]
+"""
+import argparse
+import sys
+
+import torch
+
+from . import workloads as wl
+
+PEAK_GBS = 8000.0
+
+
+def _time(fn, steps, warmup=3):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a = torch.cuda.Event(enable_timing=True)
+    b = torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(steps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / steps
+
+
+def _row(name, variant, wg, ms, nbytes):
+    gbs = nbytes / ms / 1e6
+    print(f"{name:10s} variant {variant}  wg/cu {wg:2d}  {ms:9.4f} ms  {gbs:8.0f} GB/s  {100 * gbs / PEAK_GBS:5.1f}%", flush=True)
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("workloads", nargs="*", default=["sequential", "strided", "gather", "halo", "gemm"])
+    ap.add_argument("--wg", default="0,2,4,8", help="workgroups per compute unit to try (0 = each kernel's default)")
+    ap.add_argument("--steps", type=int, default=20)
+    args = ap.parse_args(argv)
+    if not torch.cuda.is_available():
+        sys.exit("no GPU visible")
+    dev = torch.device("cuda:0")
+    wgs = [int(x) for x in args.wg.split(",")]
+    for name in args.workloads:
+        if name == "sequential":
+            src = wl.fill_uniform(torch.empty(16 << 20, device=dev), 1001)
+            dst = torch.empty_like(src)
+            for v in range(wl.num_variants(wl.SEQUENTIAL)):
+                print(f"# sequential variant {v}: {wl.variant_name(wl.SEQUENTIAL, v)}")
+                for wg in wgs:
+                    wl.set_workgroups_per_cu(wg)
+                    _row(name, v, wg, _time(lambda: wl.sequential_copy(src, dst, v), max(args.steps, 50)), 2 * src.numel() * 4)
+        elif name == "strided":
+            n = 16384
+            src = wl.fill_uniform(torch.empty(n * n, device=dev), 1002).view(n, n)
+            dst = torch.empty_like(src)
+            for v in range(wl.num_variants(wl.STRIDED)):
+                print(f"# strided variant {v}: {wl.variant_name(wl.STRIDED, v)}")
+                for wg in wgs:
+                    wl.set_workgroups_per_cu(wg)
+                    _row(name, v, wg, _time(lambda: wl.strided_transpose(src, dst, v), args.steps), 2 * n * n * 4)
+        elif name == "gather":
+            recs, n_idx = 4 << 20, 32 << 20
+            table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1003)
+            idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=dev), recs, 1003)
+            out = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, device=dev)
+            for v in range(wl.num_variants(wl.GATHER)):
+                print(f"# gather (row-sum) variant {v}: {wl.variant_name(wl.GATHER, v)}")
+                for wg in wgs:
+                    wl.set_workgroups_per_cu(wg)
+                    _row(name, v, wg, _time(lambda: wl.gather_rowsum(table, idx, out, v), args.steps),
+                         n_idx * 132 + out.numel() * 4)
+        elif name == "halo":
+            g = 512
+            gi = wl.fill_uniform(torch.empty((g + 8) ** 3, device=dev), 1004).view(g + 8, g + 8, g + 8)
+            go = torch.empty(g, g, g, device=dev)
+            for v in range(wl.num_variants(wl.HALO)):
+                print(f"# halo variant {v}: {wl.variant_name(wl.HALO, v)}")
+                for zc in (0, 128, 256, 512):
+                    wl.set_tuning("stencil_zchunk", zc)
+                    ms = _time(lambda: wl.halo_stencil(gi, go, v), args.steps)
+                    gbs = 2 * g ** 3 * 4 / ms / 1e6
+                    print(f"{name:10s} variant {v}  zchunk {zc:3d}  {ms:9.4f} ms  {gbs:8.0f} GB/s  {100 * gbs / PEAK_GBS:5.1f}%",
+                          flush=True)
+            wl.set_tuning("stencil_zchunk", 0)
+        elif name == "gemm":
+            n = 4096
+            a = torch.randn(n, n, device=dev).to(torch.bfloat16)
+            b = torch.randn(n, n, device=dev).to(torch.bfloat16)
+            c = torch.empty(n, n, device=dev)
+            ms = _time(lambda: wl.gemm_bf16(a, b, c), args.steps)
+            print(f"gemm       variant 0  {ms:9.4f} ms  {2.0 * n ** 3 / ms / 1e9:8.1f} TFLOP/s", flush=True)
+        else:
+            sys.exit(f"unknown workload {name}")
+    wl.set_workgroups_per_cu(0)
+
+
+if __name__ == "__main__":
+    main()

@@ -81,11 +81,23 @@ typedef struct cudadma_run {
   int reps;               /* transfers run back to back through the same LDS buffer   */
   int rep_src_bytes;      /* source advance per rep                                   */
   int rep_index_elmts;    /* index advance per rep                                    */
+  int reverse;            /* 1: the object moves LDS -> global.  The workgroup first copies
+                             lds_bytes from d_in (+ rep * rep_src_bytes) into LDS, the object then
+                             moves from LDS + src_offset_bytes to d_out + rep * out_bytes +
+                             dst_offset_bytes.  Only CUDADMA_CALL_UNQUALIFIED (generic pointers on
+                             both sides, include/cudaDMAv2.h:107-114,553-558) makes sense here.   */
+  int out_bytes;          /* reverse only: bytes of d_out one rep may touch            */
 } cudadma_run_t;
 
 int cudadma_num_cases(void);
 int cudadma_get_case(int case_id, cudadma_case_t* out);
 int cudadma_run_case(int case_id, const cudadma_run_t* run, void* stream);
+
+/* Failure handling of the handshake (the reference deadlocks on unbalanced calls,
+ * include/cudaDMAv2.h:1329-1347): launches one workgroup whose DMA and compute threads wait for
+ * signals that never come, with the poll limit lowered to 256.  Both sides must give up and the
+ * kernel must end; d_flags[0] (DMA side) and d_flags[1] (compute side) are then 1. */
+int cudadma_selftest_bounded_wait(int* d_flags, void* stream);
 
 /* ------------------------------------------------------------------------
  * Host-side planner.  cudadma_diagnose prints what the static diagnose()

@@ -14,9 +14,10 @@ def _round_up(v, m):
 class CaseIO:
     """Everything one run of a case needs, plus what the LDS buffer must hold afterwards."""
 
-    def __init__(self, case, flavour=0, reps=2, data="ramp"):
+    def __init__(self, case, flavour=0, reps=2, data="ramp", reverse=False):
         self.case = case
         self.reps = reps
+        self.reverse = reverse
         a = case.alignment
         rng = np.random.default_rng(1000 * case.pattern + 17 * flavour + case.bytes_per_elmt + case.dma_threads)
         self.index = None
@@ -28,33 +29,32 @@ class CaseIO:
         pat = case.pattern
         e, n = case.bytes_per_elmt, case.num_elmts
         if pat == cd.PATTERN_SEQUENTIAL:
-            footprint_src = e
-            self.lds_bytes = _round_up(self.dst_offset + e + 16, 16)
+            footprint_src = footprint_dst = e
         elif pat == cd.PATTERN_STRIDED:
             one_stride = case.dimx == 1
             self.src_stride = _round_up(e, a) + a * (2 + flavour % 2)
             self.dst_stride = self.src_stride if one_stride else _round_up(e, a) + a * (flavour % 2)
             footprint_src = n * self.src_stride
-            self.lds_bytes = _round_up(self.dst_offset + n * self.dst_stride + 16, 16)
+            footprint_dst = n * self.dst_stride
         elif pat == cd.PATTERN_GATHER:
-            self.table_elmts = 2 * n + 3
+            self.table_elmts = (n + 3) if reverse else (2 * n + 3)   # the table sits in LDS when reversed
             alt = 0 if flavour % 2 == 0 else e + a
             self.dst_stride = alt
             footprint_src = self.table_elmts * e
+            footprint_dst = n * max(alt, e)
             self.rep_src_bytes = 0
             self.rep_index_elmts = n
             idx = rng.integers(0, self.table_elmts, size=reps * n).astype(np.int32)
             idx[1::5] = idx[0]                                   # duplicates
             self.index = idx
-            self.lds_bytes = _round_up(self.dst_offset + n * max(alt, e) + 16, 16)
         elif pat == cd.PATTERN_SCATTER:
-            self.table_elmts = n + 3                              # elements the LDS side can hold
+            self.table_elmts = n + 3                              # elements the sparse side holds
             alt = 0 if flavour % 2 == 0 else e + a
             self.src_stride = alt
             footprint_src = n * max(alt, e)
+            footprint_dst = self.table_elmts * e
             self.rep_index_elmts = n
             self.index = np.concatenate([rng.permutation(self.table_elmts)[:n] for _ in range(reps)]).astype(np.int32)
-            self.lds_bytes = _round_up(self.dst_offset + self.table_elmts * e + 16, 16)
         elif pat == cd.PATTERN_HALO:
             r, dimx, dimy = case.radius, case.dimx, case.dimy
             unit = max(1, a // e)
@@ -65,10 +65,18 @@ class CaseIO:
             self.dst_offset = (-dst_origin) % a
             self.rep_src_bytes = a
             footprint_src = (dimy + 2 * r) * self.pitch * e
-            self.lds_bytes = _round_up(self.dst_offset + (dimx + 2 * r) * (dimy + 2 * r) * e + 16, 16)
+            footprint_dst = (dimx + 2 * r) * (dimy + 2 * r) * e
         else:
             raise ValueError(pat)
-        in_bytes = _round_up(self.src_offset + footprint_src + reps * self.rep_src_bytes + 64, 16)
+        if reverse:
+            # LDS holds the source image, the destination is a window of global memory
+            self.lds_bytes = _round_up(self.src_offset + footprint_src + 16, 16)
+            self.out_bytes = _round_up(self.dst_offset + footprint_dst + 16, 16)
+            in_bytes = _round_up(self.lds_bytes + reps * self.rep_src_bytes + 64, 16)
+        else:
+            self.lds_bytes = _round_up(self.dst_offset + footprint_dst + 16, 16)
+            self.out_bytes = 0
+            in_bytes = _round_up(self.src_offset + footprint_src + reps * self.rep_src_bytes + 64, 16)
         if data == "ramp":
             # the reference tests' input: h_idata[i] = float(i)
             self.input = ol.ramp(in_bytes // 4).view(np.uint8)
@@ -76,12 +84,12 @@ class CaseIO:
             self.input = ol.uniform(in_bytes // 4, 4242 + flavour).view(np.uint8)
 
     # -- the closed form, applied by the oracle to byte buffers -------------------------------
-    def apply_oracle(self, src, dst, rep):
+    def apply_oracle(self, src, dst, rep, shift_src=True):
         """Moves what the case's object moves: src/dst are numpy uint8 arrays standing for
-        the input buffer and one LDS buffer."""
+        the source and the destination buffer of one transfer."""
         O = ol.load()
         c = self.case
-        so = self.src_offset + rep * self.rep_src_bytes
+        so = self.src_offset + (rep * self.rep_src_bytes if shift_src else 0)
         do = self.dst_offset
         e, n = c.bytes_per_elmt, c.num_elmts
         idx = self.index[rep * self.rep_index_elmts:] if self.index is not None else None
@@ -99,6 +107,12 @@ class CaseIO:
                           e, r, c.corners, c.dimx, c.dimy, self.pitch)
 
     def expected(self):
+        if self.reverse:
+            out = np.zeros((self.reps, self.out_bytes), dtype=np.uint8)
+            for rep in range(self.reps):
+                image = np.ascontiguousarray(self.input[rep * self.rep_src_bytes:rep * self.rep_src_bytes + self.lds_bytes])
+                self.apply_oracle(image, out[rep], rep, shift_src=False)
+            return out
         out = np.zeros((self.reps, self.lds_bytes), dtype=np.uint8)
         for rep in range(self.reps):
             self.apply_oracle(self.input, out[rep], rep)

@@ -51,6 +51,33 @@ def test_case_matches_oracle(case_id, device):
                         f"{bad[0][0]} byte {bad[0][1]} (got {got[tuple(bad[0])]}, want {want[tuple(bad[0])]})")
 
 
+@pytest.mark.parametrize("case_id", range(len(_CASES)), ids=[case_id_str(i, c) for i, c in enumerate(_CASES)])
+def test_case_reverse_direction_matches_oracle(case_id, device):
+    """The same objects moving LDS -> global through the generic-pointer calls: the reference's
+    ld/st wrappers are direction-agnostic (include/cudaDMAv2.h:107-114,553-558), its tests never try it."""
+    case = _CASES[case_id]
+    for flavour, two_phase in ((0, False), (1, True)):
+        io = CaseIO(case, flavour=flavour, reps=2, data="uniform", reverse=True)
+        if io.lds_bytes > 64 * 1024 - 256:
+            pytest.skip("source image does not fit the harness LDS window")
+        want = io.expected()
+        d_in = torch.from_numpy(io.input).to(device)
+        d_idx = torch.from_numpy(io.index).to(device) if io.index is not None else None
+        d_out = torch.zeros(io.reps * io.out_bytes, dtype=torch.uint8, device=device)
+        print(f"reverse case {case_id} two_phase {two_phase} {case}", flush=True)
+        cd.harness.run_case(case_id, d_in, d_out, lds_bytes=io.lds_bytes, d_index=d_idx,
+                            src_offset_bytes=io.src_offset, dst_offset_bytes=io.dst_offset,
+                            src_stride=io.src_stride, dst_stride=io.dst_stride, pitch=io.pitch,
+                            call_style=cd.CALL_UNQUALIFIED, two_phase=two_phase, reps=io.reps,
+                            rep_src_bytes=io.rep_src_bytes, rep_index_elmts=io.rep_index_elmts,
+                            reverse=True, out_bytes=io.out_bytes)
+        torch.cuda.synchronize()
+        got = d_out.cpu().numpy().reshape(io.reps, io.out_bytes)
+        if not np.array_equal(got, want):
+            bad = np.argwhere(got != want)
+            raise AssertionError(f"two_phase {two_phase}: {len(bad)} wrong bytes, first at rep {bad[0][0]} byte {bad[0][1]}")
+
+
 def test_halo_case_passes_the_reference_checker(device):
     """check_halo of the reference on the GPU output of the cudaDMAHalo (older interface) cases."""
     from tests import oracle_lib as ol
@@ -71,3 +98,13 @@ def test_halo_case_passes_the_reference_checker(device):
                                    case.radius, case.corners, case.dimx, case.dimy, io.pitch) == 1
         ran += 1
     assert ran >= 4
+
+
+def test_unmatched_waits_end(device):
+    """Unbalanced start_async_dma / finish_async_dma counts must not hang the GPU: with the poll limit
+    forced down from the host side both waits give up and the kernel finishes."""
+    import ctypes
+    flags = torch.zeros(2, dtype=torch.int32, device=device)
+    cd._lib.check(cd.lib().cudadma_selftest_bounded_wait(ctypes.c_void_p(flags.data_ptr()), None))
+    torch.cuda.synchronize()
+    assert flags.tolist() == [1, 1]
