@@ -45,6 +45,8 @@ def sequential_cases():
         (1, 2, 16, 64, 1024 + 4, 64), (1, 1, 16, 64, 1024 + 8, 64), (0, 3, 16, 64, 1024 + 12, 64),
         (0, 1, 8, 16, 8 * 64 * 2 + 4, 64), (0, 2, 4, 4, 4 * 64 * 3, 64),
         (1, 3, 4, 32, 36860, 192), (0, 3, 8, 64, 40000, 960),
+        (1, 1, 16, 64, 0, 64), (0, 1, 4, 16, 0, 128),            # empty transfer (run-time size 0)
+        (1, 3, 16, 128, 64000, 128), (0, 2, 16, 256, 65200, 256),  # as large as the LDS window allows
     ]
     for c in directed:
         out.append(c)
@@ -75,6 +77,8 @@ def grid_cases(seed, n_random, with_gather):
         (0, 2, 8, 8, 1000, 128, 9), (0, 1, 4, 4, 132, 192, 31),
         (1, 4, 16, 128, 1040, 256, 16),   # 65 loads per row: two wavefront loads per row, half idle
         (0, 3, 16, 64, 512, 960, 32),     # more threads than slots
+        (1, 1, 16, 64, 256, 64, 0), (0, 3, 8, 32, 64, 128, 0),   # no elements (run-time count 0)
+        (1, 4, 16, 128, 16000, 256, 4),   # four rows that fill the LDS window
     ]
     for c in directed:
         out.append(c)
@@ -141,7 +145,8 @@ def main():
     write("cases_strided.inc",
           [f"STRIDED_CASE({i}, {bool_s(ws)}, {lv}, {bool_s(i % 4 == 3)}, {a}, {bpt}, {e}, {t}, {n})"
            for i, (ws, lv, a, bpt, e, t, n) in enumerate(strided)])
-    ind = grid_cases(977, 32, True)
+    # the sparse side of an indirect transfer holds n + 3 elements in the tests: it has to fit LDS
+    ind = [c for c in grid_cases(977, 32, True) if (c[6] + 3) * c[4] <= 60000]
     lines = []
     for i, (ws, lv, a, bpt, e, t, n) in enumerate(ind):
         gather = (i % 3) != 2          # two thirds gather, one third scatter

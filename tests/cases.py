@@ -44,8 +44,9 @@ class CaseIO:
             footprint_dst = n * max(alt, e)
             self.rep_src_bytes = 0
             self.rep_index_elmts = n
-            idx = rng.integers(0, self.table_elmts, size=reps * n).astype(np.int32)
-            idx[1::5] = idx[0]                                   # duplicates
+            idx = rng.integers(0, self.table_elmts, size=max(1, reps * n)).astype(np.int32)
+            if idx.size:
+                idx[1::5] = idx[0]                               # duplicates
             self.index = idx
         elif pat == cd.PATTERN_SCATTER:
             self.table_elmts = n + 3                              # elements the sparse side holds
@@ -55,6 +56,8 @@ class CaseIO:
             footprint_dst = self.table_elmts * e
             self.rep_index_elmts = n
             self.index = np.concatenate([rng.permutation(self.table_elmts)[:n] for _ in range(reps)]).astype(np.int32)
+            if self.index.size == 0:
+                self.index = np.zeros(1, dtype=np.int32)         # a valid pointer for an empty index list
         elif pat == cd.PATTERN_HALO:
             r, dimx, dimy = case.radius, case.dimx, case.dimy
             unit = max(1, a // e)

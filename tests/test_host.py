@@ -42,6 +42,7 @@ def test_case_table_is_sane():
         assert c.alignment in (4, 8, 16)
         assert c.bytes_per_thread % c.alignment == 0 and c.bytes_per_thread > 0
         assert c.dma_threads % 64 == 0 and 64 <= c.dma_threads <= 960
+        assert c.bytes_per_elmt % 4 == 0 and c.bytes_per_elmt >= 0
     # every constructor form is compiled: each (pattern, warp_specialized, level) combination exists
     seen = {(c.pattern, c.warp_specialized, c.level) for c in cases}
     for p, levels in ((0, (1, 2, 3)), (1, (1, 2, 3, 4)), (2, (1, 2, 3, 4)), (4, (1, 2, 3))):
@@ -114,7 +115,7 @@ def test_replay_of_every_compiled_case_matches_the_oracle(case_id):
         else:
             assert doubles == 0, f"{doubles} bytes written twice"
         assert np.array_equal(got, want)
-        assert steps >= 1
+        assert steps >= (1 if want.size and (want >= 0).any() else 0)
 
 
 def test_replay_on_random_parameters():
