@@ -23,4 +23,4 @@ from ._lib import (  # noqa: F401
     lib,
     lib_path,
 )
-from . import harness, plan, workloads  # noqa: F401
+from . import examples, harness, plan, workloads  # noqa: F401

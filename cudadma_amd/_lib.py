@@ -89,6 +89,8 @@ def lib():
     L.cudadma_set_tuning.argtypes = [ctypes.c_char_p, ci]
     L.cudadma_variant_name.restype = ctypes.c_char_p
     L.cudadma_variant_name.argtypes = [ci, ci]
+    L.cudadma_example_variant_name.restype = ctypes.c_char_p
+    L.cudadma_example_variant_name.argtypes = [ci, ci]
     _lib = L
     return L
 
@@ -109,6 +111,10 @@ _WORKLOAD_SIGNATURES = {
     "cudadma_halo_stencil": [_vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cudadma_gemm_bf16": [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cudadma_selftest_bounded_wait": [_vp, _vp],
+    "cudadma_example_num_variants": [_ci],
+    "cudadma_example_saxpy": [_ci, ctypes.c_float, _vp, _vp, ctypes.c_longlong, _vp],
+    "cudadma_example_sgemv": [_ci, _ci, _ci, ctypes.c_float, _vp, _ci, _vp, _vp, _vp],
+    "cudadma_example_stencil2d": [_ci, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
 }
 
 
@@ -120,4 +126,4 @@ def check(rc):
 def exported_symbols():
     """Every extern "C" symbol include/cudadma_amd.h declares."""
     return ["cudadma_last_error", "cudadma_device_cus", "cudadma_num_cases", "cudadma_get_case",
-            "cudadma_run_case", "cudadma_variant_name", "cudadma_plan_map", "cudadma_diagnose", "cudadma_set_tuning"] + list(_WORKLOAD_SIGNATURES)
+            "cudadma_run_case", "cudadma_variant_name", "cudadma_example_variant_name", "cudadma_plan_map", "cudadma_diagnose", "cudadma_set_tuning"] + list(_WORKLOAD_SIGNATURES)

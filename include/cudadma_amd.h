@@ -191,6 +191,42 @@ int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz
 int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k,
                       int variant, void* stream);
 
+/* ---- the reference's example programs on the wave64 objects --------------------------
+ * The kernels behind these are written against the DMA classes alone (the first-
+ * generation names of include/cudaDMA.h for saxpy and sgemv, the current ones for the
+ * stencil); the reference has them as stand-alone programs with compile-time sizes,
+ * here sizes are arguments and the launch geometry is fixed per example. */
+enum {
+  CUDADMA_EXAMPLE_SAXPY     = 0,
+  CUDADMA_EXAMPLE_SGEMV     = 1,
+  CUDADMA_EXAMPLE_STENCIL2D = 2
+};
+int cudadma_example_num_variants(int example);
+const char* cudadma_example_variant_name(int example, int variant);
+
+/* y = a*x + y in place, one fused multiply-add per element
+ * (src/examples/saxpy/saxpy_cudaDMA_kernel.cu:55-61, :270-315, :322-418; driver
+ * saxpy_cudaDMA.cu:76-175).  Variants 0/1 use no DMA object, 2/3 stage x and y through
+ * LDS with cudaDMASequential.  n a multiple of 1024 floats except for variant 0. */
+int cudadma_example_saxpy(int variant, float a, const float* d_x, float* d_y, long long n, void* stream);
+
+/* y = alpha * A x, A column-major n x m with leading dimension lda, accumulated in
+ * ascending column order with fused multiply-add (src/examples/sgemv/sgemv_dma.cu:140-175,
+ * :262-325, :329-388, :392-470; host check :752-771).  m a multiple of 256 (variant 0),
+ * 512 (variant 1) or 32 (variants 2, 3, which also need lda >= n rounded up to 128 and
+ * 16-byte aligned columns). */
+int cudadma_example_sgemv(int variant, int n, int m, float alpha, const float* d_a, int lda, const float* d_x,
+                          float* d_y, void* stream);
+
+/* The 2-D cross average of every z slice of a float2 volume in its five buffering
+ * styles (src/examples/stencil/cudaDMA_stencil2D.cu:99-204, stencil_math.h:27-87).
+ * d_src and d_dst hold (dimx+8) x (dimy+8) x (dimz+8) float2 elements (radius 4 padding on
+ * every side, x fastest); only interior points of d_dst are written.  full_cross = 0
+ * sums three neighbours per arm as the reference's loops do, 1 sums all four; the divisor
+ * is 17 either way.  dimx a multiple of 32, dimy of 4; dimz even for variants 1, 2, 4. */
+int cudadma_example_stencil2d(int variant, const float* d_src, float* d_dst, int dimx, int dimy, int dimz,
+                              int full_cross, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

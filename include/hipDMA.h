@@ -23,3 +23,4 @@
 #include "hipdma/strided.hpp"
 #include "hipdma/indirect.hpp"
 #include "hipdma/halo.hpp"
+#include "hipdma/v1.hpp"

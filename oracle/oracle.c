@@ -289,3 +289,56 @@ float oracle_gemm_bf16_entry(const uint16_t* a, const uint16_t* b, int n, int k,
     acc += oracle_bf16_to_f32(a[(size_t)row * k + kk]) * oracle_bf16_to_f32(b[(size_t)kk * n + col]);
   return acc;
 }
+
+/* ---- consumers of the reference's example programs ---- */
+
+/* saxpy (src/examples/saxpy/saxpy_cudaDMA_kernel.cu:55-59, gold loop saxpy_cudaDMA.cu:66-72).
+ * The device compiler of the reference contracts a*x+y into one fused operation; the
+ * oracle states that rounding explicitly. */
+void oracle_saxpy(float a, const float* x, float* y, size_t n)
+{
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < n; ++i) y[i] = fmaf(a, x[i], y[i]);
+}
+
+/* sgemv, "n" form (src/examples/sgemv/sgemv_dma.cu:140-175; host check :752-771): thread `i`
+ * walks row i of a column-major matrix, res += A[i + j*lda] * x[j] for ascending j starting
+ * from 0.0f, one fused multiply-add per term, then y[i] = alpha * res. */
+void oracle_sgemv(int n, int m, float alpha, const float* a, int lda, const float* x, float* y)
+{
+#pragma omp parallel for schedule(static)
+  for (int i = 0; i < n; ++i) {
+    float res = 0.0f;
+    for (int j = 0; j < m; ++j) res = fmaf(a[(size_t)i + (size_t)j * lda], x[j], res);
+    y[i] = alpha * res;
+  }
+}
+
+/* 2-D cross average of the stencil example (src/examples/stencil/stencil_math.h:52-84), on
+ * float2 elements (two independent components).  Order of the additions: centre, then the
+ * -x arm for d = 1..reach, the +x arm, the -y arm, the +y arm; the sum is divided by
+ * 4*radius + 1.  The reference's loops run d < RADIUS, i.e. reach = radius - 1, while the
+ * divisor stays 4*radius + 1; callers pass reach = radius - 1 to state exactly that.
+ * Layout (cudaDMA_stencil2D.cu:86-101): (dimx+2r) x (dimy+2r) x (dimz+2r) elements, row
+ * stride dimx+2r, slice stride (dimy+2r)*(dimx+2r); slices r .. r+dimz-1 are processed and
+ * only interior points of dst are written. */
+void oracle_stencil2d(const float* src, float* dst, int dimx, int dimy, int dimz, int radius, int reach)
+{
+  const size_t row = (size_t)dimx + 2 * radius;
+  const size_t slice = ((size_t)dimy + 2 * radius) * row;
+  const float div = (float)(4 * radius + 1);
+#pragma omp parallel for collapse(2) schedule(static)
+  for (int z = 0; z < dimz; ++z)
+    for (int y = 0; y < dimy; ++y)
+      for (int x = 0; x < dimx; ++x) {
+        const size_t o = (size_t)(z + radius) * slice + (size_t)(y + radius) * row + (size_t)(x + radius);
+        for (int c = 0; c < 2; ++c) {
+          float acc = src[2 * o + c];
+          for (int d = 1; d <= reach; ++d) acc += src[2 * (o - d) + c];
+          for (int d = 1; d <= reach; ++d) acc += src[2 * (o + d) + c];
+          for (int d = 1; d <= reach; ++d) acc += src[2 * (o - d * row) + c];
+          for (int d = 1; d <= reach; ++d) acc += src[2 * (o + d * row) + c];
+          dst[2 * o + c] = acc / div;
+        }
+      }
+}

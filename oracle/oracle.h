@@ -59,6 +59,17 @@ void oracle_gemm_bf16(const uint16_t* a, const uint16_t* b, float* c, int m, int
 /* one entry of the product, for spot checks at full size */
 float oracle_gemm_bf16_entry(const uint16_t* a, const uint16_t* b, int n, int k, int row, int col);
 
+/* ---- consumers of the reference's example programs ---- */
+/* y[i] = fma(a, x[i], y[i])  (src/examples/saxpy/saxpy_cudaDMA_kernel.cu:55-59) */
+void oracle_saxpy(float a, const float* x, float* y, size_t n);
+/* y[i] = alpha * sum_j A[i + j*lda] * x[j], A column-major n x m, ascending j, fused multiply-add
+ * (src/examples/sgemv/sgemv_dma.cu:140-175) */
+void oracle_sgemv(int n, int m, float alpha, const float* a, int lda, const float* x, float* y);
+/* two-component 2-D cross average of every z slice (src/examples/stencil/stencil_math.h:27-87);
+ * buffers are padded by `radius` on every side of all three dimensions
+ * (src/examples/stencil/cudaDMA_stencil2D.cu:86-101); `reach` neighbours per arm are summed */
+void oracle_stencil2d(const float* src, float* dst, int dimx, int dimy, int dimz, int radius, int reach);
+
 #ifdef __cplusplus
 }
 #endif

@@ -32,6 +32,9 @@ _SIGS = {
     "oracle_stencil25": (None, [_vp, _vp, _ci, _ci, _ci, _ci]),
     "oracle_gemm_bf16": (None, [_vp, _vp, _vp, _ci, _ci, _ci]),
     "oracle_gemm_bf16_entry": (ctypes.c_float, [_vp, _vp, _ci, _ci, _ci, _ci]),
+    "oracle_saxpy": (None, [ctypes.c_float, _vp, _vp, _cs]),
+    "oracle_sgemv": (None, [_ci, _ci, ctypes.c_float, _vp, _ci, _vp, _vp]),
+    "oracle_stencil2d": (None, [_vp, _vp, _ci, _ci, _ci, _ci, _ci]),
 }
 
 _lib = None

@@ -274,3 +274,107 @@ def test_gemm_bf16(O):
     ref = af.astype(np.float64) @ bf.astype(np.float64)
     assert np.max(np.abs(c - ref)) <= 1e-4 * np.max(np.abs(ref))
     assert abs(O.oracle_gemm_bf16_entry(ptr(a), ptr(b), n, k, 5, 7) - c[5, 7]) <= 1e-5 * abs(c[5, 7]) + 1e-6
+
+
+# ---- consumers of the reference's example programs ----
+
+def _round_f32(fr):
+    """The float32 nearest to an exact rational (ties to even), decided with exact arithmetic."""
+    from fractions import Fraction
+    c = np.float32(float(fr))
+    best = c
+    for cand in (np.nextafter(c, np.float32(-np.inf)), np.nextafter(c, np.float32(np.inf))):
+        dc, db = abs(Fraction(float(cand)) - fr), abs(Fraction(float(best)) - fr)
+        if dc < db or (dc == db and (int(np.float32(cand).view(np.uint32)) & 1) == 0):
+            best = cand
+    return np.float32(best)
+
+
+def test_saxpy_is_one_correctly_rounded_operation(O):
+    """y = fma(a, x, y): checked against exact rational arithmetic (a plain a*x rounded before the add
+    would differ on some of these samples), and against the reference's own tolerance on all."""
+    from fractions import Fraction
+    n = 4096
+    x, y0 = ol.uniform(n, 71), ol.uniform(n, 72)
+    a = np.float32(0.8401877)           # first rand()/RAND_MAX of glibc srand(0), as saxpy_cudaDMA.cu:89-93 draws it
+    y = y0.copy()
+    O.oracle_saxpy(a, ptr(x), ptr(y), n)
+    two_step = (a * x + y0).astype(np.float32)
+    assert np.max(np.abs(y - two_step)) <= 1e-6          # the example's PASSED criterion (saxpy_cudaDMA.cu:171)
+    assert not np.array_equal(y, two_step)               # ... and the fused form is distinguishable from it
+    for i in range(0, n, 13):
+        want = _round_f32(Fraction(float(a)) * Fraction(float(x[i])) + Fraction(float(y0[i])))
+        assert y[i] == want, i
+
+
+def test_sgemv_known_answer_of_the_reference_driver(O):
+    """The reference's driver fills A[j*n+i] = (i*j)%11, x[j] = j%11, alpha = 2 at n = m = 896
+    (sgemv_dma.cu:752-771, 72-73): small integers, so every order of summation is exact and the
+    answer is plain integer arithmetic."""
+    n = m = 896
+    i, j = np.meshgrid(np.arange(n), np.arange(m), indexing="ij")
+    a_int = (i * j) % 11                                  # [row i, column j]
+    x_int = np.arange(m) % 11
+    a = np.asfortranarray(a_int.astype(np.float32))       # column-major, lda = n
+    x = x_int.astype(np.float32)
+    y = np.empty(n, dtype=np.float32)
+    O.oracle_sgemv(n, m, 2.0, ptr(a), n, ptr(x), ptr(y))
+    assert np.array_equal(y.astype(np.int64), 2 * (a_int @ x_int))
+
+
+def test_sgemv_order_lda_and_fusion(O):
+    from fractions import Fraction
+    n, m, lda = 5, 24, 9
+    a = ol.uniform(lda * m, 81)
+    x = ol.uniform(m, 82)
+    y = np.empty(n, dtype=np.float32)
+    alpha = np.float32(1.7)
+    O.oracle_sgemv(n, m, alpha, ptr(a), lda, ptr(x), ptr(y))
+    for row in range(n):
+        res = np.float32(0.0)
+        for col in range(m):
+            res = _round_f32(Fraction(float(a[row + col * lda])) * Fraction(float(x[col])) + Fraction(float(res)))
+        assert y[row] == np.float32(alpha * res)
+    # against numpy in double, as a sanity bound that would catch a transposed matrix or a wrong lda
+    ref = a.reshape(m, lda)[:, :n].T.astype(np.float64) @ x.astype(np.float64)
+    assert np.max(np.abs(y - alpha * ref)) < 1e-5
+
+
+def _stencil2d_numpy(src, dimx, dimy, dimz, r, reach):
+    """Same additions in the same order, one numpy float32 operation per step."""
+    g = src.reshape(dimz + 2 * r, dimy + 2 * r, dimx + 2 * r, 2)
+    core = lambda dy, dx: g[r:r + dimz, r + dy:r + dy + dimy, r + dx:r + dx + dimx, :]
+    acc = core(0, 0).copy()
+    for d in range(1, reach + 1):
+        acc = acc + core(0, -d)
+    for d in range(1, reach + 1):
+        acc = acc + core(0, d)
+    for d in range(1, reach + 1):
+        acc = acc + core(-d, 0)
+    for d in range(1, reach + 1):
+        acc = acc + core(d, 0)
+    return acc / np.float32(4 * r + 1)
+
+
+@pytest.mark.parametrize("r,reach", [(4, 3), (4, 4), (2, 1), (1, 0)])
+def test_stencil2d_against_numpy_and_closed_forms(O, r, reach):
+    dimx, dimy, dimz = 24, 10, 3
+    total = (dimx + 2 * r) * (dimy + 2 * r) * (dimz + 2 * r)
+    src = ol.uniform(2 * total, 91)
+    dst = np.full(2 * total, 7.5, dtype=np.float32)
+    O.oracle_stencil2d(ptr(src), ptr(dst), dimx, dimy, dimz, r, reach)
+    got = dst.reshape(dimz + 2 * r, dimy + 2 * r, dimx + 2 * r, 2)
+    assert np.array_equal(got[r:-r, r:-r, r:-r, :], _stencil2d_numpy(src, dimx, dimy, dimz, r, reach))
+    mask = np.ones(got.shape, dtype=bool)
+    mask[r:-r, r:-r, r:-r, :] = False
+    assert np.all(got[mask] == 7.5)                       # nothing outside the interior is written
+    # a constant field: (1 + 4*reach) / (4r + 1), which is 1 only when the whole radius is summed
+    one = np.ones(2 * total, dtype=np.float32)
+    O.oracle_stencil2d(ptr(one), ptr(dst), dimx, dimy, dimz, r, reach)
+    want = np.float32(1 + 4 * reach) / np.float32(4 * r + 1)
+    assert np.all(got[r:-r, r:-r, r:-r, :] == want)
+    # a field that depends on z only: the stencil must not look across slices
+    zf = np.repeat(np.arange(dimz + 2 * r, dtype=np.float32), (dimy + 2 * r) * (dimx + 2 * r) * 2)
+    O.oracle_stencil2d(ptr(zf), ptr(dst), dimx, dimy, dimz, r, reach)
+    for z in range(dimz):
+        assert np.allclose(got[r + z, r:-r, r:-r, :], (z + r) * want, rtol=1e-6)
