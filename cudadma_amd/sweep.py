@@ -4,12 +4,14 @@ src/perf/sequential/param_sweep.py:27-58, which rewrites params_directed.h and r
 point; here the variants are compiled in and the occupancy is a run-time knob.
 
     python -m cudadma_amd.sweep [sequential] [strided] [gather] [halo] [gemm] [--wg 0,2,4,8] [--steps 20]
+    python -m cudadma_amd.sweep saxpy sgemv stencil2d        # the reference's example programs, every variant
 """
 import argparse
 import sys
 
 import torch
 
+from . import examples as ex
 from . import workloads as wl
 
 PEAK_GBS = 8000.0
@@ -93,6 +95,36 @@ def main(argv=None):
             c = torch.empty(n, n, device=dev)
             ms = _time(lambda: wl.gemm_bf16(a, b, c), args.steps)
             print(f"gemm       variant 0  {ms:9.4f} ms  {2.0 * n ** 3 / ms / 1e9:8.1f} TFLOP/s", flush=True)
+        elif name == "saxpy":
+            # bytes as the reference's driver counts them: x read, y read, y written (saxpy_cudaDMA.cu:192)
+            n = 1 << 28
+            x = wl.fill_uniform(torch.empty(n, device=dev), 11)
+            y = wl.fill_uniform(torch.empty(n, device=dev), 12)
+            for v in range(ex.num_variants(ex.SAXPY)):
+                print(f"# saxpy variant {v}: {ex.variant_name(ex.SAXPY, v)}")
+                for wg in wgs:
+                    wl.set_workgroups_per_cu(wg)
+                    _row(name, v, wg, _time(lambda: ex.saxpy(1e-3, x, y, v), args.steps), 3 * n * 4)
+        elif name == "sgemv":
+            n = m = 16384
+            a = wl.fill_uniform(torch.empty(m * n, device=dev), 21).view(m, n)
+            x = wl.fill_uniform(torch.empty(m, device=dev), 22)
+            y = torch.empty(n, device=dev)
+            for v in range(ex.num_variants(ex.SGEMV)):
+                print(f"# sgemv variant {v}: {ex.variant_name(ex.SGEMV, v)}")
+                _row(name, v, 0, _time(lambda: ex.sgemv(1.0, a, x, y, variant=v), args.steps), (m * n + m + n) * 4)
+        elif name == "stencil2d":
+            # the reference's directed size (params_directed.h): 960 x 160 x 200 float2, tiles of 32 x 4;
+            # bytes as its driver counts them: tile plus halo read, tile written (cudaDMA_stencil2D.cu:225-232)
+            dimx, dimy, dimz, r = 960, 160, 200, ex.STENCIL2D_RADIUS
+            shape = (dimz + 2 * r, dimy + 2 * r, dimx + 2 * r, 2)
+            src = wl.fill_uniform(torch.empty(shape, device=dev).view(-1), 31).view(shape)
+            dst = torch.zeros(shape, device=dev)
+            tiles = (dimx // 32) * (dimy // 4)
+            issued = tiles * dimz * ((4 + 2 * r) * (32 + 2 * r) + 4 * 32) * 8
+            for v in range(ex.num_variants(ex.STENCIL2D)):
+                print(f"# stencil2d variant {v}: {ex.variant_name(ex.STENCIL2D, v)}")
+                _row(name, v, 0, _time(lambda: ex.stencil2d(src, dst, v), args.steps), issued)
         else:
             sys.exit(f"unknown workload {name}")
     wl.set_workgroups_per_cu(0)
