@@ -77,8 +77,12 @@ static const VariantInfo kHalo[] = {
 };
 
 static const VariantInfo kGemm[] = {
-  {"warp-specialised: one DMA wavefront per operand with two CudaDMAStrided objects (two LDS stages, tile two K steps "
-   "ahead in flight), four compute wavefronts with v_mfma_f32_32x32x16_bf16, B fragments through ds_read_b64_tr_b16"},
+  {"the largest workgroup tile that divides the problem: variant 3 when m is a multiple of 256, else variant 1"},
+  {"warp-specialised: two DMA wavefronts per operand with two CudaDMAStrided objects each (two LDS stages, tile two K "
+   "steps ahead in flight), four compute wavefronts with v_mfma_f32_32x32x16_bf16, B fragments through "
+   "ds_read_b64_tr_b16; 128 x 128 workgroup tile, 64 x 64 per compute wavefront, two workgroups per compute unit"},
+  {"same structure, 128 x 256 workgroup tile, 64 x 128 per compute wavefront, one workgroup per compute unit"},
+  {"same structure, 256 x 128 workgroup tile, 128 x 64 per compute wavefront, one workgroup per compute unit"},
 };
 
 static const VariantInfo* table(int workload, int* count)

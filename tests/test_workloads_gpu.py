@@ -202,17 +202,25 @@ def _bf16_inputs(m, n, k):
     return a.reshape(m, k), b.reshape(k, n)
 
 
-@pytest.mark.parametrize("shape", [(128, 128, 128), (256, 384, 256), (512, 512, 512)])
-def test_gemm_small(device, shape):
+@pytest.mark.parametrize("variant", range(4))
+@pytest.mark.parametrize("shape", [(128, 128, 128), (256, 384, 256), (512, 512, 512), (768, 256, 384)])
+def test_gemm_small(device, shape, variant):
     m, n, k = shape
+    tile_m, tile_n = {0: (128, 128), 1: (128, 128), 2: (128, 256), 3: (256, 128)}[variant]
+    if m % tile_m or n % tile_n:
+        z = torch.zeros((m, n), dtype=torch.float32, device=device)
+        with pytest.raises(cd.CudaDMAError, match="this variant needs"):
+            wl.gemm_bf16(z.to(torch.bfloat16)[:, :k].contiguous() if k <= n else torch.zeros((m, k), dtype=torch.bfloat16, device=device),
+                         torch.zeros((k, n), dtype=torch.bfloat16, device=device), z, variant)
+        return
     a, b = _bf16_inputs(m, n, k)
     want = np.empty((m, n), dtype=np.float32)
     ol.load().oracle_gemm_bf16(ptr(a), ptr(b), ptr(want), m, n, k)
     d_a = torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
     d_b = torch.from_numpy(b.view(np.int16)).to(device).view(torch.bfloat16)
     d_c = torch.full((m, n), float("nan"), dtype=torch.float32, device=device)
-    print(f"gemm {shape}", flush=True)
-    wl.gemm_bf16(d_a, d_b, d_c)
+    print(f"gemm {shape} variant {variant}", flush=True)
+    wl.gemm_bf16(d_a, d_b, d_c, variant)
     torch.cuda.synchronize()
     got = d_c.cpu().numpy()
     scale = np.sqrt(k)                      # typical magnitude of an entry
@@ -222,13 +230,14 @@ def test_gemm_small(device, shape):
     assert float(np.max(np.abs(got - want))) <= 1e-4 * scale * np.sqrt(k)
 
 
-def test_gemm_full_size(device):
+@pytest.mark.parametrize("variant", [0, 1, 2])
+def test_gemm_full_size(device, variant):
     m = n = k = 4096
     a, b = _bf16_inputs(m, n, k)
     d_a = torch.from_numpy(a.view(np.int16)).to(device).view(torch.bfloat16)
     d_b = torch.from_numpy(b.view(np.int16)).to(device).view(torch.bfloat16)
     d_c = torch.empty((m, n), dtype=torch.float32, device=device)
-    wl.gemm_bf16(d_a, d_b, d_c)
+    wl.gemm_bf16(d_a, d_b, d_c, variant)
     torch.cuda.synchronize()
     got = d_c.cpu().numpy()
     O = ol.load()
