@@ -155,7 +155,8 @@ def main():
     ga = torch.randn((dim, dim), device=dev, dtype=torch.float32).to(torch.bfloat16)
     gb = torch.randn((dim, dim), device=dev, dtype=torch.float32).to(torch.bfloat16)
     gc = torch.empty((dim, dim), device=dev, dtype=torch.float32)
-    ms, _ = time_launches(lambda: wl.gemm_bf16(ga, gb, gc), steps, warmup)
+    # the matrix cores' clock settles only after a few tens of launches: longer untimed warm-up
+    ms, _ = time_launches(lambda: wl.gemm_bf16(ga, gb, gc), max(steps, 50), max(warmup, 30))
     flops = 2.0 * dim ** 3
     gemm = {"TFLOP/s": round(flops / ms / 1e9, 1), "frac_of_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4),
             "ms": round(ms, 4), "flop": flops,

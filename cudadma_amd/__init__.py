@@ -20,6 +20,7 @@ from ._lib import (  # noqa: F401
     CudaDMAError,
     PlanQuery,
     RunArgs,
+    V1Case,
     lib,
     lib_path,
 )

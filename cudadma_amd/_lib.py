@@ -30,6 +30,13 @@ class Case(ctypes.Structure):
         return "Case(" + ", ".join(f"{n}={getattr(self, n)}" for n, _ in self._fields_) + ")"
 
 
+class V1Case(ctypes.Structure):
+    """struct cudadma_v1_case_t"""
+    _fields_ = [(n, ctypes.c_int) for n in (
+        "pattern", "warp_specialized", "bytes_per_elmt", "num_elmts", "src_stride", "dst_stride",
+        "dma_threads", "block_threads", "window_bytes")]
+
+
 class PlanQuery(ctypes.Structure):
     """struct cudadma_plan_query"""
     _fields_ = [(n, ctypes.c_int) for n in (
@@ -89,6 +96,10 @@ def lib():
     L.cudadma_set_tuning.argtypes = [ctypes.c_char_p, ci]
     L.cudadma_variant_name.restype = ctypes.c_char_p
     L.cudadma_variant_name.argtypes = [ci, ci]
+    L.cudadma_v1_get_case.restype = ci
+    L.cudadma_v1_get_case.argtypes = [ci, ctypes.POINTER(V1Case)]
+    L.cudadma_v1_case_text.restype = ctypes.c_char_p
+    L.cudadma_v1_case_text.argtypes = [ci]
     L.cudadma_example_variant_name.restype = ctypes.c_char_p
     L.cudadma_example_variant_name.argtypes = [ci, ci]
     _lib = L
@@ -111,6 +122,8 @@ _WORKLOAD_SIGNATURES = {
     "cudadma_halo_stencil": [_vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cudadma_gemm_bf16": [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cudadma_selftest_bounded_wait": [_vp, _vp],
+    "cudadma_v1_num_cases": [],
+    "cudadma_v1_run_case": [_ci, _vp, _vp, _vp, _vp],
     "cudadma_example_num_variants": [_ci],
     "cudadma_example_saxpy": [_ci, ctypes.c_float, _vp, _vp, ctypes.c_longlong, _vp],
     "cudadma_example_sgemv": [_ci, _ci, _ci, ctypes.c_float, _vp, _ci, _vp, _vp, _vp],
@@ -126,4 +139,5 @@ def check(rc):
 def exported_symbols():
     """Every extern "C" symbol include/cudadma_amd.h declares."""
     return ["cudadma_last_error", "cudadma_device_cus", "cudadma_num_cases", "cudadma_get_case",
-            "cudadma_run_case", "cudadma_variant_name", "cudadma_example_variant_name", "cudadma_plan_map", "cudadma_diagnose", "cudadma_set_tuning"] + list(_WORKLOAD_SIGNATURES)
+            "cudadma_run_case", "cudadma_variant_name", "cudadma_example_variant_name",
+            "cudadma_v1_get_case", "cudadma_v1_case_text", "cudadma_plan_map", "cudadma_diagnose", "cudadma_set_tuning"] + list(_WORKLOAD_SIGNATURES)

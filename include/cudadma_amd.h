@@ -191,6 +191,27 @@ int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz
 int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k,
                       int variant, void* stream);
 
+/* ---- known-answer cases for the first-generation class names -------------------------
+ * One transfer per case by cudaDMASequential / cudaDMAStrided / cudaDMAIndirect as declared in
+ * include/cudaDMA.h:644-3580 (every constructor form), into a 16 KiB LDS window that holds the
+ * byte 0xA5 everywhere else; the whole window is copied to d_out.  The reference has no test
+ * of these classes beyond its examples; the expectation is the closed form of each pattern. */
+typedef struct {
+  int pattern;            /* CUDADMA_PATTERN_*                                               */
+  int warp_specialized;   /* 1: 64 compute threads + dma_threads DMA threads; 0: all transfer */
+  int bytes_per_elmt;     /* bytes of the transfer (sequential) or of one element             */
+  int num_elmts;
+  int src_stride;         /* bytes; strided source, or dense source of a scatter               */
+  int dst_stride;         /* bytes; strided destination, or dense destination of a gather      */
+  int dma_threads;
+  int block_threads;
+  int window_bytes;       /* size of d_out                                                     */
+} cudadma_v1_case_t;
+int cudadma_v1_num_cases(void);
+int cudadma_v1_get_case(int case_id, cudadma_v1_case_t* out);
+const char* cudadma_v1_case_text(int case_id);       /* the declaration the case exercises */
+int cudadma_v1_run_case(int case_id, const void* d_in, const int* d_index, void* d_out, void* stream);
+
 /* ---- the reference's example programs on the wave64 objects --------------------------
  * The kernels behind these are written against the DMA classes alone (the first-
  * generation names of include/cudaDMA.h for saxpy and sgemv, the current ones for the
