@@ -50,34 +50,64 @@ def time_launches(fn, steps, warmup):
     return start.elapsed_time(stop) / steps, wall_ms / steps
 
 
-def cpu_baseline_transpose(budget_s=20.0):
-    """The oracle's OpenMP transpose on this machine's host cores, on an 8192 x 8192 sample
-    (a quarter of the matrix: 512 MiB of traffic per repetition)."""
+def _median_time(fn, budget_s, min_reps=5, max_reps=400):
+    fn()                                             # warm-up + first touch of the output
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < min_reps or (len(times) < max_reps and time.perf_counter() - t_all < budget_s):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return sorted(times)[len(times) // 2], len(times)
+
+
+def cpu_baselines(budget_s=16.0):
+    """The oracle's OpenMP implementation of each pattern on this machine's host cores, each on a
+    bounded sample of its workload; bytes counted as for the GPU figures.  Returns the headline
+    object (strided transpose) and a per-pattern dictionary."""
     import numpy as np
     from tests import oracle_lib as ol
     from tests.oracle_lib import ptr
     O = ol.load()
-    n = 8192
-    a = ol.uniform(n * n, 1002).reshape(n, n)      # parallel first touch
-    out = np.empty_like(a)
-    O.oracle_transpose(ptr(a), ptr(out), n)          # warm-up + first touch of the output
-    times = []
-    t_all = time.perf_counter()
-    while len(times) < 5 or (len(times) < 15 and time.perf_counter() - t_all < budget_s):
-        t0 = time.perf_counter()
-        O.oracle_transpose(ptr(a), ptr(out), n)
-        times.append(time.perf_counter() - t0)
-        if time.perf_counter() - t_all > budget_s:
-            break
-    med = sorted(times)[len(times) // 2]
-    return {
-        "value": round(2.0 * n * n * 4 / med / 1e9, 2),
-        "unit": "GB/s",
-        "cores": O.oracle_num_threads(),
-        "kind": "port",
-        "sample": f"oracle_transpose (OpenMP, blocked 64x64) of an {n}x{n} float32 sample, "
-                  f"median of {len(times)} repetitions",
-    }
+    cores = O.oracle_num_threads()
+    per = budget_s / 4
+    out = {}
+
+    n = 8192                                         # a quarter of the matrix: 512 MiB of traffic per repetition
+    a = ol.uniform(n * n, 1002).reshape(n, n)        # parallel first touch
+    t = np.empty_like(a)
+    med, reps = _median_time(lambda: O.oracle_transpose(ptr(a), ptr(t), n), per)
+    out["strided"] = {"GB/s": round(2.0 * n * n * 4 / med / 1e9, 2),
+                      "sample": f"oracle_transpose (blocked 64x64) of an {n}x{n} float32 sample, median of {reps}"}
+    del a, t
+
+    m = 64 * 1024 * 1024 // 4                        # the whole config: 64 MiB
+    src = ol.uniform(m, 1001)
+    dst = np.empty_like(src)
+    med, reps = _median_time(lambda: O.oracle_copy(ptr(src), ptr(dst), m), per)
+    out["sequential"] = {"GB/s": round(2.0 * m * 4 / med / 1e9, 2),
+                         "sample": f"oracle_copy of the full 64 MiB buffer, median of {reps}"}
+    del src, dst
+
+    recs, n_idx = 4 * 1024 * 1024, 4 * 1024 * 1024   # full table, one eighth of the index list
+    table = ol.uniform(recs * 32, 1003)
+    idx = ol.indices(n_idx, recs, 1003)
+    sums = np.empty(n_idx // 32 * 32, dtype=np.float32)
+    med, reps = _median_time(lambda: O.oracle_gather_rowsum(ptr(table), ptr(idx), ptr(sums), n_idx, 32, 32), per)
+    out["gather"] = {"GB/s": round((n_idx * 132 + sums.size * 4) / med / 1e9, 2),
+                     "sample": f"oracle_gather_rowsum over the full 512 MiB table with {n_idx} indices, median of {reps}"}
+    del table, idx, sums
+
+    g, p = 256, 4                                    # one eighth of the grid
+    grid = ol.uniform((g + 2 * p) ** 3, 1004)
+    res = np.empty(g ** 3, dtype=np.float32)
+    med, reps = _median_time(lambda: O.oracle_stencil25(ptr(grid), ptr(res), g, g, g, p), per)
+    out["halo"] = {"GB/s": round(2.0 * g ** 3 * 4 / med / 1e9, 2),
+                   "sample": f"oracle_stencil25 on a {g}^3 float32 sample, median of {reps}"}
+
+    head = {"value": out["strided"]["GB/s"], "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "OpenMP " + out["strided"]["sample"]}
+    return head, out
 
 
 def main():
@@ -192,9 +222,11 @@ def main():
         "gemm": gemm,
     }
     if not args.no_cpu_baseline:
-        log("timing the host-core baseline (oracle transpose) ...")
-        result["cpu_baseline"] = cpu_baseline_transpose()
+        log("timing the host-core baselines (oracle, OpenMP) ...")
+        result["cpu_baseline"], result["cpu_baseline_patterns"] = cpu_baselines()
         log(f"cpu baseline: {result['cpu_baseline']}")
+        for name, row in result["cpu_baseline_patterns"].items():
+            log(f"  cpu {name:10s} {row['GB/s']:8.2f} GB/s   {row['sample']}")
     print(json.dumps(result), flush=True)
 
 
