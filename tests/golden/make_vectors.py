@@ -1,0 +1,103 @@
+#!/usr/bin/env python3
+"""Writes tests/golden/vectors.json: known answers for the oracle, produced WITHOUT the oracle.
+
+Every value below comes from pure-Python integer arithmetic, from numpy slicing, or from the
+expectation the reference's own test programs state (ramp input and exact comparison,
+cudaDMA_test_strided_v2.cu:561-563,659-677; the halo checker cudaDMA_test_halo.cu:91-164; the
+integer data of the sgemv driver, sgemv_dma.cu:752-771).  The reference itself is neither
+imported nor executed.  tests/test_oracle.py compares oracle/liboracle.so with this file.
+
+    python tests/golden/make_vectors.py
+"""
+import json
+import os
+
+import numpy as np
+
+M64 = (1 << 64) - 1
+
+
+def splitmix64(x):
+    z = (x + 0x9E3779B97F4A7C15) & M64
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & M64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & M64
+    return z ^ (z >> 31)
+
+
+def hash32(seed, i):
+    return splitmix64((seed + i) & M64) >> 32
+
+
+def uniform_bits(seed, n):
+    """float32 bit patterns of (h >> 8) * 2^-23 - 1: exact in binary32, so built from integers."""
+    out = []
+    for i in range(n):
+        v = np.float32(hash32(seed, i) >> 8) * np.float32(2.0 ** -23) - np.float32(1.0)
+        out.append(int(np.float32(v).view(np.uint32)))
+    return out
+
+
+def indices(seed, n, n_records):
+    out = []
+    for i in range(n):
+        j = i
+        r = hash32(seed ^ 0x5bd1e995, i)
+        if i > 1024 and r % 10 == 0:
+            j = i - 1 - ((r // 10) % 1024)
+        out.append(hash32(seed, j) % n_records)
+    return out
+
+
+def strided_ramp(e_floats, n, src_stride_floats, dst_stride_floats):
+    """The reference's strided test: source float(i), every moved element compared exactly."""
+    src = np.arange(n * src_stride_floats + e_floats, dtype=np.float32)
+    dst = np.full(n * dst_stride_floats + e_floats, -1.0, dtype=np.float32)
+    for r in range(n):
+        dst[r * dst_stride_floats:r * dst_stride_floats + e_floats] = src[r * src_stride_floats:r * src_stride_floats + e_floats]
+    return [int(x) for x in dst]
+
+
+def halo_ring(dimx, dimy, radius, corners, pitch):
+    """Ring of a dimx x dimy tile by numpy slicing; source element (y, x) holds y*pitch + x + 1, untouched cells 0."""
+    rows = dimy + 2 * radius
+    src = (np.arange(rows * pitch, dtype=np.int64) + 1).reshape(rows, pitch)
+    w = dimx + 2 * radius
+    dst = np.zeros((rows, w), dtype=np.int64)
+    x0 = 0 if corners else radius
+    x1 = w if corners else radius + dimx
+    dst[:radius, x0:x1] = src[:radius, x0:x1]
+    dst[radius + dimy:, x0:x1] = src[radius + dimy:rows, x0:x1]
+    dst[radius:radius + dimy, :radius] = src[radius:radius + dimy, :radius]
+    dst[radius:radius + dimy, radius + dimx:w] = src[radius:radius + dimy, radius + dimx:w]
+    return [int(v) for v in dst.ravel()]
+
+
+def sgemv_reference_driver(n, m, alpha):
+    i, j = np.meshgrid(np.arange(n), np.arange(m), indexing="ij")
+    return [int(v) for v in alpha * (((i * j) % 11) @ (np.arange(m) % 11))]
+
+
+def main():
+    vectors = {
+        "splitmix64": {str(x): str(splitmix64(x)) for x in (0, 1, 1001, 1234567, 0xDEADBEEFCAFEF00D, M64)},
+        "uniform_bits": {str(seed): uniform_bits(seed, 64) for seed in (1001, 1002, 1003, 1004)},
+        "indices": {"seed": 1003, "n_records": 4 * 1024 * 1024, "n": 4096, "values": indices(1003, 4096, 4 * 1024 * 1024)},
+        "strided_ramp": [
+            {"e_floats": e, "n": n, "src_stride_floats": ss, "dst_stride_floats": ds, "dst": strided_ramp(e, n, ss, ds)}
+            for (e, n, ss, ds) in ((16, 5, 40, 16), (3, 7, 9, 5), (64, 4, 64, 68))
+        ],
+        "halo_ring": [
+            {"dimx": dx, "dimy": dy, "radius": r, "corners": c, "pitch": p, "dst": halo_ring(dx, dy, r, c, p)}
+            for (dx, dy, r, c, p) in ((8, 6, 2, 0, 16), (8, 6, 2, 1, 16), (32, 32, 4, 0, 48), (5, 3, 1, 1, 9))
+        ],
+        "sgemv_reference_driver": {"n": 896, "m": 896, "alpha": 2, "y": sgemv_reference_driver(896, 896, 2)},
+    }
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "vectors.json")
+    with open(path, "w") as f:
+        json.dump(vectors, f, separators=(",", ":"))
+        f.write("\n")
+    print(path, os.path.getsize(path), "bytes")
+
+
+if __name__ == "__main__":
+    main()

@@ -378,3 +378,52 @@ def test_stencil2d_against_numpy_and_closed_forms(O, r, reach):
     O.oracle_stencil2d(ptr(zf), ptr(dst), dimx, dimy, dimz, r, reach)
     for z in range(dimz):
         assert np.allclose(got[r + z, r:-r, r:-r, :], (z + r) * want, rtol=1e-6)
+
+
+# ---- the committed golden vectors (tests/golden/vectors.json, written by make_vectors.py without the oracle) ----
+
+def _golden():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "vectors.json")) as f:
+        return json.load(f)
+
+
+def test_golden_generators(O):
+    g = _golden()
+    for x, want in g["splitmix64"].items():
+        assert O.oracle_splitmix64(int(x)) == int(want)
+    for seed, bits in g["uniform_bits"].items():
+        got = ol.uniform(len(bits), int(seed)).view(np.uint32)
+        assert [int(v) for v in got] == bits
+    idx = g["indices"]
+    assert [int(v) for v in ol.indices(idx["n"], idx["n_records"], idx["seed"])] == idx["values"]
+
+
+def test_golden_strided_ramp_and_halo_ring(O):
+    g = _golden()
+    for case in g["strided_ramp"]:
+        e, n, ss, ds = case["e_floats"], case["n"], case["src_stride_floats"], case["dst_stride_floats"]
+        src = ol.ramp(n * ss + e)
+        dst = np.full(n * ds + e, -1.0, dtype=np.float32)
+        O.oracle_strided(ptr(src), ptr(dst), 4 * e, n, 4 * ss, 4 * ds)
+        assert [int(v) for v in dst] == case["dst"]
+    for case in g["halo_ring"]:
+        dx, dy, r, c, p = case["dimx"], case["dimy"], case["radius"], case["corners"], case["pitch"]
+        rows, w = dy + 2 * r, dx + 2 * r
+        src = (np.arange(rows * p, dtype=np.int64) + 1)
+        dst = np.zeros(rows * w, dtype=np.int64)
+        O.oracle_halo(ptr(src, 8 * (r * p + r)), ptr(dst, 8 * (r * w + r)), 8, r, c, dx, dy, p)
+        assert [int(v) for v in dst] == case["dst"]
+        assert O.oracle_halo_check(ptr(src), ptr(dst), 8, r, c, dx, dy, p) == 1
+
+
+def test_golden_sgemv_of_the_reference_driver(O):
+    g = _golden()["sgemv_reference_driver"]
+    n, m = g["n"], g["m"]
+    i, j = np.meshgrid(np.arange(n), np.arange(m), indexing="ij")
+    a = np.asfortranarray(((i * j) % 11).astype(np.float32))
+    x = (np.arange(m) % 11).astype(np.float32)
+    y = np.empty(n, dtype=np.float32)
+    O.oracle_sgemv(n, m, float(g["alpha"]), ptr(a), n, ptr(x), ptr(y))
+    assert [int(v) for v in y] == g["y"]

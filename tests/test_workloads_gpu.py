@@ -27,6 +27,20 @@ def test_device_generators_match_the_host_statement(device):
     assert np.array_equal(idx, ol.indices(n, 4096 * 1024, 1003))
 
 
+def test_device_generators_match_the_golden_vectors(device):
+    """tests/golden/vectors.json was written by pure-Python integer arithmetic, without the oracle."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "vectors.json")) as f:
+        g = json.load(f)
+    for seed, bits in g["uniform_bits"].items():
+        got = wl.fill_uniform(torch.empty(len(bits), dtype=torch.float32, device=device), int(seed))
+        assert [int(v) for v in got.cpu().numpy().view(np.uint32)] == bits
+    idx = g["indices"]
+    got = wl.fill_indices(torch.empty(idx["n"], dtype=torch.int32, device=device), idx["n_records"], idx["seed"])
+    assert [int(v) for v in got.cpu().numpy()] == idx["values"]
+
+
 # ------------------------------------------------------------------ config 1
 @pytest.mark.parametrize("variant", _variants(wl.SEQUENTIAL))
 @pytest.mark.parametrize("tiles", [1, 3, 257, 4096])
