@@ -54,6 +54,21 @@ __device__ __forceinline__ void tile_of_workgroup(const int b, const int tiles_m
   }
 }
 
+// Order of one slice for the instruction scheduler: MFMAs matrix instructions with the READS
+// LDS requests of the next slice issued two at a time behind the first of them; the last
+// matrix instructions run with nothing behind them, so the data has landed when the next
+// slice starts.
+template<int G, int MFMAS, int READS>
+__device__ __forceinline__ void pin_slice()
+{
+  if constexpr (G < MFMAS) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                    // one MFMA
+    if constexpr (2 * G + 2 <= READS) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);   // two LDS reads
+    else if constexpr (2 * G < READS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    pin_slice<G + 1, MFMAS, READS>();
+  }
+}
+
 template<int WI, int WJ>
 __global__ void __launch_bounds__(kComputeThreads + 2 * kDmaWave)
 gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restrict__ b, float* __restrict__ c,
@@ -130,7 +145,6 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
             (__attribute__((address_space(3))) bf16x4_t*)(p + 4 * kBPitch));
         fb[j] = bf16x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
-      if constexpr (kPinned) __builtin_amdgcn_sched_barrier(0);      // keep the requests ahead of the products that hide them
     };
     auto multiply = [&](const bf16x8_t (&fa)[WI], const bf16x8_t (&fb)[WJ]) __attribute__((always_inline)) {
 #pragma unroll
@@ -138,7 +152,16 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
 #pragma unroll
         for (int j = 0; j < WJ; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
-      if constexpr (kPinned) __builtin_amdgcn_sched_barrier(0);
+    };
+    // One slice of the pinned schedule: the WI + 2*WJ LDS requests of the next slice are
+    // issued one by one in the shadow of the WI*WJ matrix instructions of the current slice
+    // (a matrix instruction holds its pipe for 32 cycles, the wavefront is free to issue an
+    // LDS request meanwhile), and nothing moves across the ends of the slice.
+    auto interleave = [&]() __attribute__((always_inline)) {
+      if constexpr (kPinned) {
+        pin_slice<0, WI * WJ, WI + 2 * WJ>();
+        __builtin_amdgcn_sched_barrier(0);
+      }
     };
     // The one compute wavefront of a SIMD has to keep the matrix core fed by itself: the
     // fragments of the next slice are requested before the products of the current one are
@@ -168,23 +191,23 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
       dma_b0.wait_for_dma_finish();
       load_frags(fa0, fb0, sa0, sb0, 0);
       for (int kt = 0; kt < ksteps; kt += 2) {
-        load_frags(fa1, fb1, sa0, sb0, 1); multiply(fa0, fb0);
-        load_frags(fa0, fb0, sa0, sb0, 2); multiply(fa1, fb1);
-        load_frags(fa1, fb1, sa0, sb0, 3); multiply(fa0, fb0);
+        load_frags(fa1, fb1, sa0, sb0, 1); multiply(fa0, fb0); interleave();
+        load_frags(fa0, fb0, sa0, sb0, 2); multiply(fa1, fb1); interleave();
+        load_frags(fa1, fb1, sa0, sb0, 3); multiply(fa0, fb0); interleave();
         dma_a1.wait_for_dma_finish();
         dma_b1.wait_for_dma_finish();
-        load_frags(fa0, fb0, sa1, sb1, 0); multiply(fa1, fb1);
+        load_frags(fa0, fb0, sa1, sb1, 0); multiply(fa1, fb1); interleave();
         dma_a0.start_async_dma();
         dma_b0.start_async_dma();
-        load_frags(fa1, fb1, sa1, sb1, 1); multiply(fa0, fb0);
-        load_frags(fa0, fb0, sa1, sb1, 2); multiply(fa1, fb1);
-        load_frags(fa1, fb1, sa1, sb1, 3); multiply(fa0, fb0);
+        load_frags(fa1, fb1, sa1, sb1, 1); multiply(fa0, fb0); interleave();
+        load_frags(fa0, fb0, sa1, sb1, 2); multiply(fa1, fb1); interleave();
+        load_frags(fa1, fb1, sa1, sb1, 3); multiply(fa0, fb0); interleave();
         if (kt + 2 < ksteps) {
           dma_a0.wait_for_dma_finish();
           dma_b0.wait_for_dma_finish();
           load_frags(fa0, fb0, sa0, sb0, 0);
         }
-        multiply(fa1, fb1);
+        multiply(fa1, fb1); interleave();
         dma_a1.start_async_dma();
         dma_b1.start_async_dma();
       }
