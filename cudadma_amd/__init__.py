@@ -9,6 +9,8 @@ not been built: there is no CPU fallback.
 from ._lib import (  # noqa: F401
     CALL_GLOBAL,
     CALL_LDS_DIRECT,
+    CALL_LDS_DIRECT_SWIZZLE,
+    CALL_LDS_SWIZZLE,
     CALL_QUALIFIED,
     CALL_UNQUALIFIED,
     PATTERN_GATHER,

@@ -5,7 +5,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
 PATTERN_SEQUENTIAL, PATTERN_STRIDED, PATTERN_GATHER, PATTERN_SCATTER, PATTERN_HALO = range(5)
-CALL_UNQUALIFIED, CALL_GLOBAL, CALL_QUALIFIED, CALL_LDS_DIRECT = range(4)
+CALL_UNQUALIFIED, CALL_GLOBAL, CALL_QUALIFIED, CALL_LDS_DIRECT, CALL_LDS_SWIZZLE, CALL_LDS_DIRECT_SWIZZLE = range(6)
 
 PATTERN_NAMES = {
     PATTERN_SEQUENTIAL: "sequential",

@@ -61,8 +61,15 @@ extern "C" int cudadma_run_case(int case_id, const cudadma_run_t* run, void* str
   CUDADMA_REQUIRE(run->lds_bytes > 0 && run->lds_bytes <= 64 * 1024 - 256 && (run->lds_bytes % 16) == 0,
                   "lds_bytes %d must be a positive multiple of 16 below 64 KiB", run->lds_bytes);
   CUDADMA_REQUIRE(run->reps >= 1, "reps must be >= 1");
-  CUDADMA_REQUIRE(run->call_style >= CUDADMA_CALL_UNQUALIFIED && run->call_style <= CUDADMA_CALL_LDS_DIRECT,
+  CUDADMA_REQUIRE(run->call_style >= CUDADMA_CALL_UNQUALIFIED && run->call_style <= CUDADMA_CALL_LDS_DIRECT_SWIZZLE,
                   "unknown call_style %d", run->call_style);
+  const bool swizzled = run->call_style == CUDADMA_CALL_LDS_SWIZZLE || run->call_style == CUDADMA_CALL_LDS_DIRECT_SWIZZLE;
+  const bool direct = run->call_style == CUDADMA_CALL_LDS_DIRECT || run->call_style == CUDADMA_CALL_LDS_DIRECT_SWIZZLE;
+  if (swizzled) {
+    CUDADMA_REQUIRE(d.pattern == CUDADMA_PATTERN_STRIDED, "swizzled LDS rows are a CudaDMAStrided layout");
+    CUDADMA_REQUIRE((d.bytes_per_elmt % d.alignment) == 0, "swizzled rows must be whole chunks (%d bytes per row, chunks of %d)",
+                    d.bytes_per_elmt, d.alignment);
+  }
   if (d.pattern == CUDADMA_PATTERN_HALO) {
     // the origins, not the buffer starts, carry the alignment
     const int src_origin = run->src_offset_bytes + (d.radius * run->pitch + d.radius) * d.bytes_per_elmt;
@@ -84,10 +91,10 @@ extern "C" int cudadma_run_case(int case_id, const cudadma_run_t* run, void* str
     CUDADMA_REQUIRE((run->src_stride % d.alignment) == 0 && (run->dst_stride % d.alignment) == 0,
                     "strides must be multiples of ALIGNMENT");
   if (d.pattern == CUDADMA_PATTERN_HALO)
-    CUDADMA_REQUIRE(run->call_style != CUDADMA_CALL_LDS_DIRECT, "the halo object has no direct path");
+    CUDADMA_REQUIRE(!direct, "the halo object has no direct path");
   if (d.pattern == CUDADMA_PATTERN_SCATTER)
-    CUDADMA_REQUIRE(run->call_style != CUDADMA_CALL_LDS_DIRECT, "scatter has no direct path");
-  if (run->call_style == CUDADMA_CALL_LDS_DIRECT)
+    CUDADMA_REQUIRE(!direct, "scatter has no direct path");
+  if (direct)
     CUDADMA_REQUIRE(d.alignment == 16 || d.alignment == 4, "the direct path moves 4 or 16 bytes per lane");
   if (run->reverse) {
     CUDADMA_REQUIRE(run->call_style == CUDADMA_CALL_UNQUALIFIED,

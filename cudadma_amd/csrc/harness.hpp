@@ -64,13 +64,13 @@ __device__ __forceinline__ void do_transfer(Obj& dma, const int call_style, cons
   }
 }
 
-template<typename Obj>
+template<int STORE_QUAL = STORE_LDS_DIRECT, typename Obj>
 __device__ __forceinline__ void do_transfer_direct(Obj& dma, const int two_phase, const void* src, void* dst)
 {
   if (two_phase) {
-    dma.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS_DIRECT>(src);
-    dma.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS_DIRECT>(dst);
-  } else dma.template execute_dma<true, LOAD_CACHE_ALL, STORE_LDS_DIRECT>(src, dst);
+    dma.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_QUAL>(src);
+    dma.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_QUAL>(dst);
+  } else dma.template execute_dma<true, LOAD_CACHE_ALL, STORE_QUAL>(src, dst);
 }
 
 template<typename Obj>

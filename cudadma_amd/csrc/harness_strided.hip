@@ -85,6 +85,11 @@ __global__ void __launch_bounds__(1024) strided_kernel(const Args a)
     char* dst = a.reverse ? a.out + (size_t)rep * a.out_bytes + a.dst_offset : (char*)lds + a.dst_offset;
     if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
       if constexpr (A == 16 || A == 4) harness::do_transfer_direct(dma, a.two_phase, src, dst);
+    } else if (a.call_style == CUDADMA_CALL_LDS_SWIZZLE) {
+      if constexpr ((E % A) == 0) harness::do_transfer_direct<STORE_LDS_SWIZZLE>(dma, a.two_phase, src, dst);
+    } else if (a.call_style == CUDADMA_CALL_LDS_DIRECT_SWIZZLE) {
+      if constexpr ((A == 16 || A == 4) && (E % A) == 0)
+        harness::do_transfer_direct<STORE_LDS_DIRECT_SWIZZLE>(dma, a.two_phase, src, dst);
     } else {
       harness::do_transfer(dma, a.call_style, a.two_phase, src, dst);
     }

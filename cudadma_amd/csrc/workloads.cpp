@@ -58,6 +58,9 @@ static const VariantInfo kStrided[] = {
   {"manual double buffer, unpadded LDS rows (256 B): shows the bank-conflict cost"},
   {"double buffer: two DMA groups of 1 wavefront, one CudaDMAStrided object and one padded LDS tile each"},
   {"not warp-specialised: all four wavefronts move the tile and write it out, next tile requested two-phase"},
+  {"two DMA groups, unpadded 256 B LDS rows filled by global_load_lds_dwordx4 with XOR-swizzled chunks "
+   "(STORE_LDS_DIRECT_SWIZZLE): no VGPR staging, no padding, no bank conflicts"},
+  {"two DMA groups, unpadded 256 B LDS rows with XOR-swizzled chunks written from registers (STORE_LDS_SWIZZLE)"},
 };
 static const VariantInfo kGather[] = {
   {"manual 4-stage buffering: one DMA group of 2 wavefronts, four CudaDMAIndirect objects"},

@@ -33,7 +33,7 @@ __device__ __forceinline__ void tile_coords(const int t, const int tiles_per_sid
   ty = band * band_rows + (in_band - tx * band_rows);
 }
 
-template<int LDS_ROW_BYTES, typename Dma>
+template<int LDS_ROW_BYTES, bool SWIZZLED = false, typename Dma>
 __device__ __forceinline__ void write_tile_transposed(const char* lds_tile, float* __restrict__ out, const int n,
                                                       const int ty, const int tx, const Dma& dma)
 {
@@ -41,9 +41,12 @@ __device__ __forceinline__ void write_tile_transposed(const char* lds_tile, floa
   const int lane = threadIdx.x & 63;
   const int w = threadIdx.x >> 6;
   vec4_t v[8];
-  const vec4_t* row = (const vec4_t*)(lds_tile + lane * LDS_ROW_BYTES) + w * 8;
+  // SWIZZLED: the 16-byte unit c of row r sits at unit c ^ (r & 15) of the unpadded 256-byte row
+  // (hipdma::swizzled_chunk), so the sixteen lanes of a quarter wavefront still hit sixteen
+  // different units.
+  const vec4_t* row = (const vec4_t*)(lds_tile + lane * LDS_ROW_BYTES);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) v[j] = row[j];
+  for (int j = 0; j < 8; ++j) v[j] = row[SWIZZLED ? hipdma::swizzled_chunk(lane, w * 8 + j, kRowBytes / 16) : (w * 8 + j)];
   dma.start_async_dma();
   // element (r = lane, c) of the tile goes to out[(tx*64 + c) * n + ty*64 + r]
   float* o = out + (size_t)(tx * kTile + w * 32) * n + (size_t)ty * kTile + lane;
@@ -122,7 +125,7 @@ transpose_manual_double(const float* __restrict__ in, float* __restrict__ out, c
 // issue order and s_waitcnt counts them in that order, so a wavefront that owns a
 // single object waits for exactly its own tile; the second tile in flight belongs
 // to the other wavefront.  Each DMA thread holds a whole tile share of 16 dwordx4.
-template<int LDS_ROW_BYTES>
+template<int LDS_ROW_BYTES, int SQ = STORE_LDS>
 __global__ void __launch_bounds__(kDmaThreads + kComputeThreads)
 transpose_double_groups(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles,
                         const int band)
@@ -141,12 +144,12 @@ transpose_double_groups(const float* __restrict__ in, float* __restrict__ out, c
     return (const void*)(in + (size_t)ty * kTile * n + (size_t)tx * kTile);
   };
   auto dma_loop = [&](dma_t& dma, char* buf, int t) {
-    if (t < num_tiles) dma.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t));
+    if (t < num_tiles) dma.template start_xfer_async<true, LOAD_CACHE_ALL, SQ>(src_of(t));
     for (; t + 2 * stride < num_tiles; t += 2 * stride) {
-      dma.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf);
-      dma.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t + 2 * stride));
+      dma.template wait_xfer_finish<true, LOAD_CACHE_ALL, SQ>(buf);
+      dma.template start_xfer_async<true, LOAD_CACHE_ALL, SQ>(src_of(t + 2 * stride));
     }
-    if (t < num_tiles) dma.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf);
+    if (t < num_tiles) dma.template wait_xfer_finish<true, LOAD_CACHE_ALL, SQ>(buf);
   };
   if (dma0.owns_this_thread()) {
     dma_loop(dma0, buf0, blockIdx.x);
@@ -159,11 +162,11 @@ transpose_double_groups(const float* __restrict__ in, float* __restrict__ out, c
       int ty, tx;
       tile_coords(t, tiles_per_side, band, ty, tx);
       dma0.wait_for_dma_finish();
-      write_tile_transposed<LDS_ROW_BYTES>(buf0, out, n, ty, tx, dma0);
+      write_tile_transposed<LDS_ROW_BYTES, hipdma::detail::store_is_swizzled(SQ)>(buf0, out, n, ty, tx, dma0);
       if (t + stride < num_tiles) {
         tile_coords(t + stride, tiles_per_side, band, ty, tx);
         dma1.wait_for_dma_finish();
-        write_tile_transposed<LDS_ROW_BYTES>(buf1, out, n, ty, tx, dma1);
+        write_tile_transposed<LDS_ROW_BYTES, hipdma::detail::store_is_swizzled(SQ)>(buf1, out, n, ty, tx, dma1);
       }
     }
   }
@@ -264,6 +267,8 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
     case 1: hipLaunchKernelGGL(transpose_single, dim3(workloads::persistent_grid(tiles, 8)), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 2: hipLaunchKernelGGL(transpose_manual_double<256>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 3: hipLaunchKernelGGL(transpose_double_groups<272>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 5: hipLaunchKernelGGL((transpose_double_groups<256, STORE_LDS_DIRECT_SWIZZLE>), dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 6: hipLaunchKernelGGL((transpose_double_groups<256, STORE_LDS_SWIZZLE>), dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
     default: hipLaunchKernelGGL(transpose_not_specialized, dim3(workloads::persistent_grid(tiles, 6)), block, 0, s, d_in, d_out, n, tiles, band); break;
   }
   CUDADMA_HIP_CHECK(hipGetLastError());

@@ -49,7 +49,12 @@ enum {
   CUDADMA_CALL_UNQUALIFIED  = 0,  /* execute_dma(src,dst)                                  */
   CUDADMA_CALL_GLOBAL       = 1,  /* execute_dma<true>(src,dst)                            */
   CUDADMA_CALL_QUALIFIED    = 2,  /* execute_dma<true,LOAD_CACHE_STREAMING,STORE_LDS>      */
-  CUDADMA_CALL_LDS_DIRECT   = 3   /* execute_dma<true,LOAD_CACHE_ALL,STORE_LDS_DIRECT>     */
+  CUDADMA_CALL_LDS_DIRECT   = 3,  /* execute_dma<true,LOAD_CACHE_ALL,STORE_LDS_DIRECT>     */
+  /* strided cases whose rows are whole chunks: the chunks of LDS row r are permuted,
+   * chunk c at position c ^ (r & mask), mask = largest power of two <= 16 dividing the
+   * chunks per row, minus one (hipdma::swizzled_chunk in include/hipdma/base.hpp) */
+  CUDADMA_CALL_LDS_SWIZZLE  = 4,  /* execute_dma<true,LOAD_CACHE_ALL,STORE_LDS_SWIZZLE>        */
+  CUDADMA_CALL_LDS_DIRECT_SWIZZLE = 5  /* execute_dma<true,LOAD_CACHE_ALL,STORE_LDS_DIRECT_SWIZZLE> */
 };
 
 typedef struct cudadma_case {

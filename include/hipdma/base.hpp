@@ -68,6 +68,12 @@ enum CudaDMALoadQualifier {
 //                     Needs a global source; nothing can be issued before the
 //                     buffer is free, so start_xfer_async() only records the
 //                     source and wait_xfer_finish() issues the loads.
+//   STORE_LDS_SWIZZLE / STORE_LDS_DIRECT_SWIZZLE  (CudaDMAStrided) the same two,
+//                     with the ALIGNMENT-byte chunks of every LDS row permuted:
+//                     chunk c of row r lands at chunk hipdma::swizzled_chunk(r, c, n)
+//                     of the row, n = chunks per row.  Unpadded power-of-two rows
+//                     (which is what the direct path needs) can then be read down a
+//                     column without bank conflicts.  Rows must be whole chunks.
 enum CudaDMAStoreQualifier {
   STORE_WRITE_BACK,
   STORE_CACHE_GLOBAL,
@@ -75,6 +81,8 @@ enum CudaDMAStoreQualifier {
   STORE_CACHE_WRITE_THROUGH,
   STORE_LDS,
   STORE_LDS_DIRECT,
+  STORE_LDS_SWIZZLE,
+  STORE_LDS_DIRECT_SWIZZLE,
 };
 
 namespace hipdma {
@@ -153,7 +161,24 @@ __host__ __device__ constexpr int pow2_divisor(int v, int cap)
   return p;
 }
 
+// The store qualifiers that only exist here, sorted into what they imply.
+__host__ __device__ constexpr bool store_is_lds(int q)
+{ return q == STORE_LDS || q == STORE_LDS_DIRECT || q == STORE_LDS_SWIZZLE || q == STORE_LDS_DIRECT_SWIZZLE; }
+__host__ __device__ constexpr bool store_is_direct(int q) { return q == STORE_LDS_DIRECT || q == STORE_LDS_DIRECT_SWIZZLE; }
+__host__ __device__ constexpr bool store_is_swizzled(int q) { return q == STORE_LDS_SWIZZLE || q == STORE_LDS_DIRECT_SWIZZLE; }
+
 }  // namespace detail
+
+// XOR mask of the swizzled LDS layouts for rows of `chunks_per_row` chunks: the largest power
+// of two (at most 16) that divides the row, minus one, so that the permutation never leaves
+// an aligned group of chunks inside the row.
+__host__ __device__ constexpr int swizzle_mask(int chunks_per_row)
+{ return chunks_per_row > 0 ? detail::pow2_divisor(chunks_per_row, 16) - 1 : 0; }
+// Where chunk `chunk` of row `row` sits inside its LDS row after a swizzled transfer
+// (and, the permutation being an involution, which chunk sits at position `chunk`).
+__host__ __device__ constexpr int swizzled_chunk(int row, int chunk, int chunks_per_row)
+{ return chunk ^ (row & swizzle_mask(chunks_per_row)); }
+
 }  // namespace hipdma
 
 // Base of every DMA object: role test and the empty/full handshake.

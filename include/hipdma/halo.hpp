@@ -191,6 +191,7 @@ public:
   __device__ __forceinline__ void start_xfer_async(const void* __restrict__ src_origin)
   {
     static_assert(DMA_STORE_QUAL != STORE_LDS_DIRECT, "the halo ring is too ragged for the direct path");
+    static_assert(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), "swizzled LDS rows are a CudaDMAStrided layout");
     m_src = (const char*)src_origin;
     pass<true, DMA_GLOBAL_LOAD, DMA_LOAD_QUAL, DMA_STORE_QUAL>(0, nullptr);
   }

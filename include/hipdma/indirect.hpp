@@ -113,6 +113,7 @@ public:
   {
     static_assert(DMA_STORE_QUAL != STORE_LDS_DIRECT || (GATHER && DMA_GLOBAL_LOAD),
                   "STORE_LDS_DIRECT needs a gather from a global source");
+    static_assert(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), "swizzled LDS rows are a CudaDMAStrided layout");
     m_index = index_ptr;
     m_src = (const char*)src_ptr;
     if (use_direct<DMA_STORE_QUAL>()) return;

@@ -54,7 +54,7 @@ __device__ __forceinline__ T load_vec(const void* ptr)
 template<typename T, int STORE_QUAL>
 __device__ __forceinline__ void store_vec(const T& value, void* ptr)
 {
-  if constexpr (STORE_QUAL == STORE_LDS || STORE_QUAL == STORE_LDS_DIRECT) {
+  if constexpr (store_is_lds(STORE_QUAL)) {
     *(HIPDMA_LDS_AS T*)ptr = value;
   } else if constexpr (STORE_QUAL == STORE_CACHE_STREAMING) {
     __builtin_nontemporal_store(value, (T*)ptr);

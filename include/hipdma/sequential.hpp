@@ -120,6 +120,7 @@ public:
   template<bool DMA_GLOBAL_LOAD, int DMA_LOAD_QUAL, int DMA_STORE_QUAL>
   __device__ __forceinline__ void start_xfer_async(const void* __restrict__ src_ptr)
   {
+    static_assert(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), "swizzled LDS rows are a CudaDMAStrided layout");
     m_src = (const char*)src_ptr;
     if constexpr (DMA_STORE_QUAL != STORE_LDS_DIRECT)
       load_step<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL>(0);

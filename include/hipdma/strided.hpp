@@ -153,11 +153,13 @@ public:
   __device__ __forceinline__ void wait_xfer_finish(void* __restrict__ dst_ptr)
   {
     if constexpr (DO_SYNC) CudaDMA::wait_for_dma_start();
+    static_assert(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL) || (BYTES_PER_ELMT % ALIGNMENT) == 0,
+                  "swizzled LDS rows must be whole chunks");
     if (use_direct<DMA_STORE_QUAL>()) {
-      if constexpr (DMA_STORE_QUAL == STORE_LDS_DIRECT) {
-        static_assert(DMA_STORE_QUAL != STORE_LDS_DIRECT || DMA_GLOBAL_LOAD,
+      if constexpr (hipdma::detail::store_is_direct(DMA_STORE_QUAL)) {
+        static_assert(!hipdma::detail::store_is_direct(DMA_STORE_QUAL) || DMA_GLOBAL_LOAD,
                       "STORE_LDS_DIRECT needs a global source");
-        direct_all((char*)dst_ptr);
+        direct_all<hipdma::detail::store_is_swizzled(DMA_STORE_QUAL)>((char*)dst_ptr);
       }
     } else {
       hipdma::detail::GridCursor cur = m_grid.begin();
@@ -187,7 +189,7 @@ private:
   template<int STORE_QUAL>
   __device__ __forceinline__ bool use_direct() const
   {
-    if constexpr (STORE_QUAL == STORE_LDS_DIRECT && (ALIGNMENT == 16 || ALIGNMENT == 4))
+    if constexpr (hipdma::detail::store_is_direct(STORE_QUAL) && (ALIGNMENT == 16 || ALIGNMENT == 4))
       return (m_grid.last_bytes == ALIGNMENT) && ((m_grid.T % HIPDMA_WAVE_SIZE) == 0) &&
              ((m_grid.W >= HIPDMA_WAVE_SIZE) ||
               ((m_grid.W == m_grid.LPE) && (m_dst_stride == m_grid.E)));
@@ -217,11 +219,23 @@ private:
     for (int k = 0; k < MAX_LDS; ++k) {
       if (m_grid.live(step * MAX_LDS + k, cur))
         store_chunk<ALIGNMENT, ALIGNMENT, STORE_QUAL>(
-            m_buf[k], dst + cur.row * m_dst_stride + cur.col * ALIGNMENT, m_grid.chunk_bytes(ALIGNMENT, cur));
+            m_buf[k], dst + cur.row * m_dst_stride + lds_col<store_is_swizzled(STORE_QUAL)>(cur) * ALIGNMENT,
+            m_grid.chunk_bytes(ALIGNMENT, cur));
       m_grid.advance(cur);
     }
   }
 
+  // Chunk position inside the LDS row for the chunk at cursor c.
+  template<bool SWIZZLE>
+  __device__ __forceinline__ int lds_col(const hipdma::detail::GridCursor& c) const
+  {
+    if constexpr (SWIZZLE) return hipdma::swizzled_chunk(c.row, c.col, m_grid.LPE);
+    else return c.col;
+  }
+
+  // Lane L of a wavefront always lands on LDS chunk (base + L); with SWIZZLE the lane
+  // fetches the source chunk that belongs at its landing position instead.
+  template<bool SWIZZLE>
   __device__ __forceinline__ void direct_all(char* dst)
   {
     using namespace hipdma::detail;
@@ -231,7 +245,7 @@ private:
       if (m_grid.live(r, cur)) {
         const int lds_off = cur.row * m_dst_stride + cur.col * ALIGNMENT;
         if constexpr (ALIGNMENT == 16 || ALIGNMENT == 4)
-          load_to_lds<ALIGNMENT>(m_src + cur.row * m_src_stride + cur.col * ALIGNMENT,
+          load_to_lds<ALIGNMENT>(m_src + cur.row * m_src_stride + lds_col<SWIZZLE>(cur) * ALIGNMENT,
                                  dst + (lds_off - lane * ALIGNMENT));
       }
       m_grid.advance(cur);

@@ -111,6 +111,24 @@ void oracle_strided(const void* src, void* dst, int elmt_bytes, int num_elmts, i
       d[(size_t)r * dst_stride + j] = s[(size_t)r * src_stride + j];
 }
 
+/* The swizzled LDS layout of CudaDMAStrided's STORE_LDS_SWIZZLE / STORE_LDS_DIRECT_SWIZZLE
+ * qualifiers (an addition of this library, no reference lines): the same rows as
+ * oracle_strided, with the chunks of destination row r permuted by XOR with r & mask. */
+void oracle_strided_swizzled(const void* src, void* dst, int elmt_bytes, int num_elmts, int src_stride, int dst_stride,
+                             int chunk)
+{
+  const unsigned char* s = (const unsigned char*)src;
+  unsigned char* d = (unsigned char*)dst;
+  const int chunks = elmt_bytes / chunk;
+  int p = 16;
+  while (p > 1 && (chunks % p) != 0) p >>= 1;
+  const int mask = chunks > 0 ? p - 1 : 0;
+  for (int r = 0; r < num_elmts; ++r)
+    for (int c = 0; c < chunks; ++c)
+      for (int b = 0; b < chunk; ++b)
+        d[(size_t)r * dst_stride + (size_t)((c ^ (r & mask)) * chunk) + b] = s[(size_t)r * src_stride + (size_t)c * chunk + b];
+}
+
 /* CudaDMAIndirect<GATHER=true>: row r comes from element index[r] of the source;
  * rows land max(alt_stride, elmt_bytes) apart.
  * include/cudaDMAv2.h:9940-9957 (offset = index_ptr[...]; src_ptr + offset*BYTES_PER_ELMT),

@@ -40,6 +40,12 @@ float oracle_bf16_to_f32(uint16_t v);
 /* ---- transfer patterns (one DMA object, one transfer) ---- */
 void oracle_sequential(const void* src, void* dst, size_t bytes);
 void oracle_strided(const void* src, void* dst, int elmt_bytes, int num_elmts, int src_stride, int dst_stride);
+/* strided transfer into swizzled LDS rows: chunk c (of `chunk` bytes) of row r lands at chunk
+ * c ^ (r & mask) of the destination row, mask = (largest power of two <= 16 dividing the
+ * chunks per row) - 1.  No counterpart in the reference: it states the layout of the
+ * STORE_LDS_SWIZZLE qualifiers of include/hipdma/base.hpp.  elmt_bytes must be a multiple of chunk. */
+void oracle_strided_swizzled(const void* src, void* dst, int elmt_bytes, int num_elmts, int src_stride, int dst_stride,
+                             int chunk);
 void oracle_gather(const int32_t* index, const void* src, void* dst, int elmt_bytes, int num_elmts, int alt_stride);
 void oracle_scatter(const int32_t* index, const void* src, void* dst, int elmt_bytes, int num_elmts, int alt_stride);
 void oracle_halo(const void* src_origin, void* dst_origin, int elmt_bytes, int radius, int corners,

@@ -87,7 +87,7 @@ class CaseIO:
             self.input = ol.uniform(in_bytes // 4, 4242 + flavour).view(np.uint8)
 
     # -- the closed form, applied by the oracle to byte buffers -------------------------------
-    def apply_oracle(self, src, dst, rep, shift_src=True):
+    def apply_oracle(self, src, dst, rep, shift_src=True, swizzle=False):
         """Moves what the case's object moves: src/dst are numpy uint8 arrays standing for
         the source and the destination buffer of one transfer."""
         O = ol.load()
@@ -98,6 +98,8 @@ class CaseIO:
         idx = self.index[rep * self.rep_index_elmts:] if self.index is not None else None
         if c.pattern == cd.PATTERN_SEQUENTIAL:
             O.oracle_sequential(ptr(src, so), ptr(dst, do), e)
+        elif c.pattern == cd.PATTERN_STRIDED and swizzle:
+            O.oracle_strided_swizzled(ptr(src, so), ptr(dst, do), e, n, self.src_stride, self.dst_stride, c.alignment)
         elif c.pattern == cd.PATTERN_STRIDED:
             O.oracle_strided(ptr(src, so), ptr(dst, do), e, n, self.src_stride, self.dst_stride)
         elif c.pattern == cd.PATTERN_GATHER:
@@ -109,7 +111,7 @@ class CaseIO:
             O.oracle_halo(ptr(src, so + (r * self.pitch + r) * e), ptr(dst, do + (r * (c.dimx + 2 * r) + r) * e),
                           e, r, c.corners, c.dimx, c.dimy, self.pitch)
 
-    def expected(self):
+    def expected(self, swizzle=False):
         if self.reverse:
             out = np.zeros((self.reps, self.out_bytes), dtype=np.uint8)
             for rep in range(self.reps):
@@ -118,7 +120,7 @@ class CaseIO:
             return out
         out = np.zeros((self.reps, self.lds_bytes), dtype=np.uint8)
         for rep in range(self.reps):
-            self.apply_oracle(self.input, out[rep], rep)
+            self.apply_oracle(self.input, out[rep], rep, swizzle=swizzle)
         return out
 
     def expected_map(self, rep=0):

@@ -21,6 +21,7 @@ _SIGS = {
     "oracle_bf16_to_f32": (ctypes.c_float, [ctypes.c_uint16]),
     "oracle_sequential": (None, [_vp, _vp, _cs]),
     "oracle_strided": (None, [_vp, _vp, _ci, _ci, _ci, _ci]),
+    "oracle_strided_swizzled": (None, [_vp, _vp, _ci, _ci, _ci, _ci, _ci]),
     "oracle_gather": (None, [_vp, _vp, _vp, _ci, _ci, _ci]),
     "oracle_scatter": (None, [_vp, _vp, _vp, _ci, _ci, _ci]),
     "oracle_halo": (None, [_vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci]),

@@ -20,6 +20,10 @@ def _styles(case):
     styles = [cd.CALL_UNQUALIFIED, cd.CALL_GLOBAL, cd.CALL_QUALIFIED]
     if case.pattern in (cd.PATTERN_SEQUENTIAL, cd.PATTERN_STRIDED, cd.PATTERN_GATHER) and case.alignment in (4, 16):
         styles.append(cd.CALL_LDS_DIRECT)
+    if case.pattern == cd.PATTERN_STRIDED and case.bytes_per_elmt % case.alignment == 0:
+        styles.append(cd.CALL_LDS_SWIZZLE)                    # permuted chunks, through registers
+        if case.alignment in (4, 16):
+            styles.append(cd.CALL_LDS_DIRECT_SWIZZLE)         # permuted chunks, global_load_lds where the shape allows
     return styles
 
 
@@ -32,7 +36,7 @@ def test_case_matches_oracle(case_id, device):
             for two_phase in (False, True):
                 io = CaseIO(case, flavour=flavour, reps=3, data=data)
                 flavour += 1
-                want = io.expected()
+                want = io.expected(swizzle=style in (cd.CALL_LDS_SWIZZLE, cd.CALL_LDS_DIRECT_SWIZZLE))
                 d_in = torch.from_numpy(io.input).to(device)
                 d_idx = torch.from_numpy(io.index).to(device) if io.index is not None else None
                 d_out = torch.full((io.reps * io.lds_bytes,), 0xEE, dtype=torch.uint8, device=device)

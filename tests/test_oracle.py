@@ -427,3 +427,29 @@ def test_golden_sgemv_of_the_reference_driver(O):
     y = np.empty(n, dtype=np.float32)
     O.oracle_sgemv(n, m, float(g["alpha"]), ptr(a), n, ptr(x), ptr(y))
     assert [int(v) for v in y] == g["y"]
+
+
+# ---- the swizzled LDS layout (an addition of this library) ----
+
+@pytest.mark.parametrize("chunk,chunks,mask", [(16, 16, 15), (16, 8, 7), (16, 20, 3), (4, 64, 15), (8, 1, 0), (16, 6, 1), (4, 5, 0)])
+def test_strided_swizzled_is_a_row_wise_xor_permutation(O, chunk, chunks, mask):
+    e, n = chunk * chunks, 37
+    ss, ds = e + 3 * chunk, e + chunk
+    rng = np.random.default_rng(chunks)
+    src = rng.integers(0, 256, size=n * ss, dtype=np.uint8)
+    plain = np.zeros(n * ds, dtype=np.uint8)
+    swz = np.zeros(n * ds, dtype=np.uint8)
+    O.oracle_strided(ptr(src), ptr(plain), e, n, ss, ds)
+    O.oracle_strided_swizzled(ptr(src), ptr(swz), e, n, ss, ds, chunk)
+    p = plain.reshape(n, ds)[:, :e].reshape(n, chunks, chunk)
+    s = swz.reshape(n, ds)[:, :e].reshape(n, chunks, chunk)
+    pos = np.arange(chunks)[None, :] ^ (np.arange(n)[:, None] & mask)       # position of chunk c in row r
+    assert pos.max() < chunks
+    want = np.empty_like(p)
+    want[np.arange(n)[:, None], pos] = p                                     # numpy scatter, no oracle arithmetic
+    assert np.array_equal(s, want)
+    assert np.array_equal(swz.reshape(n, ds)[:, e:], plain.reshape(n, ds)[:, e:])   # padding untouched
+    # an involution: reading position c ^ (r & mask) gives chunk c back
+    assert np.array_equal(s[np.arange(n)[:, None], pos], p)
+    if mask:
+        assert not np.array_equal(s, p)
