@@ -21,6 +21,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0           # MI355X published HBM3E bandwidth
+SETTLE_MS = 30.0                # wall time of untimed warm-up for the secondary patterns
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # scaled by what the same counters read for the plain copy kernel (see profiles/).
@@ -32,11 +33,18 @@ def log(msg):
     print(msg, file=sys.stderr, flush=True)
 
 
-def time_launches(fn, steps, warmup):
-    """Average milliseconds per launch, HIP events on the launch stream around `steps` launches."""
+def time_launches(fn, steps, warmup, settle_ms=0.0):
+    """Average milliseconds per launch, HIP events on the launch stream around `steps` launches.
+    `settle_ms` > 0 keeps the untimed warm-up going for that much wall time (used for the
+    secondary patterns: the first launches after an allocation phase run up to 25 % slow)."""
     import torch
-    for _ in range(warmup):
+    t0 = time.perf_counter()
+    done = 0
+    while done < warmup or (time.perf_counter() - t0) * 1e3 < settle_ms:
         fn()
+        done += 1
+        if done % 8 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     start = torch.cuda.Event(enable_timing=True)
     stop = torch.cuda.Event(enable_timing=True)
@@ -146,7 +154,7 @@ def main():
     strided_bytes = 2 * n * n * 4
     report("strided", strided_ms, strided_bytes, "CudaDMAStrided 64x256B tiles of a 16384^2 f32 matrix, transposed out")
     # yardstick on the same buffers: plain dwordx4 copy
-    copy_ms, _ = time_launches(lambda: wl.plain_copy(src, dst), steps, warmup)
+    copy_ms, _ = time_launches(lambda: wl.plain_copy(src, dst), steps, warmup, SETTLE_MS)
     report("plain_copy", copy_ms, strided_bytes, "grid-stride dwordx4 copy of 1 GiB, no LDS, no DMA object")
     del src, dst
 
@@ -154,7 +162,7 @@ def main():
     m = 64 * 1024 * 1024 // 4
     s_src = wl.fill_uniform(torch.empty(m, dtype=torch.float32, device=dev), 1001)
     s_dst = torch.empty_like(s_src)
-    ms, _ = time_launches(lambda: wl.sequential_copy(s_src, s_dst, 0), max(steps, 50), warmup)
+    ms, _ = time_launches(lambda: wl.sequential_copy(s_src, s_dst, 0), max(steps, 50), warmup, SETTLE_MS)
     report("sequential", ms, 2 * m * 4, "CudaDMASequential 16 KiB tiles of a 64 MiB f32 buffer (fits the 256 MB Infinity Cache)")
     del s_src, s_dst
 
@@ -163,7 +171,7 @@ def main():
     table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev), 1003)
     idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=dev), recs, 1003)
     sums = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, dtype=torch.float32, device=dev)
-    ms, _ = time_launches(lambda: wl.gather_rowsum(table, idx, sums, 0), steps, warmup)
+    ms, _ = time_launches(lambda: wl.gather_rowsum(table, idx, sums, 0), steps, warmup, SETTLE_MS)
     report("gather", ms, n_idx * 4 + n_idx * 128 + sums.numel() * 4,
            "CudaDMAIndirect 32 x 128 B records per tile from a 512 MiB table, row-sum consumer")
     del table, idx, sums
@@ -173,10 +181,10 @@ def main():
     p = 2 * wl.STENCIL_RADIUS
     grid_in = wl.fill_uniform(torch.empty((g + p) ** 3, dtype=torch.float32, device=dev), 1004).view(g + p, g + p, g + p)
     grid_out = torch.empty((g, g, g), dtype=torch.float32, device=dev)
-    ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 0), steps, warmup)
+    ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 0), steps, warmup, SETTLE_MS)
     report("halo", ms, 2 * g ** 3 * 4, "CudaDMAHalo radius-4 ring of 32x32 tiles, 25-point stencil on a 512^3 f32 grid "
            "(ring landed without handshake, one s_barrier per plane)")
-    ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 1), steps, warmup)
+    ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 1), steps, warmup, SETTLE_MS)
     report("halo_handshake", ms, 2 * g ** 3 * 4, "same kernel with the empty/full handshake on the LDS planes next to the s_barrier")
     del grid_in, grid_out
 
@@ -185,8 +193,7 @@ def main():
     ga = torch.randn((dim, dim), device=dev, dtype=torch.float32).to(torch.bfloat16)
     gb = torch.randn((dim, dim), device=dev, dtype=torch.float32).to(torch.bfloat16)
     gc = torch.empty((dim, dim), device=dev, dtype=torch.float32)
-    # the matrix cores' clock settles only after a few tens of launches: longer untimed warm-up
-    ms, _ = time_launches(lambda: wl.gemm_bf16(ga, gb, gc), max(steps, 50), max(warmup, 30))
+    ms, _ = time_launches(lambda: wl.gemm_bf16(ga, gb, gc), max(steps, 50), warmup, SETTLE_MS)
     flops = 2.0 * dim ** 3
     gemm = {"TFLOP/s": round(flops / ms / 1e9, 1), "frac_of_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4),
             "ms": round(ms, 4), "flop": flops,

@@ -17,9 +17,17 @@ from . import workloads as wl
 PEAK_GBS = 8000.0
 
 
-def _time(fn, steps, warmup=3):
-    for _ in range(warmup):
+def _time(fn, steps, warmup=3, settle_ms=30.0):
+    """Average milliseconds per launch.  Warm-up runs for at least `warmup` launches and `settle_ms`
+    of wall time: the first launches after an idle or allocation phase run up to 25 % slow."""
+    import time
+    t0 = time.perf_counter()
+    done = 0
+    while done < warmup or (time.perf_counter() - t0) * 1e3 < settle_ms:
         fn()
+        done += 1
+        if done % 8 == 0:
+            torch.cuda.synchronize()
     torch.cuda.synchronize()
     a = torch.cuda.Event(enable_timing=True)
     b = torch.cuda.Event(enable_timing=True)
