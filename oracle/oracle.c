@@ -221,16 +221,29 @@ void oracle_copy(const float* in, float* out, size_t n)
   for (long long i = 0; i < (long long)n; ++i) out[i] = in[i];
 }
 
-/* Config 2: out = in^T for an n x n row-major matrix, blocked for the cache. */
+/* Config 2: out = in^T for an n x n row-major matrix.  Two levels of blocking: 256 x 256
+ * tiles keep the pages touched on both sides within the reach of the TLB, and inside a tile
+ * 16 x 16 blocks go through a local buffer so that every cache line of the input is read
+ * once and every cache line of the output is written once and whole (with a power-of-two
+ * row pitch the rows of a block fall into the same cache set: a line must not be revisited). */
 void oracle_transpose(const float* in, float* out, int n)
 {
-  const int B = 64;
+  enum { T = 256, B = 16 };
+  const int nt = (n + T - 1) / T;
 #pragma omp parallel for collapse(2) schedule(static)
-  for (int rb = 0; rb < n; rb += B)
-    for (int cb = 0; cb < n; cb += B)
-      for (int r = rb; r < rb + B && r < n; ++r)
-        for (int c = cb; c < cb + B && c < n; ++c)
-          out[(size_t)c * n + r] = in[(size_t)r * n + c];
+  for (int tr = 0; tr < nt; ++tr)
+    for (int tc = 0; tc < nt; ++tc) {
+      const int r_end = (tr * T + T < n) ? tr * T + T : n, c_end = (tc * T + T < n) ? tc * T + T : n;
+      for (int r0 = tr * T; r0 < r_end; r0 += B)
+        for (int c0 = tc * T; c0 < c_end; c0 += B) {
+          float tmp[B][B];
+          const int nr = (r_end - r0 < B) ? r_end - r0 : B, nc = (c_end - c0 < B) ? c_end - c0 : B;
+          for (int r = 0; r < nr; ++r)
+            for (int c = 0; c < nc; ++c) tmp[r][c] = in[(size_t)(r0 + r) * n + (size_t)(c0 + c)];
+          for (int c = 0; c < nc; ++c)
+            for (int r = 0; r < nr; ++r) out[(size_t)(c0 + c) * n + (size_t)(r0 + r)] = tmp[r][c];
+        }
+    }
 }
 
 /* Config 3, record check: out[i] = table[idx[i]] */
