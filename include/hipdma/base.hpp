@@ -47,6 +47,17 @@
 #define HIPDMA_SPIN_LIMIT (1 << 24)
 #endif
 
+// DEBUG_CUDADMA (the reference's switch, include/cudaDMAv2.h:1564-1576) turns the
+// preconditions the objects rely on into device-side asserts: thread groups made of whole
+// wavefronts, dmaID in range, sizes in multiples of 4 bytes, pointers and strides aligned
+// to ALIGNMENT.  Without it nothing is checked, as in the reference.
+#ifdef DEBUG_CUDADMA
+#include <cassert>
+#define HIPDMA_ASSERT(cond) assert(cond)
+#else
+#define HIPDMA_ASSERT(cond) ((void)0)
+#endif
+
 // Load cache policies (names follow include/cudaDMAv2.h:50-56).  On gfx950:
 //   LOAD_CACHE_ALL / LOAD_CACHE_GLOBAL  plain load
 //   LOAD_CACHE_STREAMING / _LAST_USE    non-temporal load (nt bit)
@@ -202,6 +213,10 @@ public:
   {
     // A DMA thread waits on `empty` for the compute threads, a compute thread
     // waits on `full` for the DMA threads.
+    HIPDMA_ASSERT(dmaID >= 0 && dmaID < HIPDMA_MAX_DMA_IDS);
+    HIPDMA_ASSERT(num_dma_threads > 0 && (num_dma_threads % HIPDMA_WAVE_SIZE) == 0);
+    HIPDMA_ASSERT((dma_threadIdx_start % HIPDMA_WAVE_SIZE) == 0);
+    HIPDMA_ASSERT(num_compute_threads > 0);
     m_wait_unit = m_is_dma_thread ? unsigned(num_compute_threads) : unsigned(num_dma_threads);
     if (threadIdx.x == 0) {
       *m_full = 0u;

@@ -192,6 +192,7 @@ public:
   {
     static_assert(DMA_STORE_QUAL != STORE_LDS_DIRECT, "the halo ring is too ragged for the direct path");
     static_assert(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), "swizzled LDS rows are a CudaDMAStrided layout");
+    HIPDMA_ASSERT((reinterpret_cast<uintptr_t>(src_origin) % ALIGNMENT) == 0);
     m_src = (const char*)src_origin;
     pass<true, DMA_GLOBAL_LOAD, DMA_LOAD_QUAL, DMA_STORE_QUAL>(0, nullptr);
   }
@@ -215,6 +216,9 @@ private:
                                        const int pitch)
   {
     using namespace hipdma::detail;
+    HIPDMA_ASSERT(threads > 0 && (threads % HIPDMA_WAVE_SIZE) == 0);
+    HIPDMA_ASSERT(dimx > 0 && dimy > 0 && pitch >= dimx + 2 * RADIUS);
+    HIPDMA_ASSERT(((pitch * BYTES_PER_ELMT) % ALIGNMENT) == 0);
     m_tid = int(threadIdx.x) - start;
     m_threads = threads;
     m_geom.init(dimx, dimy, pitch);

@@ -114,6 +114,7 @@ public:
     static_assert(DMA_STORE_QUAL != STORE_LDS_DIRECT || (GATHER && DMA_GLOBAL_LOAD),
                   "STORE_LDS_DIRECT needs a gather from a global source");
     static_assert(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), "swizzled LDS rows are a CudaDMAStrided layout");
+    HIPDMA_ASSERT(index_ptr != nullptr && (reinterpret_cast<uintptr_t>(src_ptr) % ALIGNMENT) == 0);
     m_index = index_ptr;
     m_src = (const char*)src_ptr;
     if (use_direct<DMA_STORE_QUAL>()) return;
@@ -142,6 +143,9 @@ private:
 
   __device__ __forceinline__ void init(const int e, const int n, const int t, const int start, const int alt)
   {
+    HIPDMA_ASSERT(e >= 0 && (e % 4) == 0 && n >= 0);
+    HIPDMA_ASSERT(t > 0 && (t % HIPDMA_WAVE_SIZE) == 0);
+    HIPDMA_ASSERT((alt % ALIGNMENT) == 0);
     m_grid.init(ALIGNMENT, MAX_LDS, e, n, t, int(threadIdx.x) - start);
     m_dense_stride = (alt > e) ? alt : e;
   }

@@ -121,6 +121,7 @@ public:
   __device__ __forceinline__ void start_xfer_async(const void* __restrict__ src_ptr)
   {
     static_assert(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), "swizzled LDS rows are a CudaDMAStrided layout");
+    HIPDMA_ASSERT((reinterpret_cast<uintptr_t>(src_ptr) % ALIGNMENT) == 0);
     m_src = (const char*)src_ptr;
     if constexpr (DMA_STORE_QUAL != STORE_LDS_DIRECT)
       load_step<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL>(0);
@@ -149,6 +150,8 @@ private:
 
   __device__ __forceinline__ void init(const int bytes, const int threads, const int start)
   {
+    HIPDMA_ASSERT(bytes >= 0 && (bytes % 4) == 0);
+    HIPDMA_ASSERT(threads > 0 && (threads % HIPDMA_WAVE_SIZE) == 0);
     m_bytes = bytes;
     m_threads = threads;
     m_tid = int(threadIdx.x) - start;

@@ -144,6 +144,7 @@ public:
   template<bool DMA_GLOBAL_LOAD, int DMA_LOAD_QUAL, int DMA_STORE_QUAL>
   __device__ __forceinline__ void start_xfer_async(const void* __restrict__ src_ptr)
   {
+    HIPDMA_ASSERT((reinterpret_cast<uintptr_t>(src_ptr) % ALIGNMENT) == 0);
     m_src = (const char*)src_ptr;
     if (use_direct<DMA_STORE_QUAL>()) return;
     load_step<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL>(0, m_grid.begin());
@@ -152,6 +153,8 @@ public:
   template<bool DMA_GLOBAL_LOAD, int DMA_LOAD_QUAL, int DMA_STORE_QUAL>
   __device__ __forceinline__ void wait_xfer_finish(void* __restrict__ dst_ptr)
   {
+    HIPDMA_ASSERT((reinterpret_cast<uintptr_t>(dst_ptr) % ALIGNMENT) == 0);
+    HIPDMA_ASSERT(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL) || (m_grid.E % ALIGNMENT) == 0);
     if constexpr (DO_SYNC) CudaDMA::wait_for_dma_start();
     static_assert(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL) || (BYTES_PER_ELMT % ALIGNMENT) == 0,
                   "swizzled LDS rows must be whole chunks");
@@ -178,6 +181,9 @@ private:
   __device__ __forceinline__ void init(const int e, const int n, const int t, const int start,
                                        const int src_stride, const int dst_stride)
   {
+    HIPDMA_ASSERT(e >= 0 && (e % 4) == 0 && n >= 0);
+    HIPDMA_ASSERT(t > 0 && (t % HIPDMA_WAVE_SIZE) == 0);
+    HIPDMA_ASSERT((src_stride % ALIGNMENT) == 0 && (dst_stride % ALIGNMENT) == 0);
     m_grid.init(ALIGNMENT, MAX_LDS, e, n, t, int(threadIdx.x) - start);
     m_src_stride = src_stride;
     m_dst_stride = dst_stride;
