@@ -150,3 +150,51 @@ def test_replay_rejects_a_window_that_is_too_small():
     with pytest.raises(cd.CudaDMAError, match="outside"):
         cd.plan.plan_map(cd.PATTERN_SEQUENTIAL, alignment=16, bytes_per_thread=64, bytes_per_elmt=4096,
                          dma_threads=64, map_len=1024)
+
+
+_DROP_IN_KERNEL = r"""
+#include "%s"
+// the shape of the reference's special_xfer_* test kernels: objects built by every thread, roles split after
+__global__ void k(const float* in, const int* idx, float* out)
+{
+  __shared__ float buf[4096];
+  CudaDMASequential<true, 16, 64, 1024, 64> a(0, 64, 64);
+  CudaDMAStrided<true, 16, 64, 256, 64, 8> b(1, 64, 64, 1024, 272);
+  CudaDMAIndirect<true, true, 16, 64, 128, 64, 8> c(2, 64, 64);
+  CudaDMAHalo<true, 16, 64, 4, 64, 4, false, 32, 32> h(3, 64, 64, 48);
+  cudaDMACustom d(4, 64, 64, 64);
+  if (a.owns_this_thread()) {
+    a.execute_dma(in, buf);
+    b.execute_dma<true>(in, buf);
+    c.execute_dma<true, LOAD_CACHE_STREAMING, STORE_WRITE_BACK>(idx, in, buf);
+    h.execute_dma(in + 1024, buf + 512);
+    d.wait_for_dma_start(); d.finish_async_dma();
+  } else {
+    a.start_async_dma(); a.wait_for_dma_finish();
+    b.start_async_dma(); b.wait_for_dma_finish();
+    c.start_async_dma(); c.wait_for_dma_finish();
+    h.start_async_dma(); h.wait_for_dma_finish();
+    d.start_async_dma(); d.wait_for_dma_finish();
+    out[threadIdx.x] = buf[threadIdx.x];
+  }
+}
+static_assert(WARP_SIZE == 64, "thread groups are sized in wavefronts");
+"""
+
+
+@pytest.mark.parametrize("header,flags", [("cudaDMAv2.h", []), ("hipDMA.h", ["-DWARP_SIZE=64"]), ("cudaDMA.h", []),
+                                          ("cudaDMAv2.h", ["-DDEBUG_CUDADMA"])])
+def test_headers_compile_standalone_for_gfx950(tmp_path, header, flags):
+    """The drop-in boundary is the include line: a kernel that names only the reference's header must build
+    (device pass only, no GPU needed), also with the reference's DEBUG_CUDADMA switch."""
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("no hipcc")
+    src = tmp_path / "drop_in.hip"
+    src.write_text(_DROP_IN_KERNEL % header)
+    cmd = [hipcc, "-std=c++17", "-O1", "--offload-arch=gfx950", "--cuda-device-only", "-c", str(src), "-o", str(tmp_path / "k.o"),
+           "-I", os.path.join(ROOT, "include"), "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"] + flags
+    res = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-2000:]
