@@ -5,6 +5,7 @@ point; here the variants are compiled in and the occupancy is a run-time knob.
 
     python -m cudadma_amd.sweep [sequential] [strided] [gather] [halo] [gemm] [--wg 0,2,4,8] [--steps 20]
     python -m cudadma_amd.sweep saxpy sgemv stencil2d        # the reference's example programs, every variant
+    python -m cudadma_amd.sweep perf_sequential --wg 2,8     # read-bandwidth probe: element size x DMA wavefronts x buffering
 """
 import argparse
 import sys
@@ -103,6 +104,24 @@ def main(argv=None):
             c = torch.empty(n, n, device=dev)
             ms = _time(lambda: wl.gemm_bf16(a, b, c), args.steps)
             print(f"gemm       variant 0  {ms:9.4f} ms  {2.0 * n ** 3 / ms / 1e9:8.1f} TFLOP/s", flush=True)
+        elif name == "perf_sequential":
+            # src/perf/sequential/param_sweep.py:27-58: element size x DMA wavefronts x workgroups per CU x
+            # buffering; a launch reads 1 GiB whatever the point (loop count follows from that)
+            src = wl.fill_uniform(torch.empty(1 << 28, device=dev), 1001)
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            print("# read bandwidth into LDS, GB/s (1 GiB per launch); columns: buffering none / single / double / manual")
+            for elmt in (32, 128, 512, 2048, 4096, 8192, 16384):
+                for waves in (1, 2, 4):
+                    for wg in wgs if wgs != [0] else [4]:
+                        wg = wg or 4
+                        groups = cus * wg
+                        loops = max(1, (1 << 30) // (groups * elmt))
+                        cells = []
+                        for b in range(4):
+                            nbytes = wl.perf_sequential(src, elmt, waves, b, loops, groups)
+                            ms = _time(lambda: wl.perf_sequential(src, elmt, waves, b, loops, groups), args.steps, settle_ms=5.0)
+                            cells.append(f"{nbytes / ms / 1e6:7.0f}")
+                        print(f"elmt {elmt:6d} B  dma waves {waves}  wg/cu {wg:2d}  loops {loops:6d}  " + " ".join(cells), flush=True)
         elif name == "saxpy":
             # bytes as the reference's driver counts them: x read, y read, y written (saxpy_cudaDMA.cu:192)
             n = 1 << 28

@@ -117,6 +117,24 @@ def halo_stencil(grid_in, grid_out, variant=0):
     return grid_out
 
 
+BUFFERING_NONE, BUFFERING_SINGLE, BUFFERING_DOUBLE, BUFFERING_MANUAL = range(4)
+BUFFERING_NAMES = ("none", "single", "double", "manual")
+
+
+def perf_sequential(src, elmt_bytes, dma_wavefronts, buffering, loop_iters, workgroups, sums=None):
+    """The read-bandwidth probe of the sequential object (all parameters at run time).  Returns the
+    bytes one launch reads.  `sums` (uint32/int32, one zeroed word per workgroup) switches the checksum on."""
+    if not (src.is_cuda and src.is_contiguous()):
+        raise ValueError("src must be a contiguous CUDA tensor")
+    if sums is not None and not (sums.is_cuda and sums.is_contiguous() and sums.element_size() == 4 and sums.numel() >= workgroups):
+        raise ValueError("sums must hold one 32-bit word per workgroup")
+    n = lib().cudadma_perf_sequential(_p(src), src.numel() * src.element_size(), _p(sums) if sums is not None else None,
+                                      elmt_bytes, dma_wavefronts, buffering, loop_iters, workgroups, _stream())
+    if n < 0:
+        check(int(n))
+    return int(n)
+
+
 def gemm_bf16(a, b, c, variant=0):
     """a: (m, k) and b: (k, n) torch.bfloat16, c: (m, n) float32; returns c = a @ b with fp32 accumulation."""
     _need(a, torch.bfloat16, "a")

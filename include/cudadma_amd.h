@@ -196,6 +196,24 @@ int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz
 int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k,
                       int variant, void* stream);
 
+/* ---- read-bandwidth probe with run-time parameters ------------------------------------
+ * src/perf/sequential/perf_sequential.cu:52-228 with the macros of params_directed.h as
+ * arguments: every workgroup brings loop_iters consecutive elements of elmt_bytes into
+ * LDS with CudaDMASequential (run-time size and thread count), one compute wavefront
+ * standing for the consumer.  buffering picks the kernel shape of the reference's four.
+ * Returns the bytes read (workgroups * elmt_bytes * loop_iters) or a negative CUDADMA_E*
+ * code.  d_sums may be NULL (pure probe, nothing is written, as in the reference); otherwise
+ * it holds one zero-initialised word per workgroup, to which the 32-bit words that arrived
+ * in LDS are added. */
+enum {
+  CUDADMA_BUFFERING_NONE   = 0,  /* not warp-specialised, two workgroup barriers per element */
+  CUDADMA_BUFFERING_SINGLE = 1,  /* one buffer, one object                                    */
+  CUDADMA_BUFFERING_DOUBLE = 2,  /* two buffers, two objects on disjoint DMA wavefronts       */
+  CUDADMA_BUFFERING_MANUAL = 3   /* two buffers, two objects on the same DMA wavefronts       */
+};
+long long cudadma_perf_sequential(const void* d_src, size_t src_bytes, unsigned* d_sums, int elmt_bytes,
+                                  int dma_wavefronts, int buffering, int loop_iters, int workgroups, void* stream);
+
 /* ---- known-answer cases for the first-generation class names -------------------------
  * One transfer per case by cudaDMASequential / cudaDMAStrided / cudaDMAIndirect as declared in
  * include/cudaDMA.h:644-3580 (every constructor form), into a 16 KiB LDS window that holds the

@@ -270,3 +270,32 @@ def test_gemm_rejects_ragged_shapes(device):
     c = torch.zeros((100, 128), dtype=torch.float32, device=device)
     with pytest.raises(cd.CudaDMAError, match="multiples"):
         wl.gemm_bf16(a, b, c)
+
+
+# ------------------------------------------------------------------ read-bandwidth probe (perf_sequential)
+@pytest.mark.parametrize("buffering", range(4))
+@pytest.mark.parametrize("elmt,waves,loops,groups", [(32, 1, 1, 3), (48, 2, 5, 7), (4096, 2, 8, 64), (16384, 4, 3, 33),
+                                                     (2064, 7, 2, 5), (16, 1, 9, 2)])
+def test_perf_sequential_checksum(device, buffering, elmt, waves, loops, groups):
+    """Every byte of every element reaches LDS: per-workgroup sum of the 32-bit words, modulo 2^32."""
+    total = groups * elmt * loops
+    rng = np.random.default_rng(elmt + waves)
+    words = rng.integers(0, 2 ** 32, size=total // 4 + 64, dtype=np.uint64).astype(np.uint32)
+    src = torch.from_numpy(words.view(np.int32)).to(device)
+    sums = torch.zeros(groups, dtype=torch.int32, device=device)
+    print(f"perf_sequential elmt {elmt} waves {waves} loops {loops} groups {groups} buffering {buffering}", flush=True)
+    n = wl.perf_sequential(src, elmt, waves, buffering, loops, groups, sums)
+    torch.cuda.synchronize()
+    assert n == total
+    want = words[:total // 4].reshape(groups, -1).astype(np.uint64).sum(axis=1).astype(np.uint32)
+    assert np.array_equal(sums.cpu().numpy().view(np.uint32), want)
+
+
+def test_perf_sequential_argument_checks(device):
+    src = torch.zeros(1024, dtype=torch.int32, device=device)
+    with pytest.raises(cd.CudaDMAError, match="multiple of 16"):
+        wl.perf_sequential(src, 40, 1, 0, 1, 1)
+    with pytest.raises(cd.CudaDMAError, match="must be 16-byte aligned and hold"):
+        wl.perf_sequential(src, 4096, 1, 1, 2, 1)
+    with pytest.raises(cd.CudaDMAError, match="unknown buffering"):
+        wl.perf_sequential(src, 64, 1, 4, 1, 1)
