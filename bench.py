@@ -25,8 +25,8 @@ SETTLE_MS = 30.0                # wall time of untimed warm-up for the secondary
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # scaled by what the same counters read for the plain copy kernel (see profiles/).
-# profiles/bench_all_patterns_mi355x.md: FETCH_SIZE 524384 KiB x 2.0000 + WRITE_SIZE 1048576 KiB x 1.0000.
-MEASURED_TRAFFIC_BYTES = {"strided": 2147680256}
+# profiles/bench_all_patterns_mi355x.md: FETCH_SIZE 524393 KiB x 1.99995 + WRITE_SIZE 1048576 KiB x 1.00000.
+MEASURED_TRAFFIC_BYTES = {"strided": 2147667896}
 
 
 def log(msg):
