@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one launch of the CudaDMAStrided tile-transpose kernel over the whole
-16384 x 16384 float32 matrix (BASELINE config 2, the configuration the metric is
+16384 x 16384 float32 matrix (benchmark config 2, the configuration the metric is
 quoted on); inputs are resident in HBM before the timed region.  The other three
 HBM-bound patterns (sequential copy, indirect gather, halo stencil) and a plain
 copy kernel are timed the same way and reported under "patterns".  One JSON line
@@ -218,7 +218,7 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "CudaDMAStrided 2D tile extraction: 16384x16384 f32, 64 rows x 256 B tiles, "
-                               "double-buffered, transposed to output (BASELINE configs[1])",
+                               "double-buffered, transposed to output (benchmark config 2 of 5)",
                    "tile_rows": 64, "tile_row_bytes": 256, "src_stride_bytes": 65536,
                    "workgroup": "128 DMA + 128 compute threads"},
         "roofline": {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",

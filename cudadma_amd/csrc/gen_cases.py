@@ -7,7 +7,7 @@ ALIGNMENT in {4,8,16}, BYTES_PER_THREAD = ALIGNMENT * U{1..8}, element size
 |N(256,256)| floats, NUM_ELMTS ~ U{1..32}, DMA warps ~ U{1..16}; here it is a
 fixed, seeded list instead of an endless loop, wavefronts have 64 lanes, and the
 template level and the warp-specialised flag cycle so that every constructor
-form is compiled.  A directed part pins the BASELINE shapes and the edge cases
+form is compiled.  A directed part pins the full benchmark shapes and the edge cases
 (4/8/12-byte tails, one element, one wavefront, many steps).
 
 Run from this directory:  python3 gen_cases.py
@@ -37,7 +37,7 @@ def sequential_cases():
     out = []
     directed = [
         # ws level A  BPT   E     T
-        (1, 3, 16, 128, 16384, 128),   # BASELINE config 1 tile: 8 dwordx4 per lane, one step
+        (1, 3, 16, 128, 16384, 128),   # benchmark config 1 tile: 8 dwordx4 per lane, one step
         (1, 3, 16, 64, 16384, 128),    # same tile in two steps
         (1, 2, 16, 32, 16384, 64),     # one wavefront, many steps
         (1, 1, 16, 16, 4, 64),         # smallest transfer
@@ -67,9 +67,9 @@ def grid_cases(seed, n_random, with_gather):
     combos = [(ws, lv) for ws in (1, 0) for lv in (1, 2, 3, 4)]
     directed = [
         # ws lv  A  BPT   E    T   N
-        (1, 4, 16, 128, 256, 128, 64),    # BASELINE config 2 tile: 64 rows x 256 B, one step
+        (1, 4, 16, 128, 256, 128, 64),    # benchmark config 2 tile: 64 rows x 256 B, one step
         (1, 4, 16, 64, 256, 128, 64),     # same in two steps
-        (1, 4, 16, 64, 128, 128, 32),     # BASELINE config 3 tile: 32 records x 128 B
+        (1, 4, 16, 64, 128, 128, 32),     # benchmark config 3 tile: 32 records x 128 B
         (1, 3, 16, 64, 128, 128, 128),    # GEMM A tile: 128 rows x 128 B
         (1, 2, 16, 64, 4, 64, 1), (1, 1, 16, 64, 12, 64, 7), (0, 4, 16, 32, 20, 64, 5),
         (1, 4, 16, 32, 2048, 128, 3),     # rows wider than one wavefront load
@@ -98,7 +98,7 @@ def halo_cases():
     out = []
     # ws level A BPT ES T R C DX DY
     directed = [
-        (1, 3, 16, 64, 4, 128, 4, 0, 32, 32),   # BASELINE config 4 ring
+        (1, 3, 16, 64, 4, 128, 4, 0, 32, 32),   # benchmark config 4 ring
         (1, 3, 16, 16, 4, 64, 4, 0, 32, 32),    # same ring, one load per step
         (1, 2, 16, 64, 4, 128, 4, 1, 32, 32),
         (1, 0, 4, 16, 4, 64, 1, 0, 8, 8), (1, 0, 4, 16, 4, 128, 3, 1, 17, 9),

@@ -1,5 +1,5 @@
 """GPU parity of the five benchmark workloads, called through the C ABI.
-Small shapes are compared with the oracle element by element; the BASELINE shapes are
+Small shapes are compared with the oracle element by element; the full benchmark shapes are
 checked through properties that do not need a host pass over gigabytes where one would
 be slow (double transpose = identity, gather of identity indices = table, linearity)."""
 import numpy as np
@@ -161,7 +161,7 @@ def test_gather_full_size(device):
 
 
 # ------------------------------------------------------------------ config 4
-STENCIL_RTOL = 1e-5       # BASELINE config 4: fp32 within 1e-5 relative of the host reference
+STENCIL_RTOL = 1e-5       # benchmark config 4: fp32 within 1e-5 relative of the host reference
 
 
 @pytest.mark.parametrize("variant", _variants(wl.HALO))
@@ -204,7 +204,7 @@ def test_halo_stencil_full_size(device):
 
 
 # ------------------------------------------------------------------ config 5
-GEMM_RTOL = 1e-2          # BASELINE config 5: within 1e-2 relative of the fp32 host GEMM
+GEMM_RTOL = 1e-2          # benchmark config 5: within 1e-2 relative of the fp32 host GEMM
 
 
 def _bf16_inputs(m, n, k):
