@@ -58,3 +58,25 @@ def test_captured_workloads_replay_like_eager_launches(device):
         for name, got, ref in zip(("transpose", "sequential", "gather", "halo", "saxpy"), (out_t, out_s, out_g, out_h, y), want):
             assert torch.equal(got.view(torch.int32), ref.view(torch.int32)), f"{name}, replay {replay}"
     assert torch.equal(out_t, src.t())
+
+
+def test_workloads_on_two_streams_at_once(device):
+    """The handshake words live in each kernel's own LDS, so kernels of different workloads running
+    concurrently on two streams cannot disturb each other."""
+    n, recs, n_idx = 2048, 1 << 16, 32 * 4096
+    src = wl.fill_uniform(torch.empty(n * n, dtype=torch.float32, device=device), 21).view(n, n)
+    table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=device), 22)
+    idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=device), recs, 22)
+    out_t = torch.empty_like(src)
+    out_g = torch.empty(n_idx * wl.REC_FLOATS, dtype=torch.float32, device=device)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    for _ in range(10):
+        with torch.cuda.stream(s1):
+            wl.strided_transpose(src, out_t, 0)
+        with torch.cuda.stream(s2):
+            wl.gather_copy(table, idx, out_g, 0)
+    torch.cuda.synchronize()
+    assert torch.equal(out_t, src.t())
+    want = table.view(recs, wl.REC_FLOATS)[idx.long()].reshape(-1)
+    assert torch.equal(out_g.view(torch.int32), want.view(torch.int32))
