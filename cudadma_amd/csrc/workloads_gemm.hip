@@ -34,8 +34,8 @@ struct GemmShape {
   static constexpr int kBPitch = kBN * 2 + 64;      // B row in LDS: the four rows a transposing read touches land 64 B apart modulo 256
   static constexpr int kAStage = kBM * kAPitch;
   static constexpr int kBStage = kBK * kBPitch;
-  typedef CudaDMAStrided<true, 16, kBM * kBK * 2 / kDmaWave, kBK * 2, kDmaWave, kBM> dma_a_t;   // kBM rows x 128 B
-  typedef CudaDMAStrided<true, 16, kBK * kBN * 2 / kDmaWave, kBN * 2, kDmaWave, kBK> dma_b_t;   // 64 rows x 2*kBN B
+  typedef CudaDMAStrided<false, 16, kBM * kBK * 2 / kDmaWave, kBK * 2, kDmaWave, kBM> dma_a_t;   // kBM rows x 128 B
+  typedef CudaDMAStrided<false, 16, kBK * kBN * 2 / kDmaWave, kBN * 2, kDmaWave, kBK> dma_b_t;   // 64 rows x 2*kBN B
 };
 
 // Workgroup -> tile.  Workgroup b runs on XCD b % 8; when the tile grid divides into eight
@@ -80,10 +80,15 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
   constexpr int kAPitch = shape::kAPitch, kBPitch = shape::kBPitch;
   __shared__ __attribute__((aligned(16))) char lds_a[2][shape::kAStage];
   __shared__ __attribute__((aligned(16))) char lds_b[2][shape::kBStage];
-  dma_a_t dma_a0(0, kComputeThreads, kComputeThreads, k * 2, kAPitch);
-  dma_a_t dma_a1(1, kComputeThreads, kComputeThreads, k * 2, kAPitch);
-  dma_b_t dma_b0(2, kComputeThreads, kComputeThreads + kDmaWave, n * 2, kBPitch);
-  dma_b_t dma_b1(3, kComputeThreads, kComputeThreads + kDmaWave, n * 2, kBPitch);
+  // The transfer objects carry no handshake of their own: a stage holds an A tile and a B tile,
+  // and one sync object per stage covers the four DMA wavefronts of both operands, so the
+  // compute wavefronts wait and signal once per stage instead of once per operand.
+  dma_a_t dma_a0(k * 2, kAPitch, kComputeThreads);
+  dma_a_t dma_a1(k * 2, kAPitch, kComputeThreads);
+  dma_b_t dma_b0(n * 2, kBPitch, kComputeThreads + kDmaWave);
+  dma_b_t dma_b1(n * 2, kBPitch, kComputeThreads + kDmaWave);
+  cudaDMACustom stage0(0, 2 * kDmaWave, kComputeThreads, kComputeThreads);
+  cudaDMACustom stage1(1, 2 * kDmaWave, kComputeThreads, kComputeThreads);
   int tile_m, tile_n;
   tile_of_workgroup(blockIdx.x, m / shape::kBM, n / shape::kBN, tile_m, tile_n);
   const int ksteps = k / kBK;            // even: k is a multiple of 2 * kBK
@@ -96,9 +101,13 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
     d0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src);
     d1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src + step);
     for (int kt = 0; kt < ksteps; kt += 2) {
+      stage0.wait_for_dma_start();
       d0.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(s0);
+      stage0.finish_async_dma();
       d0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src + (size_t)(kt + 2 < klast ? kt + 2 : klast) * step);
+      stage1.wait_for_dma_start();
       d1.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(s1);
+      stage1.finish_async_dma();
       d1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src + (size_t)(kt + 3 < klast ? kt + 3 : klast) * step);
     }
   };
@@ -118,8 +127,8 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
     // both stages are free to begin with
-    dma_a0.start_async_dma(); dma_a1.start_async_dma();
-    dma_b0.start_async_dma(); dma_b1.start_async_dma();
+    stage0.start_async_dma();
+    stage1.start_async_dma();
     // A fragment: row wm + 32*i + lane%32, eight k starting at 16*ks + 8*(lane/32)
     const int a_off = (wm + (lane & 31)) * kAPitch + (lane >> 5) * 16;
     // B fragment through the transposing read: inside a group of 16 lanes, lane j points at
@@ -173,43 +182,37 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
     static_assert(kBK / 16 == 4, "the slice schedule below is written for four slices per stage");
     if constexpr (!kPinned) {
       for (int kt = 0; kt < ksteps; kt += 2) {
-        dma_a0.wait_for_dma_finish();
-        dma_b0.wait_for_dma_finish();
+        stage0.wait_for_dma_finish();
 #pragma unroll
         for (int ks = 0; ks < kBK / 16; ++ks) { load_frags(fa0, fb0, sa0, sb0, ks); multiply(fa0, fb0); }
-        dma_a0.start_async_dma();
-        dma_b0.start_async_dma();
-        dma_a1.wait_for_dma_finish();
-        dma_b1.wait_for_dma_finish();
+        stage0.start_async_dma();
+        stage1.wait_for_dma_finish();
 #pragma unroll
         for (int ks = 0; ks < kBK / 16; ++ks) { load_frags(fa0, fb0, sa1, sb1, ks); multiply(fa0, fb0); }
-        dma_a1.start_async_dma();
-        dma_b1.start_async_dma();
+        stage1.start_async_dma();
       }
     } else {
-      dma_a0.wait_for_dma_finish();
-      dma_b0.wait_for_dma_finish();
+      stage0.wait_for_dma_finish();
       load_frags(fa0, fb0, sa0, sb0, 0);
       for (int kt = 0; kt < ksteps; kt += 2) {
         load_frags(fa1, fb1, sa0, sb0, 1); multiply(fa0, fb0); interleave();
         load_frags(fa0, fb0, sa0, sb0, 2); multiply(fa1, fb1); interleave();
+        // the `full` word of the next stage is read here and looked at one slice later
+        const unsigned seen1 = stage1.peek_dma_finish();
         load_frags(fa1, fb1, sa0, sb0, 3); multiply(fa0, fb0); interleave();
-        dma_a1.wait_for_dma_finish();
-        dma_b1.wait_for_dma_finish();
+        stage1.wait_for_dma_finish(seen1);
         load_frags(fa0, fb0, sa1, sb1, 0); multiply(fa1, fb1); interleave();
-        dma_a0.start_async_dma();
-        dma_b0.start_async_dma();
+        stage0.start_async_dma();
         load_frags(fa1, fb1, sa1, sb1, 1); multiply(fa0, fb0); interleave();
         load_frags(fa0, fb0, sa1, sb1, 2); multiply(fa1, fb1); interleave();
+        const unsigned seen0 = stage0.peek_dma_finish();
         load_frags(fa1, fb1, sa1, sb1, 3); multiply(fa0, fb0); interleave();
         if (kt + 2 < ksteps) {
-          dma_a0.wait_for_dma_finish();
-          dma_b0.wait_for_dma_finish();
+          stage0.wait_for_dma_finish(seen0);
           load_frags(fa0, fb0, sa0, sb0, 0);
         }
         multiply(fa1, fb1); interleave();
-        dma_a1.start_async_dma();
-        dma_b1.start_async_dma();
+        stage1.start_async_dma();
       }
     }
     // 32 x 32 block: register e of lane L holds row 8*(e/4) + 4*(L/32) + e%4, column L%32

@@ -104,6 +104,13 @@ int cudadma_run_case(int case_id, const cudadma_run_t* run, void* stream);
  * kernel must end; d_flags[0] (DMA side) and d_flags[1] (compute side) are then 1. */
 int cudadma_selftest_bounded_wait(int* d_flags, void* stream);
 
+/* The split wait that only exists here (peek_dma_finish() + wait_for_dma_finish(peeked),
+ * include/hipdma/base.hpp): one workgroup hands a 64-word buffer from a DMA wavefront to a
+ * compute wavefront `phases` times, the DMA side early on even and late on odd phases.
+ * d_out (two zeroed ints): [0] = words the compute side saw wrong (must be 0), [1] = phases in
+ * which the peek already found the buffer full. */
+int cudadma_selftest_split_wait(int* d_out, int phases, void* stream);
+
 /* ------------------------------------------------------------------------
  * Host-side planner.  cudadma_diagnose prints what the static diagnose()
  * members of the objects print (include/cudaDMAv2.h:1402-1458, :3208-3493,

@@ -252,6 +252,22 @@ public:
       hipdma::detail::wait_word(m_full, m_wait_target);
     }
   }
+  // Compute side, the wait split in two so that the round trip to LDS can hide behind other
+  // work: peek_dma_finish() reads the `full` word without blocking, wait_for_dma_finish(peeked)
+  // later completes the wait (and only polls when the peeked value was not there yet).  An
+  // addition of this library: with named barriers there is nothing to peek at.
+  __device__ __forceinline__ unsigned peek_dma_finish(void) const
+  {
+    return m_has_sync ? __hip_atomic_load(m_full, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : 0u;
+  }
+  __device__ __forceinline__ void wait_for_dma_finish(const unsigned peeked) const
+  {
+    if (m_has_sync) {
+      m_wait_target += m_wait_unit;
+      if ((int)(peeked - m_wait_target) < 0) hipdma::detail::wait_word(m_full, m_wait_target);
+      else hipdma::detail::acquire_lds();
+    }
+  }
   __device__ __forceinline__ bool owns_this_thread(void) const { return m_is_dma_thread; }
   // DMA side: block until every compute thread has released the buffer.
   __device__ __forceinline__ void wait_for_dma_start(void) const

@@ -112,3 +112,16 @@ def test_unmatched_waits_end(device):
     cd._lib.check(cd.lib().cudadma_selftest_bounded_wait(ctypes.c_void_p(flags.data_ptr()), None))
     torch.cuda.synchronize()
     assert flags.tolist() == [1, 1]
+
+
+def test_split_wait_sees_every_phase(device):
+    """peek_dma_finish() + wait_for_dma_finish(peeked): the data of every phase is seen, both when the
+    peek already found the buffer full and when the wait has to poll."""
+    import ctypes
+    out = torch.zeros(2, dtype=torch.int32, device=device)
+    phases = 200
+    cd._lib.check(cd.lib().cudadma_selftest_split_wait(ctypes.c_void_p(out.data_ptr()), phases, None))
+    torch.cuda.synchronize()
+    wrong, early = out.tolist()
+    assert wrong == 0
+    assert 0 < early < phases, f"both branches of the split wait should have run ({early} early of {phases})"
