@@ -41,7 +41,7 @@ __device__ __forceinline__ void write_tile_transposed(const char* lds_tile, floa
   const int lane = threadIdx.x & 63;
   const int w = threadIdx.x >> 6;
   vec4_t v[8];
-  // SWIZZLED: the 16-byte unit c of row r sits at unit c ^ (r & 15) of the unpadded 256-byte row
+  // SWIZZLED: the 16-byte unit c of row r sits at unit c ^ bitreverse4(r & 15) of the unpadded 256-byte row
   // (hipdma::swizzled_chunk), so the sixteen lanes of a quarter wavefront still hit sixteen
   // different units.
   const vec4_t* row = (const vec4_t*)(lds_tile + lane * LDS_ROW_BYTES);

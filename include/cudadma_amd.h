@@ -50,9 +50,9 @@ enum {
   CUDADMA_CALL_GLOBAL       = 1,  /* execute_dma<true>(src,dst)                            */
   CUDADMA_CALL_QUALIFIED    = 2,  /* execute_dma<true,LOAD_CACHE_STREAMING,STORE_LDS>      */
   CUDADMA_CALL_LDS_DIRECT   = 3,  /* execute_dma<true,LOAD_CACHE_ALL,STORE_LDS_DIRECT>     */
-  /* strided cases whose rows are whole chunks: the chunks of LDS row r are permuted,
-   * chunk c at position c ^ (r & mask), mask = largest power of two <= 16 dividing the
-   * chunks per row, minus one (hipdma::swizzled_chunk in include/hipdma/base.hpp) */
+  /* strided cases whose rows are whole chunks: the chunks of LDS row r are permuted, chunk c
+   * at position c ^ key(r) (hipdma::swizzled_chunk in include/hipdma/base.hpp: key = bit-reversed
+   * low bits of the row number, as many bits as the row has aligned chunks, at most 256 bytes) */
   CUDADMA_CALL_LDS_SWIZZLE  = 4,  /* execute_dma<true,LOAD_CACHE_ALL,STORE_LDS_SWIZZLE>        */
   CUDADMA_CALL_LDS_DIRECT_SWIZZLE = 5  /* execute_dma<true,LOAD_CACHE_ALL,STORE_LDS_DIRECT_SWIZZLE> */
 };

@@ -81,7 +81,7 @@ enum CudaDMALoadQualifier {
 //                     source and wait_xfer_finish() issues the loads.
 //   STORE_LDS_SWIZZLE / STORE_LDS_DIRECT_SWIZZLE  (CudaDMAStrided) the same two,
 //                     with the ALIGNMENT-byte chunks of every LDS row permuted:
-//                     chunk c of row r lands at chunk hipdma::swizzled_chunk(r, c, n)
+//                     chunk c of row r lands at chunk hipdma::swizzled_chunk(r, c, n, ALIGNMENT)
 //                     of the row, n = chunks per row.  Unpadded power-of-two rows
 //                     (which is what the direct path needs) can then be read down a
 //                     column without bank conflicts.  Rows must be whole chunks.
@@ -180,15 +180,32 @@ __host__ __device__ constexpr bool store_is_swizzled(int q) { return q == STORE_
 
 }  // namespace detail
 
-// XOR mask of the swizzled LDS layouts for rows of `chunks_per_row` chunks: the largest power
-// of two (at most 16) that divides the row, minus one, so that the permutation never leaves
-// an aligned group of chunks inside the row.
-__host__ __device__ constexpr int swizzle_mask(int chunks_per_row)
-{ return chunks_per_row > 0 ? detail::pow2_divisor(chunks_per_row, 16) - 1 : 0; }
+// The swizzled LDS layouts.  The LDS has 64 banks of 4 bytes: addresses 256 bytes apart share
+// their banks.  For rows of `chunks_per_row` chunks of `chunk_bytes` bytes each:
+//   P     = the largest power of two that divides chunks_per_row and is at most 256/chunk_bytes
+//   shift = log2 of the rows that fit one 256-byte bank line, 256 / (P * chunk_bytes), at least 0
+//   key(row) = the low log2(P) bits of (row >> shift), bit-reversed
+// and chunk c of row r sits at chunk position c ^ key(r) of its row.  The permutation stays
+// inside aligned groups of P chunks (so inside the row), is its own inverse, and serves the
+// three ways a tile is read back: down a column (sixteen consecutive rows, one chunk each: the
+// keys are a bijection), row fragments of narrow rows (rows sharing a bank line get different
+// keys), and blocks of a few consecutive rows (bit reversal sends neighbouring rows to
+// opposite ends of the bank line).
+__host__ __device__ constexpr int swizzle_span(int chunks_per_row, int chunk_bytes)
+{ return chunks_per_row > 0 ? detail::pow2_divisor(chunks_per_row, 256 / chunk_bytes) : 1; }
+__host__ __device__ constexpr int swizzle_key(int row, int chunks_per_row, int chunk_bytes)
+{
+  const int span = swizzle_span(chunks_per_row, chunk_bytes);
+  if (span <= 1) return 0;
+  const int bits = __builtin_ctz((unsigned)span);
+  const int rows_per_line = 256 / (span * chunk_bytes);                 // a power of two, or 0 for rows beyond 256 bytes
+  const int shift = rows_per_line > 1 ? __builtin_ctz((unsigned)rows_per_line) : 0;
+  return (int)(__builtin_bitreverse32((unsigned)(row >> shift)) >> (32 - bits));
+}
 // Where chunk `chunk` of row `row` sits inside its LDS row after a swizzled transfer
 // (and, the permutation being an involution, which chunk sits at position `chunk`).
-__host__ __device__ constexpr int swizzled_chunk(int row, int chunk, int chunks_per_row)
-{ return chunk ^ (row & swizzle_mask(chunks_per_row)); }
+__host__ __device__ constexpr int swizzled_chunk(int row, int chunk, int chunks_per_row, int chunk_bytes = 16)
+{ return chunk ^ swizzle_key(row, chunks_per_row, chunk_bytes); }
 
 }  // namespace hipdma
 

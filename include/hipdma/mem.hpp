@@ -163,6 +163,15 @@ __device__ __forceinline__ void wait_lds_direct()
   __builtin_amdgcn_s_waitcnt(0x0F70);
 }
 
+// Wait until all but the YOUNGER most recent vector-memory operations of this wavefront have
+// completed (they complete in issue order).
+template<int YOUNGER>
+__device__ __forceinline__ void wait_lds_direct_but()
+{
+  static_assert(YOUNGER >= 0 && YOUNGER < 64, "vmcnt holds six bits");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (YOUNGER & 15) | ((YOUNGER >> 4) << 14));
+}
+
 // Lane number inside the wavefront.
 __device__ __forceinline__ int lane_id()
 {

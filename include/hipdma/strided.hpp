@@ -175,6 +175,31 @@ public:
     if constexpr (DO_SYNC) CudaDMA::finish_async_dma();
   }
 
+  // ---- direct-to-LDS transfers kept in flight (an addition of this library) ----
+  // The two-phase calls cannot request a STORE_LDS_DIRECT transfer before the handshake says the
+  // buffer is free, so with them a DMA wavefront has one direct transfer in flight at a time.  A
+  // kernel that does its own hand-off (a sync-only object, src/examples usage of cudaDMACustom)
+  // can keep several in flight: issue_direct() requests the whole transfer into a buffer the
+  // caller knows to be free and returns; the loads of a wavefront land in issue order, so
+  // hipdma::wait_direct_loads<YOUNGER>() waits for this transfer while the YOUNGER loads issued
+  // after it (loads_per_thread() of each later transfer) stay in flight.  Needs the shape the
+  // direct path needs (direct_ready()); neither call touches the handshake.
+  template<int DMA_STORE_QUAL = STORE_LDS_DIRECT>
+  __device__ __forceinline__ void issue_direct(const void* __restrict__ src_ptr, void* __restrict__ dst_ptr)
+  {
+    static_assert(hipdma::detail::store_is_direct(DMA_STORE_QUAL), "issue_direct takes one of the STORE_LDS_DIRECT qualifiers");
+    static_assert(ALIGNMENT == 16 || ALIGNMENT == 4, "global_load_lds moves 4 or 16 bytes per lane");
+    HIPDMA_ASSERT(direct_ready());
+    m_src = (const char*)src_ptr;
+    issue_direct_rounds<hipdma::detail::store_is_swizzled(DMA_STORE_QUAL)>((char*)dst_ptr);
+  }
+  // True when this object's shape can use global_load_lds (whole chunks, whole wavefronts, rows of
+  // at least a wavefront of chunks or unpadded power-of-two rows).
+  __device__ __forceinline__ bool direct_ready() const { return use_direct<STORE_LDS_DIRECT>(); }
+  // Loads each thread issues per transfer on the direct path (the unit of wait_direct_loads).
+  __host__ __device__ static constexpr int loads_per_thread()
+  { return hipdma::GridPlan(ALIGNMENT, BYTES_PER_THREAD, BYTES_PER_ELMT, DMA_THREADS, NUM_ELMTS).rounds; }
+
 private:
   __device__ __forceinline__ static int threads_or_block(const int n) { return (n <= 0) ? int(blockDim.x) : n; }
 
@@ -235,7 +260,7 @@ private:
   template<bool SWIZZLE>
   __device__ __forceinline__ int lds_col(const hipdma::detail::GridCursor& c) const
   {
-    if constexpr (SWIZZLE) return hipdma::swizzled_chunk(c.row, c.col, m_grid.LPE);
+    if constexpr (SWIZZLE) return hipdma::swizzled_chunk(c.row, c.col, m_grid.LPE, ALIGNMENT);
     else return c.col;
   }
 
@@ -243,6 +268,13 @@ private:
   // fetches the source chunk that belongs at its landing position instead.
   template<bool SWIZZLE>
   __device__ __forceinline__ void direct_all(char* dst)
+  {
+    issue_direct_rounds<SWIZZLE>(dst);
+    hipdma::detail::wait_lds_direct();
+  }
+
+  template<bool SWIZZLE>
+  __device__ __forceinline__ void issue_direct_rounds(char* dst)
   {
     using namespace hipdma::detail;
     const int lane = lane_id();
@@ -256,7 +288,6 @@ private:
       }
       m_grid.advance(cur);
     }
-    wait_lds_direct();
   }
 
 private:
@@ -266,6 +297,13 @@ private:
   const char* m_src;
   chunk_t m_buf[MAX_LDS];
 };
+
+namespace hipdma {
+// Waits until every direct-to-LDS load of the calling wavefront except the YOUNGER most recent
+// ones has landed (see CudaDMAStrided::issue_direct).
+template<int YOUNGER>
+__device__ __forceinline__ void wait_direct_loads() { detail::wait_lds_direct_but<YOUNGER>(); }
+}  // namespace hipdma
 
 // Host-side planner report (include/cudaDMAv2.h:3208-3493).
 template<bool DO_SYNC>

@@ -113,20 +113,37 @@ void oracle_strided(const void* src, void* dst, int elmt_bytes, int num_elmts, i
 
 /* The swizzled LDS layout of CudaDMAStrided's STORE_LDS_SWIZZLE / STORE_LDS_DIRECT_SWIZZLE
  * qualifiers (an addition of this library, no reference lines): the same rows as
- * oracle_strided, with the chunks of destination row r permuted by XOR with r & mask. */
+ * oracle_strided, with the chunks of destination row r permuted by XOR with key(r):
+ *   span  = largest power of two dividing the chunks per row, at most 256 / chunk
+ *   key   = the low log2(span) bits of r / (rows per 256-byte bank line), bit-reversed,
+ *           rows per bank line = max(1, 256 / (span * chunk)). */
+static int swizzle_key(int row, int chunks, int chunk)
+{
+  int span = 256 / chunk;
+  while (span > 1 && (chunks % span) != 0) span >>= 1;
+  if (chunks <= 0) span = 1;
+  int rows_per_line = 256 / (span * chunk);
+  if (rows_per_line < 1) rows_per_line = 1;
+  int v = row / rows_per_line, key = 0;
+  for (int bit = 1; bit < span; bit <<= 1) {
+    key = (key << 1) | (v & 1);
+    v >>= 1;
+  }
+  return key;
+}
+
 void oracle_strided_swizzled(const void* src, void* dst, int elmt_bytes, int num_elmts, int src_stride, int dst_stride,
                              int chunk)
 {
   const unsigned char* s = (const unsigned char*)src;
   unsigned char* d = (unsigned char*)dst;
   const int chunks = elmt_bytes / chunk;
-  int p = 16;
-  while (p > 1 && (chunks % p) != 0) p >>= 1;
-  const int mask = chunks > 0 ? p - 1 : 0;
-  for (int r = 0; r < num_elmts; ++r)
+  for (int r = 0; r < num_elmts; ++r) {
+    const int key = swizzle_key(r, chunks, chunk);
     for (int c = 0; c < chunks; ++c)
       for (int b = 0; b < chunk; ++b)
-        d[(size_t)r * dst_stride + (size_t)((c ^ (r & mask)) * chunk) + b] = s[(size_t)r * src_stride + (size_t)c * chunk + b];
+        d[(size_t)r * dst_stride + (size_t)((c ^ key) * chunk) + b] = s[(size_t)r * src_stride + (size_t)c * chunk + b];
+  }
 }
 
 /* CudaDMAIndirect<GATHER=true>: row r comes from element index[r] of the source;

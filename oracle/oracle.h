@@ -41,9 +41,10 @@ float oracle_bf16_to_f32(uint16_t v);
 void oracle_sequential(const void* src, void* dst, size_t bytes);
 void oracle_strided(const void* src, void* dst, int elmt_bytes, int num_elmts, int src_stride, int dst_stride);
 /* strided transfer into swizzled LDS rows: chunk c (of `chunk` bytes) of row r lands at chunk
- * c ^ (r & mask) of the destination row, mask = (largest power of two <= 16 dividing the
- * chunks per row) - 1.  No counterpart in the reference: it states the layout of the
- * STORE_LDS_SWIZZLE qualifiers of include/hipdma/base.hpp.  elmt_bytes must be a multiple of chunk. */
+ * c ^ key(r) of the destination row; key(r) = bit-reversed low bits of r / (rows per 256-byte
+ * bank line), as many bits as the row has aligned chunks (at most 256 bytes' worth).  No
+ * counterpart in the reference: it states the layout of the STORE_LDS_SWIZZLE qualifiers of
+ * include/hipdma/base.hpp.  elmt_bytes must be a multiple of chunk. */
 void oracle_strided_swizzled(const void* src, void* dst, int elmt_bytes, int num_elmts, int src_stride, int dst_stride,
                              int chunk);
 void oracle_gather(const int32_t* index, const void* src, void* dst, int elmt_bytes, int num_elmts, int alt_stride);

@@ -431,8 +431,19 @@ def test_golden_sgemv_of_the_reference_driver(O):
 
 # ---- the swizzled LDS layout (an addition of this library) ----
 
-@pytest.mark.parametrize("chunk,chunks,mask", [(16, 16, 15), (16, 8, 7), (16, 20, 3), (4, 64, 15), (8, 1, 0), (16, 6, 1), (4, 5, 0)])
-def test_strided_swizzled_is_a_row_wise_xor_permutation(O, chunk, chunks, mask):
+def _bitrev(v, bits):
+    out = 0
+    for _ in range(bits):
+        out = (out << 1) | (v & 1)
+        v >>= 1
+    return out
+
+
+# chunk bytes, chunks per row, bits of the key, rows per 256-byte bank line
+@pytest.mark.parametrize("chunk,chunks,bits,rows_per_line", [(16, 16, 4, 1), (16, 8, 3, 2), (16, 20, 2, 4), (4, 64, 6, 1),
+                                                              (8, 1, 0, 32), (16, 6, 1, 8), (4, 5, 0, 64), (16, 32, 4, 1),
+                                                              (4, 16, 4, 4)])
+def test_strided_swizzled_is_a_row_wise_xor_permutation(O, chunk, chunks, bits, rows_per_line):
     e, n = chunk * chunks, 37
     ss, ds = e + 3 * chunk, e + chunk
     rng = np.random.default_rng(chunks)
@@ -443,13 +454,25 @@ def test_strided_swizzled_is_a_row_wise_xor_permutation(O, chunk, chunks, mask):
     O.oracle_strided_swizzled(ptr(src), ptr(swz), e, n, ss, ds, chunk)
     p = plain.reshape(n, ds)[:, :e].reshape(n, chunks, chunk)
     s = swz.reshape(n, ds)[:, :e].reshape(n, chunks, chunk)
-    pos = np.arange(chunks)[None, :] ^ (np.arange(n)[:, None] & mask)       # position of chunk c in row r
+    key = np.array([_bitrev((r // rows_per_line) & ((1 << bits) - 1), bits) for r in range(n)])
+    pos = np.arange(chunks)[None, :] ^ key[:, None]                          # position of chunk c in row r
     assert pos.max() < chunks
     want = np.empty_like(p)
     want[np.arange(n)[:, None], pos] = p                                     # numpy scatter, no oracle arithmetic
     assert np.array_equal(s, want)
     assert np.array_equal(swz.reshape(n, ds)[:, e:], plain.reshape(n, ds)[:, e:])   # padding untouched
-    # an involution: reading position c ^ (r & mask) gives chunk c back
+    # an involution: reading position c ^ key(r) gives chunk c back
     assert np.array_equal(s[np.arange(n)[:, None], pos], p)
-    if mask:
+    if bits:
         assert not np.array_equal(s, p)
+
+
+def test_swizzle_keys_spread_over_the_bank_line():
+    """What the layout is for, checked on the key function alone: sixteen consecutive rows of a 256-byte row get
+    sixteen different keys (column reads), two rows sharing a bank line get the same key but sixteen consecutive
+    128-byte rows cover all sixteen 16-byte units, and four consecutive rows land in four different quarters."""
+    key16 = [_bitrev(r & 15, 4) for r in range(16)]
+    assert sorted(key16) == list(range(16))
+    assert sorted(k >> 2 for k in key16[:4]) == [0, 1, 2, 3] and sorted(k >> 2 for k in key16[8:12]) == [0, 1, 2, 3]
+    units = {((r & 1) * 8 + (5 ^ _bitrev((r >> 1) & 7, 3))) for r in range(16)}      # chunk 5 of 128-byte rows
+    assert len(units) == 16
