@@ -230,6 +230,169 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
   }
 }
 
+// ---- the same GEMM with the tiles brought in by global_load_lds_dwordx4 ----
+// Why: a ds_write_b128 and a ds_read of another wavefront take turns on the LDS, a direct-to-LDS
+// load does not hold up the reads (measured: readers + ds_write run as long as the sum of the
+// two, readers + global_load_lds as long as the loads alone).  The tiles land unpadded, with the
+// chunks of every row XOR-swizzled (STORE_LDS_DIRECT_SWIZZLE); without padding three stages fit
+// in LDS (3 x 48 KB), and they are needed: a direct transfer cannot be requested before its stage
+// is free, so the memory latency has to fit into two K steps instead of being bridged by
+// registers.  Each DMA wavefront keeps two transfers in flight (issue_direct + wait_direct_loads).
+template<typename T>
+struct Three {
+  T a0, a1, a2;
+  template<int I> __device__ __forceinline__ T& get() { if constexpr (I == 0) return a0; else if constexpr (I == 1) return a1; else return a2; }
+};
+
+__global__ void __launch_bounds__(kComputeThreads + 2 * kDmaWave)
+gemm_bf16_ws_direct(const unsigned short* __restrict__ a, const unsigned short* __restrict__ b, float* __restrict__ c,
+                    const int m, const int n, const int k)
+{
+  constexpr int WI = 4, WJ = 2, kStages = 3;
+  constexpr int kBM = 64 * WI, kBN = 64 * WJ;
+  constexpr int kARow = kBK * 2, kBRow = kBN * 2;                 // 128 B and 256 B, unpadded
+  constexpr int kAStage = kBM * kARow, kBStage = kBK * kBRow;     // 32 KB and 16 KB
+  typedef CudaDMAStrided<false, 16, 16, kARow, kDmaWave, kBM> dma_a_t;
+  typedef CudaDMAStrided<false, 16, 16, kBRow, kDmaWave, kBK> dma_b_t;
+  __shared__ __attribute__((aligned(1024))) char lds_a[kStages][kAStage];
+  __shared__ __attribute__((aligned(1024))) char lds_b[kStages][kBStage];
+  dma_a_t dma_a(k * 2, kARow, kComputeThreads);
+  dma_b_t dma_b(n * 2, kBRow, kComputeThreads + kDmaWave);
+  Three<cudaDMACustom> stage{cudaDMACustom(0, 2 * kDmaWave, kComputeThreads, kComputeThreads),
+                             cudaDMACustom(1, 2 * kDmaWave, kComputeThreads, kComputeThreads),
+                             cudaDMACustom(2, 2 * kDmaWave, kComputeThreads, kComputeThreads)};
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, m / kBM, n / kBN, tile_m, tile_n);
+  const int ksteps = k / kBK;
+
+  // One DMA wavefront: tile t lands in stage t % 3.  Tiles t+1 and t+2 are in flight while the
+  // compute wavefronts work on tile t: the wavefront waits for tile t (leaving the younger
+  // loads in flight), reports it, and then requests tile t+2 as soon as its stage is free.
+  auto feed = [&](auto& dma, char* lds, auto stage_bytes, const unsigned short* src, const size_t step) {
+    constexpr int kStageBytes = decltype(stage_bytes)::value;
+    constexpr int kLoads = std::remove_reference<decltype(dma)>::type::loads_per_thread();
+    stage.a0.wait_for_dma_start_direct();
+    dma.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src, lds);
+    stage.a1.wait_for_dma_start_direct();
+    dma.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src + step, lds + kStageBytes);
+    auto land = [&](auto cur, auto nxt2, const int t) __attribute__((always_inline)) {
+      if (t + 1 < ksteps) hipdma::wait_direct_loads<kLoads>(); else hipdma::wait_direct_loads<0>();
+      stage.template get<decltype(cur)::value>().finish_async_dma_direct();
+      if (t + 2 < ksteps) {
+        stage.template get<decltype(nxt2)::value>().wait_for_dma_start_direct();
+        dma.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src + (size_t)(t + 2) * step, lds + decltype(nxt2)::value * kStageBytes);
+      }
+    };
+    typedef std::integral_constant<int, 0> s0;
+    typedef std::integral_constant<int, 1> s1;
+    typedef std::integral_constant<int, 2> s2;
+    for (int t = 0; t < ksteps; t += 3) {
+      land(s0(), s2(), t);
+      if (t + 1 < ksteps) land(s1(), s0(), t + 1);
+      if (t + 2 < ksteps) land(s2(), s1(), t + 2);
+    }
+  };
+  if (dma_a.owns_this_thread()) {
+    feed(dma_a, &lds_a[0][0], std::integral_constant<int, kAStage>(), a + (size_t)tile_m * kBM * k, (size_t)kBK);
+  } else if (dma_b.owns_this_thread()) {
+    feed(dma_b, &lds_b[0][0], std::integral_constant<int, kBStage>(), b + (size_t)tile_n * kBN, (size_t)kBK * n);
+  } else {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = (wave >> 1) * 32 * WI, wn = (wave & 1) * 32 * WJ;
+    f32x16_t acc[WI][WJ];
+#pragma unroll
+    for (int i = 0; i < WI; ++i)
+#pragma unroll
+      for (int j = 0; j < WJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+    stage.a0.start_async_dma();
+    stage.a1.start_async_dma();
+    stage.a2.start_async_dma();
+    // A fragment of slice ks: row wm + 32*i + lane%32, chunk 2*ks + lane/32 of the 8 chunks of the row,
+    // found at chunk position (2*ks + lane/32) ^ key(row); the key only depends on lane%32 here.
+    int a_lane[kBK / 16];
+    {
+      const int row = wm + (lane & 31);
+#pragma unroll
+      for (int ks = 0; ks < kBK / 16; ++ks)
+        a_lane[ks] = row * kARow + hipdma::swizzled_chunk(row, 2 * ks + (lane >> 5), kARow / 16) * 16;
+    }
+    // B fragment through the transposing read: inside a group of 16 lanes, lane j points at row (j/4) of a
+    // 4-row block and at column 4*(j%4); the rows of the "lo" and "hi" reads are 4 apart.  Adding 16 rows
+    // (the next slice) does not change a row's key.
+    int b_lo[WJ], b_hi[WJ];
+    {
+      const int j16 = lane & 15;
+      const int row = (lane >> 5) * 8 + (j16 >> 2);
+#pragma unroll
+      for (int j = 0; j < WJ; ++j) {
+        const int col_bytes = (wn + j * 32 + ((lane >> 4) & 1) * 16 + (j16 & 3) * 4) * 2;
+        b_lo[j] = row * kBRow + hipdma::swizzled_chunk(row, col_bytes >> 4, kBRow / 16) * 16 + (col_bytes & 15);
+        b_hi[j] = (row + 4) * kBRow + hipdma::swizzled_chunk(row + 4, col_bytes >> 4, kBRow / 16) * 16 + (col_bytes & 15);
+      }
+    }
+    auto load_frags = [&](bf16x8_t (&fa)[WI], bf16x8_t (&fb)[WJ], const char* sa, const char* sb, const int ks)
+        __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < WI; ++i)
+        fa[i] = *(const bf16x8_t*)(sa + i * 32 * kARow + a_lane[ks]);
+#pragma unroll
+      for (int j = 0; j < WJ; ++j) {
+        const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+            (__attribute__((address_space(3))) bf16x4_t*)(sb + ks * 16 * kBRow + b_lo[j]));
+        const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+            (__attribute__((address_space(3))) bf16x4_t*)(sb + ks * 16 * kBRow + b_hi[j]));
+        fb[j] = bf16x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      }
+    };
+    auto multiply = [&](const bf16x8_t (&fa)[WI], const bf16x8_t (&fb)[WJ]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < WI; ++i)
+#pragma unroll
+        for (int j = 0; j < WJ; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      pin_slice<0, WI * WJ, WI + 2 * WJ>();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    bf16x8_t fa0[WI], fb0[WJ], fa1[WI], fb1[WJ];
+    // One stage: on entry fa0/fb0 hold its slice 0; on exit they hold slice 0 of the next stage.
+    auto k_stage = [&](const cudaDMACustom& cur, const cudaDMACustom& nxt, const int s, const int sn, const bool has_next)
+        __attribute__((always_inline)) {
+      const char* sa = lds_a[s]; const char* sb = lds_b[s];
+      load_frags(fa1, fb1, sa, sb, 1); multiply(fa0, fb0);
+      load_frags(fa0, fb0, sa, sb, 2); multiply(fa1, fb1);
+      const unsigned seen = nxt.peek_dma_finish();
+      load_frags(fa1, fb1, sa, sb, 3); multiply(fa0, fb0);
+      if (has_next) {
+        nxt.wait_for_dma_finish(seen);
+        load_frags(fa0, fb0, lds_a[sn], lds_b[sn], 0);
+      }
+      multiply(fa1, fb1);
+      cur.start_async_dma();
+    };
+    stage.a0.wait_for_dma_finish();
+    load_frags(fa0, fb0, lds_a[0], lds_b[0], 0);
+    for (int kt = 0; kt < ksteps; kt += 3) {
+      k_stage(stage.a0, stage.a1, 0, 1, kt + 1 < ksteps);
+      if (kt + 1 < ksteps) k_stage(stage.a1, stage.a2, 1, 2, kt + 2 < ksteps);
+      if (kt + 2 < ksteps) k_stage(stage.a2, stage.a0, 2, 0, kt + 3 < ksteps);
+    }
+    float* cbase = c + (size_t)(tile_m * kBM + wm) * n + (size_t)tile_n * kBN + wn;
+#pragma unroll
+    for (int i = 0; i < WI; ++i)
+#pragma unroll
+      for (int j = 0; j < WJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
+          const int col = j * 32 + (lane & 31);
+          cbase[(size_t)row * n + col] = acc[i][j][e];
+        }
+  }
+}
+
 template<int WI, int WJ>
 int launch_gemm(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k, hipStream_t stream)
 {
@@ -265,6 +428,14 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
   switch (variant) {
     case 1: return launch_gemm<2, 2>(d_a, d_b, d_c, m, n, k, s);
     case 2: return launch_gemm<2, 4>(d_a, d_b, d_c, m, n, k, s);
-    default: return launch_gemm<4, 2>(d_a, d_b, d_c, m, n, k, s);
+    case 3: return launch_gemm<4, 2>(d_a, d_b, d_c, m, n, k, s);
+    default: {
+      CUDADMA_REQUIRE((m % 256) == 0, "this variant needs m a multiple of 256 (got %d)", m);
+      const long long grid = (long long)(m / 256) * (n / 128);
+      CUDADMA_REQUIRE(grid <= 0x7fffffffLL, "grid too large");
+      hipLaunchKernelGGL(gemm_bf16_ws_direct, dim3((unsigned)grid), dim3(kComputeThreads + 2 * kDmaWave), 0, s, d_a, d_b, d_c, m, n, k);
+      CUDADMA_HIP_CHECK(hipGetLastError());
+      return CUDADMA_OK;
+    }
   }
 }

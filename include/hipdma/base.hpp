@@ -154,6 +154,39 @@ __device__ __forceinline__ void wait_word(lds_word_t* word, unsigned target)
   acquire_lds();
 }
 
+// The same two operations for a DMA wavefront that keeps direct-to-LDS loads in flight across
+// the hand-off.  The compiler counts a global_load_lds as an LDS write: any fence or LDS access
+// it can see makes it wait for ALL outstanding ones (s_waitcnt vmcnt(0)), which would leave
+// one transfer in flight at a time.  These versions keep the LDS word accesses out of its sight
+// (inline assembly) and carry no fence; the caller orders things itself: it waits for the loads
+// it reports with s_waitcnt vmcnt(N) before signalling, and it only issues loads into a buffer
+// after the wait for that buffer has returned (a control dependence the hardware honours).
+__device__ __forceinline__ void signal_word_unfenced(lds_word_t* word)
+{
+  const unsigned long long active = __builtin_amdgcn_ballot_w64(true);
+  const unsigned lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  if (lane == (unsigned)__builtin_ctzll(active)) {
+    const unsigned addr = (unsigned)(size_t)word;
+    const unsigned count = (unsigned)__builtin_popcountll(active);
+    asm volatile("ds_add_u32 %0, %1" : : "v"(addr), "v"(count) : "memory");
+  }
+}
+
+__device__ __forceinline__ void wait_word_unfenced(lds_word_t* word, unsigned target)
+{
+  const unsigned addr = (unsigned)(size_t)word;
+  unsigned seen;
+#if HIPDMA_SPIN_LIMIT > 0
+  for (int polls = 0; polls < HIPDMA_SPIN_LIMIT; ++polls) {
+#else
+  for (;;) {
+#endif
+    asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : "v"(addr) : "memory");
+    if ((int)(seen - target) >= 0) break;
+    __builtin_amdgcn_s_sleep(HIPDMA_SPIN_SLEEP);
+  }
+}
+
 struct no_sync_t {};
 
 __host__ __device__ constexpr int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -298,6 +331,23 @@ public:
   __device__ __forceinline__ void finish_async_dma(void) const
   {
     if (m_has_sync) hipdma::detail::signal_word(m_full);
+  }
+  // DMA side, for wavefronts that keep direct-to-LDS loads (CudaDMAStrided::issue_direct) in
+  // flight across the hand-off: the same two calls without a fence and without an LDS access the
+  // compiler could see, because either would make it wait for every outstanding direct load.
+  // The caller waits for the loads it reports (hipdma::wait_direct_loads<YOUNGER>()) before
+  // finish_async_dma_direct(), and requests loads into a buffer only after
+  // wait_for_dma_start_direct() for that buffer has returned.
+  __device__ __forceinline__ void wait_for_dma_start_direct(void) const
+  {
+    if (m_has_sync) {
+      m_wait_target += m_wait_unit;
+      hipdma::detail::wait_word_unfenced(m_empty, m_wait_target);
+    }
+  }
+  __device__ __forceinline__ void finish_async_dma_direct(void) const
+  {
+    if (m_has_sync) hipdma::detail::signal_word_unfenced(m_full);
   }
 protected:
   const bool m_is_dma_thread;
