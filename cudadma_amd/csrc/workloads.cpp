@@ -80,7 +80,8 @@ static const VariantInfo kHalo[] = {
 };
 
 static const VariantInfo kGemm[] = {
-  {"the largest workgroup tile that divides the problem: variant 3 when m is a multiple of 256, else variant 1"},
+  {"the largest workgroup tile that divides the problem: variant 3 when m is a multiple of 256, variant 2 when only n "
+   "is, else variant 1"},
   {"warp-specialised: two DMA wavefronts per operand with two CudaDMAStrided objects each (two LDS stages, tile two K "
    "steps ahead in flight), four compute wavefronts with v_mfma_f32_32x32x16_bf16, B fragments through "
    "ds_read_b64_tr_b16; 128 x 128 workgroup tile, 64 x 64 per compute wavefront, two workgroups per compute unit"},

@@ -424,7 +424,7 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
                   "pointers must be 16-byte aligned");
   CUDADMA_REQUIRE((long long)k * 2 <= 0x7fffffffLL && (long long)n * 2 <= 0x7fffffffLL, "row pitch must fit an int");
   hipStream_t s = (hipStream_t)stream;
-  if (variant == 0) variant = (m % 256) == 0 ? 3 : 1;      // the largest tile that divides the problem
+  if (variant == 0) variant = (m % 256) == 0 ? 3 : (n % 256) == 0 ? 2 : 1;      // the largest tile that divides the problem
   switch (variant) {
     case 1: return launch_gemm<2, 2>(d_a, d_b, d_c, m, n, k, s);
     case 2: return launch_gemm<2, 4>(d_a, d_b, d_c, m, n, k, s);

@@ -199,7 +199,10 @@ int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz
 /* Config 5 (no GEMM in the reference; nearest: src/examples/sgemv/sgemv_dma.cu:329-388):
  * C = A * B with A m x k and B k x n row-major bf16 (as uint16 bit patterns), C m x n
  * float, fp32 accumulation on the matrix cores.  m, n and k multiples of 128.
- * DMA wavefronts stage 128 x 64 tiles of A and 64 x 128 tiles of B through CudaDMAStrided. */
+ * Four DMA wavefronts stage the A and B tiles of one K step (64) through CudaDMAStrided, four
+ * compute wavefronts multiply.  variant 0 picks the largest workgroup tile that divides the
+ * problem; 1: 128 x 128; 2: 128 x 256 (n a multiple of 256); 3: 256 x 128 (m a multiple of 256);
+ * 4: 256 x 128 with the tiles brought in by global_load_lds into swizzled LDS rows. */
 int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k,
                       int variant, void* stream);
 
