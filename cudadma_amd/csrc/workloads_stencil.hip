@@ -400,17 +400,22 @@ stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int
     }
     *(f32x4_t*)(&plane[0][kOrigin] + ly * kPitch + lx) = q[kR];
     float* o = w.out_origin + (size_t)ly * nx + lx;
+    // The wait for a plane's ring is split: its `full` word is read at the end of the plane before,
+    // after that plane's arithmetic (by then the ring has landed), and looked at here.
+    unsigned seen = 0;
+    if constexpr (SYNC != kBarrierOnly) seen = guard.a0.peek_dma_finish();
     HIPDMA_FOR_Z(w.planes, {
       constexpr int B = ROT % kBufs;
       const cudaDMACustom& cur_halo = guard.get<B>();
       // past the end of the chunk the last plane is fetched again: unconditional loads keep the wait counts exact
       const int zf = (z + kQueue - 1 < avail) ? (z + kQueue - 1) : (avail - 1);
       q[HIPDMA_QSLOT(ROT, kQueue - 1)] = *(const f32x4_t*)(col + (size_t)zf * in_plane);
-      if constexpr (SYNC != kBarrierOnly) cur_halo.wait_for_dma_finish();
+      if constexpr (SYNC != kBarrierOnly) cur_halo.wait_for_dma_finish(seen);
       if constexpr (SYNC == kHandshakeAndGroupBarrier) compute_barrier.sync();
       else __syncthreads();
       const f32x4_t r = stencil_cells4<ROT>(plane[B], lx, ly, q, k);
       if constexpr (SYNC != kBarrierOnly) cur_halo.start_async_dma();
+      if constexpr (SYNC != kBarrierOnly) seen = guard.get<(B + 1) % kBufs>().peek_dma_finish();
       *(f32x4_t*)(&plane[(B + 1) % kBufs][kOrigin] + ly * kPitch + lx) = q[HIPDMA_QSLOT(ROT, kR + 1)];
       *(f32x4_t*)o = r;
       o += out_plane;
