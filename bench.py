@@ -6,9 +6,9 @@
 A step is one launch of the CudaDMAStrided tile-transpose kernel over the whole
 16384 x 16384 float32 matrix (benchmark config 2, the configuration the metric is
 quoted on); inputs are resident in HBM before the timed region.  The other three
-HBM-bound patterns (sequential copy, indirect gather, halo stencil) and a plain
-copy kernel are timed the same way and reported under "patterns".  One JSON line
-goes to stdout; progress goes to stderr.
+HBM-bound patterns (sequential copy, indirect gather, halo stencil), the scatter in
+the opposite direction and a plain copy kernel are timed the same way and reported
+under "patterns".  One JSON line goes to stdout; progress goes to stderr.
 """
 import argparse
 import json
@@ -78,7 +78,7 @@ def cpu_baselines(budget_s=16.0):
     from tests.oracle_lib import ptr
     O = ol.load()
     cores = O.oracle_num_threads()
-    per = budget_s / 4
+    per = budget_s / 5
     out = {}
 
     n = 8192                                         # a quarter of the matrix: 512 MiB of traffic per repetition
@@ -105,6 +105,16 @@ def cpu_baselines(budget_s=16.0):
     out["gather"] = {"GB/s": round((n_idx * 132 + sums.size * 4) / med / 1e9, 2),
                      "sample": f"oracle_gather_rowsum over the full 512 MiB table with {n_idx} indices, median of {reps}"}
     del table, idx, sums
+
+    log2_recs = 22                                   # the whole scatter: 512 MiB of records, 4 Mi indices
+    n_rec = 1 << log2_recs
+    records = ol.uniform(n_rec * 32, 1006)
+    perm = ol.permutation(log2_recs, 1006)
+    table = np.empty(n_rec * 32, dtype=np.float32)
+    med, reps = _median_time(lambda: O.oracle_scatter_copy(ptr(records), ptr(perm), ptr(table), n_rec, 32), per)
+    out["scatter"] = {"GB/s": round(n_rec * 260 / med / 1e9, 2),
+                      "sample": f"oracle_scatter_copy of {n_rec} records of 128 B by a permutation, median of {reps}"}
+    del records, perm, table
 
     g, p = 256, 4                                    # one eighth of the grid
     grid = ol.uniform((g + 2 * p) ** 3, 1004)
@@ -175,6 +185,15 @@ def main():
     report("gather", ms, n_idx * 4 + n_idx * 128 + sums.numel() * 4,
            "CudaDMAIndirect 32 x 128 B records per tile from a 512 MiB table, row-sum consumer")
     del table, idx, sums
+
+    # ---- the opposite direction (LDS -> global): scatter of 4 Mi records by a permutation ----
+    records = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev), 1006)
+    perm = wl.fill_permutation(torch.empty(recs, dtype=torch.int32, device=dev), 1006)
+    table = torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev)
+    ms, _ = time_launches(lambda: wl.scatter_copy(records, perm, table, 0), steps, warmup, SETTLE_MS)
+    report("scatter", ms, recs * 4 + 2 * recs * 128,
+           "CudaDMAIndirect<false> LDS -> global: 4 Mi records of 128 B placed by a permutation, 32 records per tile")
+    del records, perm, table
 
     # ---- config 4: halo stencil ----
     g = 512

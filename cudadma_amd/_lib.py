@@ -119,6 +119,8 @@ _WORKLOAD_SIGNATURES = {
     "cudadma_set_workgroups_per_cu": [_ci],
     "cudadma_sequential_copy": [_vp, _vp, _cs, _ci, _vp],
     "cudadma_strided_transpose": [_vp, _vp, _ci, _ci, _vp],
+    "cudadma_fill_permutation": [_vp, _ci, _u64, _vp],
+    "cudadma_scatter_copy": [_vp, _vp, _vp, _cs, _cs, _ci, _vp],
     "cudadma_gather_copy": [_vp, _vp, _vp, _cs, _cs, _ci, _vp],
     "cudadma_gather_rowsum": [_vp, _vp, _vp, _cs, _cs, _ci, _vp],
     "cudadma_halo_stencil": [_vp, _vp, _ci, _ci, _ci, _ci, _vp],

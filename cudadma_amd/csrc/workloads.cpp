@@ -91,6 +91,14 @@ static const VariantInfo kGemm[] = {
    "unpadded swizzled LDS stages, two transfers in flight per DMA wavefront, no ds_write"},
 };
 
+static const VariantInfo kScatter[] = {
+  {"manual 4-stage buffering, LDS -> global: the compute wavefronts fill four LDS tiles of 32 records, one DMA group of "
+   "2 wavefronts drains them with one CudaDMAIndirect<false> object, a cudaDMACustom guard per tile"},
+  {"single buffer: one LDS tile, one guard"},
+  {"manual double buffer: two LDS tiles, two guards"},
+  {"not warp-specialised: all four wavefronts fill the tile, meet, and all four scatter it"},
+};
+
 static const VariantInfo* table(int workload, int* count)
 {
   switch (workload) {
@@ -99,6 +107,7 @@ static const VariantInfo* table(int workload, int* count)
     case CUDADMA_WORKLOAD_GATHER:     *count = sizeof(kGather) / sizeof(VariantInfo);     return kGather;
     case CUDADMA_WORKLOAD_HALO:       *count = sizeof(kHalo) / sizeof(VariantInfo);       return kHalo;
     case CUDADMA_WORKLOAD_GEMM:       *count = sizeof(kGemm) / sizeof(VariantInfo);       return kGemm;
+    case CUDADMA_WORKLOAD_SCATTER:    *count = sizeof(kScatter) / sizeof(VariantInfo);    return kScatter;
     default: *count = 0; return nullptr;
   }
 }

@@ -183,7 +183,37 @@ fill_indices_kernel(int* __restrict__ dst, const size_t n, const unsigned n_reco
   }
 }
 
+__global__ void __launch_bounds__(256)
+fill_permutation_kernel(int* __restrict__ dst, const int log2_n, const unsigned long long k0,
+                        const unsigned long long k1)
+{
+  const unsigned long long n = 1ull << log2_n, mask = n - 1;
+  const int h = (log2_n + 1) / 2;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    unsigned long long x = i;
+    x = (x * ((k0 & 0xffffffffull) | 1ull) + (k0 >> 32)) & mask;
+    x ^= x >> h;
+    x = (x * ((k1 & 0xffffffffull) | 1ull) + (k1 >> 32)) & mask;
+    x ^= x >> h;
+    x = (x * 0x9E3779B1ull) & mask;
+    dst[i] = (int)x;
+  }
+}
+
 }  // namespace
+
+extern "C" int cudadma_fill_permutation(int32_t* d_dst, int log2_n, uint64_t seed, void* stream)
+{
+  CUDADMA_REQUIRE(log2_n >= 1 && log2_n <= 31, "log2_n (%d) must lie in 1..31", log2_n);
+  CUDADMA_REQUIRE(d_dst != nullptr, "d_dst is NULL");
+  const size_t n = (size_t)1 << log2_n;
+  const int grid = workloads::persistent_grid((long long)((n + 255) / 256), 8);
+  hipLaunchKernelGGL(fill_permutation_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, d_dst, log2_n,
+                     workloads::splitmix64(seed), workloads::splitmix64(seed + 1));
+  CUDADMA_HIP_CHECK(hipGetLastError());
+  return CUDADMA_OK;
+}
 
 extern "C" int cudadma_fill_uniform(float* d_dst, size_t n, uint64_t seed, void* stream)
 {

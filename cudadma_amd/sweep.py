@@ -3,7 +3,7 @@ compute unit, timed with HIP events.  The counterpart of the reference's
 src/perf/sequential/param_sweep.py:27-58, which rewrites params_directed.h and recompiles per
 point; here the variants are compiled in and the occupancy is a run-time knob.
 
-    python -m cudadma_amd.sweep [sequential] [strided] [gather] [halo] [gemm] [--wg 0,2,4,8] [--steps 20]
+    python -m cudadma_amd.sweep [sequential] [strided] [gather] [scatter] [halo] [gemm] [--wg 0,2,4,8] [--steps 20]
     python -m cudadma_amd.sweep saxpy sgemv stencil2d        # the reference's example programs, every variant
     python -m cudadma_amd.sweep perf_sequential --wg 2,8     # read-bandwidth probe: element size x DMA wavefronts x buffering
 """
@@ -84,6 +84,16 @@ def main(argv=None):
                     wl.set_workgroups_per_cu(wg)
                     _row(name, v, wg, _time(lambda: wl.gather_rowsum(table, idx, out, v), args.steps),
                          n_idx * 132 + out.numel() * 4)
+        elif name == "scatter":
+            recs = 4 << 20
+            records = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1006)
+            perm = wl.fill_permutation(torch.empty(recs, dtype=torch.int32, device=dev), 1006)
+            table = torch.empty(recs * wl.REC_FLOATS, device=dev)
+            for v in range(wl.num_variants(wl.SCATTER)):
+                print(f"# scatter variant {v}: {wl.variant_name(wl.SCATTER, v)}")
+                for wg in wgs:
+                    wl.set_workgroups_per_cu(wg)
+                    _row(name, v, wg, _time(lambda: wl.scatter_copy(records, perm, table, v), args.steps), recs * 260)
         elif name == "halo":
             g = 512
             gi = wl.fill_uniform(torch.empty((g + 8) ** 3, device=dev), 1004).view(g + 8, g + 8, g + 8)

@@ -7,7 +7,7 @@ import torch
 
 from ._lib import check, lib
 
-SEQUENTIAL, STRIDED, GATHER, HALO, GEMM = range(5)
+SEQUENTIAL, STRIDED, GATHER, HALO, GEMM, SCATTER = range(6)
 
 REC_FLOATS = 32          # 128-byte records
 RECS_PER_TILE = 32
@@ -59,6 +59,16 @@ def fill_indices(out, n_records, seed):
     return out
 
 
+def fill_permutation(out, seed):
+    """out: int32 tensor of 2^k elements; receives a seeded permutation of [0, 2^k)."""
+    _need(out, torch.int32, "out")
+    n = out.numel()
+    if n < 2 or n & (n - 1):
+        raise ValueError("out must hold a power of two of elements, at least 2")
+    check(lib().cudadma_fill_permutation(_p(out), n.bit_length() - 1, seed, _stream()))
+    return out
+
+
 def plain_copy(src, dst):
     check(lib().cudadma_plain_copy(_p(src), _p(dst), src.numel() * src.element_size(), _stream()))
     return dst
@@ -103,6 +113,18 @@ def gather_rowsum(table, idx, out, variant=0):
     check(lib().cudadma_gather_rowsum(_p(table), _p(idx), _p(out), table.numel() // REC_FLOATS, idx.numel(),
                                       variant, _stream()))
     return out
+
+
+def scatter_copy(records, idx, table, variant=0):
+    """table[idx[i]] = records[i]; idx holds distinct record numbers of the table."""
+    _need(records, torch.float32, "records")
+    _need(idx, torch.int32, "idx")
+    _need(table, torch.float32, "table")
+    if records.numel() != idx.numel() * REC_FLOATS:
+        raise ValueError("records must hold one record per index")
+    check(lib().cudadma_scatter_copy(_p(records), _p(idx), _p(table), table.numel() // REC_FLOATS, idx.numel(),
+                                     variant, _stream()))
+    return table
 
 
 def halo_stencil(grid_in, grid_out, variant=0):

@@ -148,7 +148,8 @@ enum {
   CUDADMA_WORKLOAD_STRIDED    = 1,
   CUDADMA_WORKLOAD_GATHER     = 2,
   CUDADMA_WORKLOAD_HALO       = 3,
-  CUDADMA_WORKLOAD_GEMM       = 4
+  CUDADMA_WORKLOAD_GEMM       = 4,
+  CUDADMA_WORKLOAD_SCATTER    = 5
 };
 int cudadma_num_variants(int workload);
 /* One-line description of a variant ("" when out of range). */
@@ -168,6 +169,15 @@ int cudadma_set_tuning(const char* name, int value);
 int cudadma_fill_uniform(float* d_dst, size_t n, uint64_t seed, void* stream);
 /* Element indices uniform over [0, n_records), one in ten repeating an earlier draw. */
 int cudadma_fill_indices(int32_t* d_dst, size_t n, uint32_t n_records, uint64_t seed, void* stream);
+
+/* A seeded permutation of [0, 2^log2_n), 1 <= log2_n <= 31: distinct element indices for the
+ * scatter.  With mask = 2^log2_n - 1, h = (log2_n + 1) / 2, k0 = splitmix64(seed) and
+ * k1 = splitmix64(seed + 1), entry i is x after
+ *   x = i;  x = (x * (lo32(k0) | 1) + hi32(k0)) & mask;  x ^= x >> h;
+ *           x = (x * (lo32(k1) | 1) + hi32(k1)) & mask;  x ^= x >> h;
+ *           x = (x * 0x9E3779B1) & mask
+ * (an odd multiplier, an added constant and a right xor-shift are each one-to-one on log2_n bits). */
+int cudadma_fill_permutation(int32_t* d_dst, int log2_n, uint64_t seed, void* stream);
 
 /* Calibration kernel: grid-stride dwordx4 copy with no LDS and no DMA object.
  * bytes must be a multiple of 16. */
@@ -189,6 +199,15 @@ int cudadma_gather_copy(const float* d_table, const int32_t* d_idx, float* d_out
                         size_t n_records, size_t n_idx, int variant, void* stream);
 int cudadma_gather_rowsum(const float* d_table, const int32_t* d_idx, float* d_out,
                           size_t n_records, size_t n_idx, int variant, void* stream);
+
+/* The opposite direction of config 3, LDS -> global (include/cudaDMAv2.h:10199-10217; the
+ * reference has no test or program of it): d_table[d_idx[i]] = d_records[i] for i < n_idx,
+ * records of 128 B, n_idx a multiple of 32.  The compute wavefronts fill LDS tiles of 32
+ * records, the DMA wavefronts scatter them with CudaDMAIndirect<false>.  d_idx[i] must lie
+ * in [0, n_records); records of the table that no index names are left untouched; when an
+ * index repeats, which of its records ends up in the table is unspecified. */
+int cudadma_scatter_copy(const float* d_records, const int32_t* d_idx, float* d_table,
+                         size_t n_records, size_t n_idx, int variant, void* stream);
 
 /* Config 4 (src/examples/stencil/cudaDMA_stencil2D.cu:100-240): 8th-order
  * 25-point star stencil.  d_in is (nx+8) x (ny+8) x (nz+8) floats, x fastest;

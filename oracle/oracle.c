@@ -59,6 +59,27 @@ void oracle_fill_indices(int32_t* dst, size_t n, uint32_t n_records, uint64_t se
   }
 }
 
+/* A permutation of [0, 2^log2_n): an odd multiplier, an added constant and a right xor-shift are
+ * each one-to-one on log2_n bits.  States the generator the scatter workload draws its distinct
+ * indices from (no counterpart in the reference, whose tests draw non-overlapping offsets with
+ * srand/rand, src/tests/test_indirect/cudaDMA_test_indirect_v2.cu:721-760). */
+void oracle_fill_permutation(int32_t* dst, int log2_n, uint64_t seed)
+{
+  const uint64_t n = (uint64_t)1 << log2_n, mask = n - 1;
+  const uint64_t k0 = oracle_splitmix64(seed), k1 = oracle_splitmix64(seed + 1);
+  const int h = (log2_n + 1) / 2;
+#pragma omp parallel for schedule(static)
+  for (long long i = 0; i < (long long)n; ++i) {
+    uint64_t x = (uint64_t)i;
+    x = (x * ((k0 & 0xffffffffu) | 1u) + (k0 >> 32)) & mask;
+    x ^= x >> h;
+    x = (x * ((k1 & 0xffffffffu) | 1u) + (k1 >> 32)) & mask;
+    x ^= x >> h;
+    x = (x * 0x9E3779B1u) & mask;
+    dst[i] = (int32_t)x;
+  }
+}
+
 uint16_t oracle_f32_to_bf16(float v)
 {
   uint32_t u;
@@ -269,6 +290,15 @@ void oracle_gather_copy(const float* table, const int32_t* idx, float* out, size
 #pragma omp parallel for schedule(static)
   for (long long i = 0; i < (long long)n_idx; ++i)
     memcpy(out + (size_t)i * rec_floats, table + (size_t)idx[i] * rec_floats, (size_t)rec_floats * sizeof(float));
+}
+
+/* The scatter workload: table[idx[i]] = records[i] (addressing of include/cudaDMAv2.h:10199-10217
+ * with the dense side packed).  Indices are distinct, so the iterations are independent. */
+void oracle_scatter_copy(const float* records, const int32_t* idx, float* table, size_t n_idx, int rec_floats)
+{
+#pragma omp parallel for schedule(static)
+  for (long long i = 0; i < (long long)n_idx; ++i)
+    memcpy(table + (size_t)idx[i] * rec_floats, records + (size_t)i * rec_floats, (size_t)rec_floats * sizeof(float));
 }
 
 /* Config 3, headline consumer: out[t][j] = sum over the recs_per_tile records of

@@ -33,6 +33,7 @@ uint32_t oracle_hash32(uint64_t seed, uint64_t i);            /* splitmix64(seed
 void oracle_fill_uniform(float* dst, size_t n, uint64_t seed);/* (h >> 8) * 2^-23 - 1, in [-1,1) */
 void oracle_fill_ramp(float* dst, size_t n);                  /* dst[i] = (float)i, as the reference tests */
 void oracle_fill_indices(int32_t* dst, size_t n, uint32_t n_records, uint64_t seed);
+void oracle_fill_permutation(int32_t* dst, int log2_n, uint64_t seed);  /* of [0, 2^log2_n) */
 void oracle_fill_normal_bf16(uint16_t* dst, size_t n, uint64_t seed);
 uint16_t oracle_f32_to_bf16(float v);
 float oracle_bf16_to_f32(uint16_t v);
@@ -59,6 +60,7 @@ int oracle_halo_check(const void* idata, const void* odata, int elmt_bytes, int 
 void oracle_copy(const float* in, float* out, size_t n);
 void oracle_transpose(const float* in, float* out, int n);
 void oracle_gather_copy(const float* table, const int32_t* idx, float* out, size_t n_idx, int rec_floats);
+void oracle_scatter_copy(const float* records, const int32_t* idx, float* table, size_t n_idx, int rec_floats);
 void oracle_gather_rowsum(const float* table, const int32_t* idx, float* out, size_t n_idx, int rec_floats,
                           int recs_per_tile);
 void oracle_stencil25(const float* in, float* out, int nx, int ny, int nz, int radius_pad);

@@ -48,6 +48,23 @@ def indices(seed, n, n_records):
     return out
 
 
+def permutation_head(log2_n, seed, count):
+    """First entries of the seeded permutation of [0, 2^log2_n) in Python integers."""
+    mask = (1 << log2_n) - 1
+    h = (log2_n + 1) // 2
+    k0, k1 = splitmix64(seed), splitmix64((seed + 1) & M64)
+    out = []
+    for i in range(min(count, 1 << log2_n)):
+        x = i
+        x = (x * ((k0 & 0xFFFFFFFF) | 1) + (k0 >> 32)) & mask
+        x ^= x >> h
+        x = (x * ((k1 & 0xFFFFFFFF) | 1) + (k1 >> 32)) & mask
+        x ^= x >> h
+        x = (x * 0x9E3779B1) & mask
+        out.append(x)
+    return out
+
+
 def strided_ramp(e_floats, n, src_stride_floats, dst_stride_floats):
     """The reference's strided test: source float(i), every moved element compared exactly."""
     src = np.arange(n * src_stride_floats + e_floats, dtype=np.float32)
@@ -82,6 +99,8 @@ def main():
         "splitmix64": {str(x): str(splitmix64(x)) for x in (0, 1, 1001, 1234567, 0xDEADBEEFCAFEF00D, M64)},
         "uniform_bits": {str(seed): uniform_bits(seed, 64) for seed in (1001, 1002, 1003, 1004)},
         "indices": {"seed": 1003, "n_records": 4 * 1024 * 1024, "n": 4096, "values": indices(1003, 4096, 4 * 1024 * 1024)},
+        "permutations": [{"log2_n": b, "seed": seed, "head": permutation_head(b, seed, 256)}
+                         for (b, seed) in ((1, 7), (5, 1006), (16, 1006), (22, 1006), (31, 3))],
         "strided_ramp": [
             {"e_floats": e, "n": n, "src_stride_floats": ss, "dst_stride_floats": ds, "dst": strided_ramp(e, n, ss, ds)}
             for (e, n, ss, ds) in ((16, 5, 40, 16), (3, 7, 9, 5), (64, 4, 64, 68))

@@ -16,6 +16,7 @@ _SIGS = {
     "oracle_fill_uniform": (None, [_vp, _cs, _u64]),
     "oracle_fill_ramp": (None, [_vp, _cs]),
     "oracle_fill_indices": (None, [_vp, _cs, ctypes.c_uint32, _u64]),
+    "oracle_fill_permutation": (None, [_vp, _ci, _u64]),
     "oracle_fill_normal_bf16": (None, [_vp, _cs, _u64]),
     "oracle_f32_to_bf16": (ctypes.c_uint16, [ctypes.c_float]),
     "oracle_bf16_to_f32": (ctypes.c_float, [ctypes.c_uint16]),
@@ -30,6 +31,7 @@ _SIGS = {
     "oracle_transpose": (None, [_vp, _vp, _ci]),
     "oracle_gather_copy": (None, [_vp, _vp, _vp, _cs, _ci]),
     "oracle_gather_rowsum": (None, [_vp, _vp, _vp, _cs, _ci, _ci]),
+    "oracle_scatter_copy": (None, [_vp, _vp, _vp, _cs, _ci]),
     "oracle_stencil25": (None, [_vp, _vp, _ci, _ci, _ci, _ci]),
     "oracle_gemm_bf16": (None, [_vp, _vp, _vp, _ci, _ci, _ci]),
     "oracle_gemm_bf16_entry": (ctypes.c_float, [_vp, _vp, _ci, _ci, _ci, _ci]),
@@ -71,6 +73,12 @@ def uniform(n, seed):
 def ramp(n):
     out = np.empty(n, dtype=np.float32)
     load().oracle_fill_ramp(ptr(out), n)
+    return out
+
+
+def permutation(log2_n, seed):
+    out = np.empty(1 << log2_n, dtype=np.int32)
+    load().oracle_fill_permutation(ptr(out), log2_n, seed)
     return out
 
 

@@ -221,6 +221,35 @@ def test_gather_copy_and_rowsum(O):
     assert np.allclose(sums, tiles.astype(np.float64).sum(axis=1), rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("log2_n", [1, 2, 3, 7, 12, 20])
+@pytest.mark.parametrize("seed", [0, 1006, 2**63 + 5])
+def test_permutation_is_one(O, log2_n, seed):
+    p = ol.permutation(log2_n, seed)
+    assert np.array_equal(np.sort(p), np.arange(1 << log2_n, dtype=np.int32))
+    if log2_n >= 12:                                     # and not the identity or a plain rotation
+        assert np.count_nonzero(np.diff(p.astype(np.int64)) == 1) < (1 << log2_n) // 16
+        assert not np.array_equal(p, ol.permutation(log2_n, seed + 1))
+
+
+def test_scatter_copy_inverts_gather_copy(O):
+    log2_recs, n_idx = 12, 32 * 100
+    recs = 1 << log2_recs
+    records = ol.uniform(n_idx * 32, 1006).reshape(n_idx, 32)
+    idx = np.ascontiguousarray(ol.permutation(log2_recs, 1006)[:n_idx])
+    table = np.full((recs, 32), np.float32(-7.0))
+    O.oracle_scatter_copy(ptr(records), ptr(idx), ptr(table), n_idx, 32)
+    want = np.full((recs, 32), np.float32(-7.0))
+    want[idx] = records                                   # numpy's own scatter
+    assert np.array_equal(table, want)
+    back = np.empty_like(records)
+    O.oracle_gather_copy(ptr(table), ptr(idx), ptr(back), n_idx, 32)
+    assert np.array_equal(back, records)
+    # the same statement as one transfer of the scatter object over the whole list
+    table2 = np.full((recs, 32), np.float32(-7.0))
+    O.oracle_scatter(ptr(idx), ptr(records), ptr(table2), 128, n_idx, 0)
+    assert np.array_equal(table2, want)
+
+
 def stencil_numpy64(g, nx, ny, nz, p):
     c = [3.0 * (-205.0 / 72.0), 8.0 / 5.0, -1.0 / 5.0, 8.0 / 315.0, -1.0 / 560.0]
     g = g.astype(np.float64)
@@ -398,6 +427,10 @@ def test_golden_generators(O):
         assert [int(v) for v in got] == bits
     idx = g["indices"]
     assert [int(v) for v in ol.indices(idx["n"], idx["n_records"], idx["seed"])] == idx["values"]
+    for perm in g["permutations"]:
+        if perm["log2_n"] <= 22:                       # the 2^31 case is checked on its formula below
+            got = ol.permutation(perm["log2_n"], perm["seed"])
+            assert [int(v) for v in got[:len(perm["head"])]] == perm["head"]
 
 
 def test_golden_strided_ramp_and_halo_ring(O):

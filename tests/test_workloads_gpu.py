@@ -39,6 +39,16 @@ def test_device_generators_match_the_golden_vectors(device):
     idx = g["indices"]
     got = wl.fill_indices(torch.empty(idx["n"], dtype=torch.int32, device=device), idx["n_records"], idx["seed"])
     assert [int(v) for v in got.cpu().numpy()] == idx["values"]
+    for perm in g["permutations"]:
+        got = wl.fill_permutation(torch.empty(1 << perm["log2_n"], dtype=torch.int32, device=device), perm["seed"])
+        assert [int(v) for v in got.cpu().numpy()[:len(perm["head"])]] == perm["head"]
+
+
+@pytest.mark.parametrize("log2_n", [1, 5, 16, 22])
+def test_device_permutation_is_one(device, log2_n):
+    got = wl.fill_permutation(torch.empty(1 << log2_n, dtype=torch.int32, device=device), 1006)
+    assert torch.equal(torch.sort(got).values, torch.arange(1 << log2_n, dtype=torch.int32, device=device))
+    assert np.array_equal(got.cpu().numpy(), ol.permutation(log2_n, 1006))
 
 
 # ------------------------------------------------------------------ config 1
@@ -158,6 +168,63 @@ def test_gather_full_size(device):
     assert int((idx[1025:100000] == idx[1024:99999]).sum()) >= 0
     # empty index list is a no-op
     wl.gather_copy(table, idx[:0], out[:0], 0)
+
+
+# ------------------------------------------------------------------ scatter, LDS -> global
+@pytest.mark.parametrize("variant", _variants(wl.SCATTER))
+@pytest.mark.parametrize("n_tiles", [1, 5, 2048, 4099])
+def test_scatter_small(device, variant, n_tiles):
+    log2_recs = 18
+    recs = 1 << log2_recs
+    n_idx = n_tiles * wl.RECS_PER_TILE                      # 2048 tiles name a quarter of the table, 4099 about half
+    records = ol.uniform(n_idx * wl.REC_FLOATS, 1006)
+    idx = np.ascontiguousarray(ol.permutation(log2_recs, 1006)[:n_idx])
+    want = np.full(recs * wl.REC_FLOATS, np.float32(-7.0))   # records no index names keep this value
+    ol.load().oracle_scatter_copy(ptr(records), ptr(idx), ptr(want), n_idx, wl.REC_FLOATS)
+    d_table = torch.full((recs * wl.REC_FLOATS,), -7.0, dtype=torch.float32, device=device)
+    print(f"scatter variant {variant} tiles {n_tiles}", flush=True)
+    wl.scatter_copy(torch.from_numpy(records).to(device), torch.from_numpy(idx).to(device), d_table, variant)
+    torch.cuda.synchronize()
+    assert np.array_equal(d_table.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_scatter_full_size(device):
+    """4 Mi records of 128 B scattered by a permutation, then gathered back by the same indices."""
+    log2_recs = 22
+    recs = 1 << log2_recs
+    records = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=device), 1006)
+    idx = wl.fill_permutation(torch.empty(recs, dtype=torch.int32, device=device), 1006)
+    table = torch.full((recs * wl.REC_FLOATS,), float("nan"), dtype=torch.float32, device=device)
+    for variant in _variants(wl.SCATTER):
+        print(f"scatter full size variant {variant}", flush=True)
+        table.fill_(float("nan"))
+        wl.scatter_copy(records, idx, table, variant)
+        torch.cuda.synchronize()
+        # torch's own indexing states the same thing: row idx[i] of the table is record i
+        r2 = records.view(recs, wl.REC_FLOATS)
+        t2 = table.view(recs, wl.REC_FLOATS)
+        slab = 1 << 20
+        for s in range(0, recs, slab):
+            assert torch.equal(t2[idx[s:s + slab].long()].view(torch.int32), r2[s:s + slab].view(torch.int32))
+    back = torch.empty_like(records)
+    wl.gather_copy(table, idx, back, 0)
+    torch.cuda.synchronize()
+    assert torch.equal(back.view(torch.int32), records.view(torch.int32))
+    # an empty index list is a no-op
+    wl.scatter_copy(records[:0], idx[:0], table, 0)
+
+
+def test_scatter_argument_checks(device):
+    recs = 1 << 10
+    records = torch.zeros(33 * wl.REC_FLOATS, dtype=torch.float32, device=device)
+    table = torch.zeros(recs * wl.REC_FLOATS, dtype=torch.float32, device=device)
+    idx = torch.zeros(33, dtype=torch.int32, device=device)
+    with pytest.raises(cd.CudaDMAError):
+        wl.scatter_copy(records, idx, table, 0)                       # 33 is not a multiple of 32
+    with pytest.raises(cd.CudaDMAError):
+        wl.scatter_copy(records[:32 * wl.REC_FLOATS], idx[:32], table, wl.num_variants(wl.SCATTER))
+    with pytest.raises(ValueError):
+        wl.fill_permutation(torch.empty(48, dtype=torch.int32, device=device), 1)
 
 
 # ------------------------------------------------------------------ config 4
