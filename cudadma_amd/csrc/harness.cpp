@@ -10,27 +10,29 @@ static std::vector<Entry>& registry()
   static std::vector<Entry> r;
   return r;
 }
-static bool g_sorted = false;
 
+// Called from static initialisers only (the Registrar objects), before any entry point can run.
 void register_case(const cudadma_case_t& desc, launch_fn fn, int order)
 {
   registry().push_back(Entry{desc, fn, order});
-  g_sorted = false;
 }
 
 // Static initialisers of different translation units run in no fixed order:
 // give the cases a stable numbering (pattern, then order of appearance in its list).
+// Sorted once, on the first call of an entry point (the initialisation of a local static
+// is thread-safe); the registry does not change afterwards.
 static const std::vector<Entry>& sorted()
 {
-  std::vector<Entry>& r = registry();
-  if (!g_sorted) {
+  static const bool once = [] {
+    std::vector<Entry>& r = registry();
     std::stable_sort(r.begin(), r.end(), [](const Entry& x, const Entry& y) {
       if (x.desc.pattern != y.desc.pattern) return x.desc.pattern < y.desc.pattern;
       return x.order < y.order;
     });
-    g_sorted = true;
-  }
-  return r;
+    return true;
+  }();
+  (void)once;
+  return registry();
 }
 
 }  // namespace harness

@@ -6,22 +6,21 @@
 namespace workloads {
 
 static std::atomic<int> g_wg_per_cu{0};
-static int g_cus = 0;
 
 int device_cus()
 {
-  if (g_cus <= 0) {
-    g_cus = cudadma_device_cus();
-    if (g_cus <= 0) g_cus = 256;
-  }
-  return g_cus;
+  // queried once (thread-safe initialisation of a local static); 256 if the query fails
+  static const int cus = [] {
+    const int n = cudadma_device_cus();
+    return n > 0 ? n : 256;
+  }();
+  return cus;
 }
 
 int persistent_grid(long long work_items, int default_wg_per_cu)
 {
-  device_cus();
   const int knob = g_wg_per_cu.load();
-  const long long want = (long long)g_cus * (knob > 0 ? knob : default_wg_per_cu);
+  const long long want = (long long)device_cus() * (knob > 0 ? knob : default_wg_per_cu);
   return (int)(work_items < want ? work_items : want);
 }
 
