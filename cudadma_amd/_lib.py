@@ -53,6 +53,8 @@ class RunArgs(ctypes.Structure):
         ("call_style", ctypes.c_int), ("two_phase", ctypes.c_int), ("reps", ctypes.c_int),
         ("rep_src_bytes", ctypes.c_int), ("rep_index_elmts", ctypes.c_int),
         ("reverse", ctypes.c_int), ("out_bytes", ctypes.c_int),
+        ("rt_bytes_per_elmt", ctypes.c_int), ("rt_dma_threads", ctypes.c_int), ("rt_num_elmts", ctypes.c_int),
+        ("rt_dimx", ctypes.c_int), ("rt_dimy", ctypes.c_int),
     ]
 
 

@@ -58,7 +58,37 @@ extern "C" int cudadma_run_case(int case_id, const cudadma_run_t* run, void* str
     return CUDADMA_ERANGE;
   }
   CUDADMA_REQUIRE(run != nullptr, "run is NULL");
-  const cudadma_case_t& d = r[case_id].desc;
+  // the case as it runs: the compiled description with the run-time values of this call
+  cudadma_case_t d = r[case_id].desc;
+  {
+    const bool halo = d.pattern == CUDADMA_PATTERN_HALO;
+    const bool rows = d.pattern == CUDADMA_PATTERN_STRIDED || d.pattern == CUDADMA_PATTERN_GATHER ||
+                      d.pattern == CUDADMA_PATTERN_SCATTER;
+    if (run->rt_bytes_per_elmt != 0) {
+      CUDADMA_REQUIRE(!halo && d.level == 1, "bytes_per_elmt is a compile-time parameter of case %d", case_id);
+      CUDADMA_REQUIRE(run->rt_bytes_per_elmt > 0 && (run->rt_bytes_per_elmt % 4) == 0,
+                      "rt_bytes_per_elmt %d must be a positive multiple of 4", run->rt_bytes_per_elmt);
+      d.bytes_per_elmt = run->rt_bytes_per_elmt;
+    }
+    if (run->rt_dma_threads != 0) {
+      CUDADMA_REQUIRE(halo ? d.level <= 1 : d.level <= 2, "dma_threads is a compile-time parameter of case %d", case_id);
+      CUDADMA_REQUIRE(run->rt_dma_threads > 0 && (run->rt_dma_threads % 64) == 0 &&
+                      run->rt_dma_threads + (d.warp_specialized ? harness::kComputeThreads : 0) <= 1024,
+                      "rt_dma_threads %d must be a multiple of 64 that fits a workgroup of 1024", run->rt_dma_threads);
+      d.dma_threads = run->rt_dma_threads;
+    }
+    if (run->rt_num_elmts != 0) {
+      CUDADMA_REQUIRE(rows && d.level <= 3, "num_elmts is not a run-time parameter of case %d", case_id);
+      CUDADMA_REQUIRE(run->rt_num_elmts > 0, "rt_num_elmts must be positive");
+      d.num_elmts = run->rt_num_elmts;
+    }
+    if (run->rt_dimx != 0 || run->rt_dimy != 0) {
+      CUDADMA_REQUIRE(halo && d.level <= 2, "dimx / dimy are not run-time parameters of case %d", case_id);
+      CUDADMA_REQUIRE(run->rt_dimx >= 0 && run->rt_dimy >= 0, "rt_dimx / rt_dimy must not be negative");
+      if (run->rt_dimx != 0) d.dimx = run->rt_dimx;
+      if (run->rt_dimy != 0) d.dimy = run->rt_dimy;
+    }
+  }
   CUDADMA_REQUIRE(run->d_in != nullptr && run->d_out != nullptr, "d_in / d_out must not be NULL");
   CUDADMA_REQUIRE(run->lds_bytes > 0 && run->lds_bytes <= 64 * 1024 - 256 && (run->lds_bytes % 16) == 0,
                   "lds_bytes %d must be a positive multiple of 16 below 64 KiB", run->lds_bytes);

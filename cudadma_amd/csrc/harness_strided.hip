@@ -97,15 +97,18 @@ __global__ void __launch_bounds__(1024) strided_kernel(const Args a)
 {
   extern __shared__ __attribute__((aligned(16))) unsigned lds[];
   auto dma = Make<WS, LEVEL, ONE, A, BPT, E, T, N>::make(a);
+  // swizzled rows are whole chunks: known here when the element size is a template parameter,
+  // checked by the host for the level that takes it at run time
+  constexpr bool kWholeChunks = (LEVEL == 1) || (E % A) == 0;
   harness::run_body<WS>(dma, a, lds, [&](const int rep) __attribute__((always_inline)) {
     const char* src = a.reverse ? (const char*)lds + a.src_offset : a.in + a.src_offset + (size_t)rep * a.rep_src_bytes;
     char* dst = a.reverse ? a.out + (size_t)rep * a.out_bytes + a.dst_offset : (char*)lds + a.dst_offset;
     if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
       if constexpr (A == 16 || A == 4) direct_transfer<WS, STORE_LDS_DIRECT>(dma, a.two_phase, src, dst);
     } else if (a.call_style == CUDADMA_CALL_LDS_SWIZZLE) {
-      if constexpr ((E % A) == 0) harness::do_transfer_direct<STORE_LDS_SWIZZLE>(dma, a.two_phase, src, dst);
+      if constexpr (kWholeChunks) harness::do_transfer_direct<STORE_LDS_SWIZZLE>(dma, a.two_phase, src, dst);
     } else if (a.call_style == CUDADMA_CALL_LDS_DIRECT_SWIZZLE) {
-      if constexpr ((A == 16 || A == 4) && (E % A) == 0)
+      if constexpr ((A == 16 || A == 4) && kWholeChunks)
         direct_transfer<WS, STORE_LDS_DIRECT_SWIZZLE>(dma, a.two_phase, src, dst);
     } else {
       harness::do_transfer(dma, a.call_style, a.two_phase, src, dst);

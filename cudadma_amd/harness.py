@@ -26,9 +26,12 @@ def _ptr(t):
 
 def run_case(case_id, d_in, d_out, *, lds_bytes, d_index=None, src_offset_bytes=0, dst_offset_bytes=0,
              src_stride=0, dst_stride=0, pitch=0, call_style=_lib.CALL_UNQUALIFIED, two_phase=False, reps=1,
-             rep_src_bytes=0, rep_index_elmts=0, reverse=False, out_bytes=0, stream=None):
+             rep_src_bytes=0, rep_index_elmts=0, reverse=False, out_bytes=0, stream=None,
+             bytes_per_elmt=0, dma_threads=0, num_elmts=0, dimx=0, dimy=0):
     """Launch one case.  d_in / d_out / d_index are torch CUDA tensors; d_out must
-    hold reps * lds_bytes bytes.  Raises CudaDMAError when the library rejects the arguments."""
+    hold reps * lds_bytes bytes.  bytes_per_elmt, dma_threads, num_elmts, dimx and dimy (0 = the
+    case's own) replace the parameters the case's level passes to its constructor at run time.
+    Raises CudaDMAError when the library rejects the arguments."""
     need = reps * (out_bytes if reverse else lds_bytes)
     if d_out.numel() * d_out.element_size() < need:
         raise ValueError("d_out is smaller than reps * (out_bytes if reverse else lds_bytes)")
@@ -37,5 +40,6 @@ def run_case(case_id, d_in, d_out, *, lds_bytes, d_index=None, src_offset_bytes=
         lds_bytes=lds_bytes, src_offset_bytes=src_offset_bytes, dst_offset_bytes=dst_offset_bytes,
         src_stride=src_stride, dst_stride=dst_stride, pitch=pitch, call_style=call_style,
         two_phase=int(bool(two_phase)), reps=reps, rep_src_bytes=rep_src_bytes, rep_index_elmts=rep_index_elmts,
-        reverse=int(bool(reverse)), out_bytes=out_bytes)
+        reverse=int(bool(reverse)), out_bytes=out_bytes, rt_bytes_per_elmt=bytes_per_elmt,
+        rt_dma_threads=dma_threads, rt_num_elmts=num_elmts, rt_dimx=dimx, rt_dimy=dimy)
     check(lib().cudadma_run_case(case_id, ctypes.byref(r), ctypes.c_void_p(stream or 0)))

@@ -92,6 +92,15 @@ typedef struct cudadma_run {
                              dst_offset_bytes.  Only CUDADMA_CALL_UNQUALIFIED (generic pointers on
                              both sides, include/cudaDMAv2.h:107-114,553-558) makes sense here.   */
   int out_bytes;          /* reverse only: bytes of d_out one rep may touch            */
+  /* Other values for the parameters that the case's level hands to the constructor at run time
+   * (0 keeps the case's own), so that one compiled case can be swept the way the reference's
+   * param_sweep_v2.py recompiles its test (src/tests/test_strided/param_sweep_v2.py:51-75):
+   *   rt_bytes_per_elmt  level 1 of sequential / strided / indirect (a multiple of 4)
+   *   rt_dma_threads     levels 1-2 of those, levels 0-1 of halo (a multiple of 64)
+   *   rt_num_elmts       levels 1-3 of strided / indirect
+   *   rt_dimx, rt_dimy   levels 0-2 of halo
+   * A value for a parameter that the case fixes at compile time is refused. */
+  int rt_bytes_per_elmt, rt_dma_threads, rt_num_elmts, rt_dimx, rt_dimy;
 } cudadma_run_t;
 
 int cudadma_num_cases(void);

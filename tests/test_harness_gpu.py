@@ -82,6 +82,88 @@ def test_case_reverse_direction_matches_oracle(case_id, device):
             raise AssertionError(f"two_phase {two_phase}: {len(bad)} wrong bytes, first at rep {bad[0][0]} byte {bad[0][1]}")
 
 
+def _runtime_draw(case, rng):
+    """Other values for the parameters the case's level leaves to run time, drawn as the reference's
+    sweep draws them (src/tests/test_strided/param_sweep_v2.py:51-75: element size |ceil(N(256,256))|
+    floats, 1-32 elements, 1-16 DMA warps), kept inside the harness's LDS window.  Returns the keyword
+    arguments for run_case and the case description as it then runs."""
+    import types
+    c = types.SimpleNamespace(**{f: getattr(case, f) for f, _ in case._fields_})
+    kw = {}
+    halo = case.pattern == cd.PATTERN_HALO
+    max_threads = 1024 - (64 if case.warp_specialized else 0)
+    if (case.level <= 1) if halo else (case.level <= 2):
+        c.dma_threads = kw["dma_threads"] = 64 * int(rng.integers(1, min(16, max_threads // 64) + 1))
+    if halo:
+        if case.level <= 2:
+            unit = max(1, case.alignment // case.bytes_per_elmt)
+            c.dimx = kw["dimx"] = unit * int(rng.integers(1, max(2, 48 // unit)))
+            c.dimy = kw["dimy"] = int(rng.integers(1, 41))
+        return kw, c
+    if case.level == 1:
+        c.bytes_per_elmt = kw["bytes_per_elmt"] = 4 * max(1, abs(int(np.ceil(rng.normal(256, 256)))))
+    if case.pattern != cd.PATTERN_SEQUENTIAL and case.level <= 3:
+        c.num_elmts = kw["num_elmts"] = int(rng.integers(1, 33))
+        row = (c.bytes_per_elmt + 15) // 16 * 16 + 48               # an LDS row with the widest padding CaseIO adds
+        while (c.num_elmts + 3) * row > 60000:                      # the harness's LDS window
+            c.num_elmts = kw["num_elmts"] = max(1, c.num_elmts // 2)
+            if c.num_elmts == 1 and 4 * row > 60000:
+                c.bytes_per_elmt = kw["bytes_per_elmt"] = 4 * int(rng.integers(1, 2048))
+                row = (c.bytes_per_elmt + 15) // 16 * 16 + 48
+    elif case.pattern == cd.PATTERN_SEQUENTIAL and case.level == 1 and c.bytes_per_elmt > 60000:
+        c.bytes_per_elmt = kw["bytes_per_elmt"] = 60000
+    return kw, c
+
+
+_RUNTIME_CASES = [i for i, c in enumerate(_CASES)
+                  if (c.level <= 2 if c.pattern == cd.PATTERN_HALO else c.level <= (2 if c.pattern == cd.PATTERN_SEQUENTIAL else 3))]
+
+
+@pytest.mark.parametrize("case_id", _RUNTIME_CASES, ids=[case_id_str(i, _CASES[i]) for i in _RUNTIME_CASES])
+def test_runtime_parameters_swept(case_id, device):
+    """One compiled case, other run-time sizes: what the reference's endless param_sweep_v2.py loop does by
+    recompiling.  Every draw is first replayed on the host (the device objects' own index arithmetic,
+    which refuses a step outside the buffers) and only then launched."""
+    case = _CASES[case_id]
+    rng = np.random.default_rng(7000 + case_id)
+    for draw in range(6):
+        kw, c = _runtime_draw(case, rng)
+        style = _styles(c)[draw % len(_styles(c))]
+        two_phase = bool(draw & 1)
+        io = CaseIO(c, flavour=draw, reps=2, data="uniform")
+        if io.lds_bytes > 64 * 1024 - 256:
+            continue
+        got_map, _, doubles = io.replay_map()
+        assert doubles == 0 and np.array_equal(got_map, io.expected_map()), f"host replay disagrees for {kw}"
+        want = io.expected(swizzle=style in (cd.CALL_LDS_SWIZZLE, cd.CALL_LDS_DIRECT_SWIZZLE))
+        d_in = torch.from_numpy(io.input).to(device)
+        d_idx = torch.from_numpy(io.index).to(device) if io.index is not None else None
+        d_out = torch.full((io.reps * io.lds_bytes,), 0xEE, dtype=torch.uint8, device=device)
+        print(f"case {case_id} draw {draw} {kw} style {style} two_phase {two_phase}", flush=True)
+        cd.harness.run_case(case_id, d_in, d_out, lds_bytes=io.lds_bytes, d_index=d_idx,
+                            src_offset_bytes=io.src_offset, dst_offset_bytes=io.dst_offset,
+                            src_stride=io.src_stride, dst_stride=io.dst_stride, pitch=io.pitch,
+                            call_style=style, two_phase=two_phase, reps=io.reps,
+                            rep_src_bytes=io.rep_src_bytes, rep_index_elmts=io.rep_index_elmts, **kw)
+        torch.cuda.synchronize()
+        got = d_out.cpu().numpy().reshape(io.reps, io.lds_bytes)
+        if not np.array_equal(got, want):
+            bad = np.argwhere(got != want)
+            raise AssertionError(f"draw {draw} {kw} style {style} two_phase {two_phase}: {len(bad)} wrong bytes, "
+                                 f"first at rep {bad[0][0]} byte {bad[0][1]}")
+
+
+def test_runtime_parameters_of_a_compile_time_case_are_refused(device):
+    full = next(i for i, c in enumerate(_CASES) if c.pattern == cd.PATTERN_STRIDED and c.level == 4)
+    io = CaseIO(_CASES[full], reps=1)
+    d_in = torch.from_numpy(io.input).to(device)
+    d_out = torch.zeros(io.lds_bytes, dtype=torch.uint8, device=device)
+    for kw in ({"bytes_per_elmt": 64}, {"dma_threads": 64}, {"num_elmts": 3}, {"dimx": 8}):
+        with pytest.raises(cd.CudaDMAError):
+            cd.harness.run_case(full, d_in, d_out, lds_bytes=io.lds_bytes, src_stride=io.src_stride,
+                                dst_stride=io.dst_stride, **kw)
+
+
 def test_halo_case_passes_the_reference_checker(device):
     """check_halo of the reference on the GPU output of the cudaDMAHalo (older interface) cases."""
     from tests import oracle_lib as ol

@@ -65,6 +65,19 @@ def test_run_case_validates_before_launching():
     r = cd.RunArgs(d_in=4096, d_out=8192, lds_bytes=1024, reps=1, src_offset_bytes=2)
     assert L.cudadma_run_case(0, ctypes.byref(r), None) == -1
     assert L.cudadma_run_case(10 ** 6, ctypes.byref(r), None) == -3
+    # run-time values are only taken for parameters the case's level leaves to its constructor
+    cases = cd.harness.all_cases()
+    full = next(i for i, c in enumerate(cases) if c.pattern == cd.PATTERN_STRIDED and c.level == 4)
+    for field in ("rt_bytes_per_elmt", "rt_dma_threads", "rt_num_elmts", "rt_dimx"):
+        r = cd.RunArgs(d_in=4096, d_out=8192, lds_bytes=1024, reps=1, **{field: 64})
+        assert L.cudadma_run_case(full, ctypes.byref(r), None) == -1, field
+        assert b"case" in L.cudadma_last_error()
+    loose = next(i for i, c in enumerate(cases) if c.pattern == cd.PATTERN_STRIDED and c.level == 1)
+    for field, value in (("rt_bytes_per_elmt", 6), ("rt_dma_threads", 100), ("rt_dma_threads", 2048), ("rt_num_elmts", -1)):
+        r = cd.RunArgs(d_in=4096, d_out=8192, lds_bytes=1024, reps=1, **{field: value})
+        assert L.cudadma_run_case(loose, ctypes.byref(r), None) == -1, (field, value)
+    assert L.cudadma_scatter_copy(4096, 4096, 8192, 16, 33, 0, None) == -1
+    assert L.cudadma_fill_permutation(4096, 0, 1, None) == -1
     # workloads: sizes and variants are checked first
     assert L.cudadma_sequential_copy(4096, 8192, 1000, 0, None) == -1
     assert L.cudadma_sequential_copy(4096, 8192, 16384, 99, None) == -3
@@ -75,7 +88,7 @@ def test_run_case_validates_before_launching():
 
 
 def test_variants_are_described():
-    for w, least in ((cd.workloads.SEQUENTIAL, 4), (cd.workloads.STRIDED, 2), (cd.workloads.GATHER, 2),
+    for w, least in ((cd.workloads.SEQUENTIAL, 4), (cd.workloads.STRIDED, 2), (cd.workloads.GATHER, 2), (cd.workloads.SCATTER, 4),
                      (cd.workloads.HALO, 2)):
         n = cd.workloads.num_variants(w)
         assert n >= least
