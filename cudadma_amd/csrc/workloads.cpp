@@ -79,8 +79,8 @@ static const VariantInfo kHalo[] = {
 };
 
 static const VariantInfo kGemm[] = {
-  {"the largest workgroup tile that divides the problem: variant 3 when m is a multiple of 256, variant 2 when only n "
-   "is, else variant 1"},
+  {"the largest workgroup tile that divides the problem and gives every compute unit a tile: variant 5, 3 or 2, else "
+   "variant 1"},
   {"warp-specialised: two DMA wavefronts per operand with two CudaDMAStrided objects each (two LDS stages, tile two K "
    "steps ahead in flight), four compute wavefronts with v_mfma_f32_32x32x16_bf16, B fragments through "
    "ds_read_b64_tr_b16; 128 x 128 workgroup tile, 64 x 64 per compute wavefront, two workgroups per compute unit"},
@@ -88,6 +88,8 @@ static const VariantInfo kGemm[] = {
   {"same structure, 256 x 128 workgroup tile, 128 x 64 per compute wavefront, one workgroup per compute unit"},
   {"256 x 128 workgroup tile with the tiles brought in by global_load_lds_dwordx4 (STORE_LDS_DIRECT_SWIZZLE): three "
    "unpadded swizzled LDS stages, two transfers in flight per DMA wavefront, no ds_write"},
+  {"256 x 256 workgroup tile (m and n multiples of 256): eight compute wavefronts of 128 x 64, two per SIMD, next to the "
+   "four DMA wavefronts; twelve wavefronts leave 168 registers each"},
 };
 
 static const VariantInfo kScatter[] = {

@@ -1,18 +1,21 @@
 // Config 5: C = A * B, bf16 inputs, fp32 accumulate, warp-specialised and
 // double-buffered.  The reference has no GEMM; the nearest code is the SGEMV of
 // src/examples/sgemv/sgemv_dma.cu:329-388 (Strided matrix tiles staged by DMA
-// warps, FMA loop in the compute warps).  Here:
-//   * workgroup tile 128 x 128 of C, K step 64;
-//   * wavefronts 4-5 stage the A tiles (128 rows x 128 B, source stride K*2 bytes),
-//     wavefronts 6-7 the B tiles (64 rows x 256 B, source stride N*2 bytes).  Each
-//     pair owns two CudaDMAStrided objects, one per LDS stage, and uses the two-phase
-//     calls so that the tile two K steps ahead is already in flight (in the
+// warps, FMA loop in the compute warps).  Here, for a workgroup tile BM x BN and K step 64:
+//   * the first WM x WN wavefronts compute, each on WI x WJ blocks of
+//     v_mfma_f32_32x32x16_bf16 (BM = 32*WI*WM, BN = 32*WJ*WN).  A fragments are
+//     ds_read_b128 from rows padded to 144 B; B stays row-major [k][n] in LDS (rows
+//     padded by 64 B) and is turned into k-major fragments on the way to the
+//     registers by ds_read_b64_tr_b16;
+//   * the next two wavefronts stage the A tiles (BM rows x 128 B, source stride K*2
+//     bytes), the last two the B tiles (64 rows x 2*BN B, source stride N*2 bytes).
+//     Each pair owns two CudaDMAStrided objects, one per LDS stage, and uses the
+//     two-phase calls so that the tile two K steps ahead is already in flight (in the
 //     object's registers) while the current one is consumed: a K step is shorter
-//     than a trip to memory, one tile of look-ahead is not enough;
-//   * wavefronts 0..3 each own a 64 x 64 quadrant: 2 x 2 blocks of
-//     v_mfma_f32_32x32x16_bf16.  A fragments are ds_read_b128 from rows padded to
-//     144 B; B stays row-major [k][n] in LDS (rows padded to 320 B) and is turned
-//     into k-major fragments on the way to the registers by ds_read_b64_tr_b16.
+//     than a trip to memory, one tile of look-ahead is not enough.
+// Four compute wavefronts (2 x 2) share the SIMDs with the four DMA wavefronts one to
+// one and get 256 registers each; eight (2 x 4, the 256 x 256 tile) make it three
+// wavefronts per SIMD and 168 registers each, but two of them compute.
 #include "workloads.hpp"
 
 namespace {
@@ -25,11 +28,12 @@ constexpr int kBK = 64;
 constexpr int kComputeThreads = 256;
 constexpr int kDmaWave = 128;              // DMA threads per operand: two wavefronts
 
-// Tile geometry for compute wavefronts that each own WI x WJ blocks of 32 x 32: the four
-// wavefronts sit 2 x 2, so the workgroup tile is 64*WI x 64*WJ.
-template<int WI, int WJ>
+// Tile geometry for compute wavefronts that each own WI x WJ blocks of 32 x 32: the WM x WN
+// wavefronts sit in a grid, so the workgroup tile is 32*WI*WM x 32*WJ*WN.
+template<int WI, int WJ, int WM = 2, int WN = 2>
 struct GemmShape {
-  static constexpr int kBM = 64 * WI, kBN = 64 * WJ;
+  static constexpr int kCompute = 64 * WM * WN;     // compute threads; the DMA threads follow them
+  static constexpr int kBM = 32 * WI * WM, kBN = 32 * WJ * WN;
   static constexpr int kAPitch = kBK * 2 + 16;      // 144 B per A row in LDS
   static constexpr int kBPitch = kBN * 2 + 64;      // B row in LDS: the four rows a transposing read touches land 64 B apart modulo 256
   static constexpr int kAStage = kBM * kAPitch;
@@ -69,12 +73,13 @@ __device__ __forceinline__ void pin_slice()
   }
 }
 
-template<int WI, int WJ>
-__global__ void __launch_bounds__(kComputeThreads + 2 * kDmaWave)
+template<int WI, int WJ, int WM = 2, int WN = 2>
+__global__ void __launch_bounds__(64 * WM * WN + 2 * kDmaWave)
 gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restrict__ b, float* __restrict__ c,
              const int m, const int n, const int k)
 {
-  typedef GemmShape<WI, WJ> shape;
+  typedef GemmShape<WI, WJ, WM, WN> shape;
+  constexpr int kComputeThreads = shape::kCompute;
   typedef typename shape::dma_a_t dma_a_t;
   typedef typename shape::dma_b_t dma_b_t;
   constexpr int kAPitch = shape::kAPitch, kBPitch = shape::kBPitch;
@@ -118,7 +123,7 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
   } else {
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int wm = (wave >> 1) * 32 * WI, wn = (wave & 1) * 32 * WJ;     // this wavefront's corner in the workgroup tile
+    const int wm = (wave / WN) * 32 * WI, wn = (wave % WN) * 32 * WJ;     // this wavefront's corner in the workgroup tile
     f32x16_t acc[WI][WJ];
 #pragma unroll
     for (int i = 0; i < WI; ++i)
@@ -139,7 +144,7 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
     // own LDS latency: the order "request the next slice, then multiply the current one" is
     // pinned against the instruction scheduler.  With the small tile two workgroups share a
     // compute unit and the scheduler's own order does better.
-    constexpr bool kPinned = (WI * WJ >= 8);
+    constexpr bool kPinned = (WI * WJ >= 8) && (WM * WN == 4);
     // Fragments of one 16-deep slice of the K step: WI row blocks of A, WJ column blocks of B.
     auto load_frags = [&](bf16x8_t (&fa)[WI], bf16x8_t (&fb)[WJ], const char* sa, const char* sb, const int ks)
         __attribute__((always_inline)) {
@@ -393,15 +398,15 @@ gemm_bf16_ws_direct(const unsigned short* __restrict__ a, const unsigned short* 
   }
 }
 
-template<int WI, int WJ>
+template<int WI, int WJ, int WM = 2, int WN = 2>
 int launch_gemm(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k, hipStream_t stream)
 {
-  typedef GemmShape<WI, WJ> shape;
+  typedef GemmShape<WI, WJ, WM, WN> shape;
   CUDADMA_REQUIRE((m % shape::kBM) == 0 && (n % shape::kBN) == 0,
                   "this variant needs m a multiple of %d and n of %d (got %d x %d)", shape::kBM, shape::kBN, m, n);
   const long long grid = (long long)(m / shape::kBM) * (n / shape::kBN);
   CUDADMA_REQUIRE(grid <= 0x7fffffffLL, "grid too large");
-  hipLaunchKernelGGL((gemm_bf16_ws<WI, WJ>), dim3((unsigned)grid), dim3(kComputeThreads + 2 * kDmaWave), 0, stream,
+  hipLaunchKernelGGL((gemm_bf16_ws<WI, WJ, WM, WN>), dim3((unsigned)grid), dim3(shape::kCompute + 2 * kDmaWave), 0, stream,
                      d_a, d_b, d_c, m, n, k);
   CUDADMA_HIP_CHECK(hipGetLastError());
   return CUDADMA_OK;
@@ -424,11 +429,20 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
                   "pointers must be 16-byte aligned");
   CUDADMA_REQUIRE((long long)k * 2 <= 0x7fffffffLL && (long long)n * 2 <= 0x7fffffffLL, "row pitch must fit an int");
   hipStream_t s = (hipStream_t)stream;
-  if (variant == 0) variant = (m % 256) == 0 ? 3 : (n % 256) == 0 ? 2 : 1;      // the largest tile that divides the problem
+  if (variant == 0) {
+    // the largest tile that divides the problem and still gives every compute unit a tile; the small one otherwise
+    const long long cus = workloads::device_cus();
+    const bool m256 = (m % 256) == 0, n256 = (n % 256) == 0;
+    if (m256 && n256 && (long long)(m / 256) * (n / 256) >= cus) variant = 5;
+    else if (m256 && (long long)(m / 256) * (n / 128) >= cus) variant = 3;
+    else if (n256 && (long long)(m / 128) * (n / 256) >= cus) variant = 2;
+    else variant = 1;
+  }
   switch (variant) {
     case 1: return launch_gemm<2, 2>(d_a, d_b, d_c, m, n, k, s);
     case 2: return launch_gemm<2, 4>(d_a, d_b, d_c, m, n, k, s);
     case 3: return launch_gemm<4, 2>(d_a, d_b, d_c, m, n, k, s);
+    case 5: return launch_gemm<4, 2, 2, 4>(d_a, d_b, d_c, m, n, k, s);
     default: {
       CUDADMA_REQUIRE((m % 256) == 0, "this variant needs m a multiple of 256 (got %d)", m);
       const long long grid = (long long)(m / 256) * (n / 128);

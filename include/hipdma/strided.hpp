@@ -232,6 +232,29 @@ private:
   __device__ __forceinline__ void load_step(const int step, hipdma::detail::GridCursor cur)
   {
     using namespace hipdma::detail;
+    if constexpr (GLOBAL_LOAD) {
+      // When a round moves every thread down whole rows (the threads cover whole rows: dcol == 0), the address
+      // splits into a part that is the same for all threads and changes per load (round * drow rows down) and a
+      // part per thread that never changes (its row and column of round 0).  Written that way the thread keeps
+      // one offset instead of a 64-bit address per load in flight, and the per-load part is scalar arithmetic.
+      if (m_grid.dcol == 0) {
+        const long long lane_part = (long long)(m_grid.row0 * m_src_stride + m_grid.col0 * ALIGNMENT);
+#pragma unroll
+        for (int k = 0; k < MAX_LDS; ++k) {
+          if (m_grid.live(step * MAX_LDS + k, cur)) {
+            // the same value in every lane (object parameters are); saying so keeps it in scalar registers
+            const long long rows_down = (long long)((step * MAX_LDS + k) * m_grid.drow) * (long long)m_src_stride;
+            const long long uniform = (long long)(
+                ((unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)((unsigned long long)rows_down >> 32)) << 32) |
+                (unsigned long long)__builtin_amdgcn_readfirstlane((unsigned)(unsigned long long)rows_down));
+            load_chunk<ALIGNMENT, ALIGNMENT, GLOBAL_LOAD, LOAD_QUAL>(m_buf[k], m_src + uniform + lane_part,
+                                                                     m_grid.chunk_bytes(ALIGNMENT, cur));
+          }
+          m_grid.advance(cur);
+        }
+        return;
+      }
+    }
 #pragma unroll
     for (int k = 0; k < MAX_LDS; ++k) {
       if (m_grid.live(step * MAX_LDS + k, cur))
