@@ -3,7 +3,7 @@ compute unit, timed with HIP events.  The counterpart of the reference's
 src/perf/sequential/param_sweep.py:27-58, which rewrites params_directed.h and recompiles per
 point; here the variants are compiled in and the occupancy is a run-time knob.
 
-    python -m cudadma_amd.sweep [sequential] [strided] [gather] [scatter] [halo] [gemm] [--wg 0,2,4,8] [--steps 20]
+    python -m cudadma_amd.sweep [sequential] [strided] [gather] [scatter] [halo] [gemm] [memory] [--wg 0,2,4,8] [--steps 20]
     python -m cudadma_amd.sweep saxpy sgemv stencil2d        # the reference's example programs, every variant
     python -m cudadma_amd.sweep perf_sequential --wg 2,8     # read-bandwidth probe: element size x DMA wavefronts x buffering
 """
@@ -84,6 +84,21 @@ def main(argv=None):
                     wl.set_workgroups_per_cu(wg)
                     _row(name, v, wg, _time(lambda: wl.gather_rowsum(table, idx, out, v), args.steps),
                          n_idx * 132 + out.numel() * 4)
+        elif name == "memory":
+            # what copy-shaped kernels without LDS reach on 1 GiB + 1 GiB, per launch shape
+            n = 16384
+            src = wl.fill_uniform(torch.empty(n * n, device=dev), 1002)
+            dst = torch.empty_like(src)
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            print("# memory probes on 2 x 1 GiB; GB/s of bytes read + written; columns: workgroups per CU 2 / 4 / 8 / 16")
+            for mode, label in enumerate(wl.PROBE_MODES):
+                cells = []
+                for wg in (2, 4, 8, 16):
+                    s_, d_ = (None if label.startswith("write") else src), (None if label == "read" else dst)
+                    nbytes = wl.probe_memory(mode, s_, d_, cus * wg)
+                    ms = _time(lambda: wl.probe_memory(mode, s_, d_, cus * wg), args.steps, settle_ms=10.0)
+                    cells.append(f"{ms:7.4f} ms {nbytes / ms / 1e6:6.0f}")
+                print(f"{label:22s} " + "   ".join(cells), flush=True)
         elif name == "scatter":
             recs = 4 << 20
             records = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1006)

@@ -157,6 +157,26 @@ def perf_sequential(src, elmt_bytes, dma_wavefronts, buffering, loop_iters, work
     return int(n)
 
 
+PROBE_MODES = ("read", "write", "write_nontemporal", "copy", "copy_nontemporal", "blocks_in_place", "blocks_swapped",
+               "blocks_permuted", "write_blocks_swapped")
+
+
+def probe_memory(mode, src, dst, workgroups):
+    """One launch of a memory-system probe (mode: index into PROBE_MODES or its name).  src / dst are CUDA tensors
+    of the same size in bytes (None where the mode does not use one).  Returns bytes read + bytes written."""
+    if isinstance(mode, str):
+        mode = PROBE_MODES.index(mode)
+    t = src if src is not None else dst
+    nbytes = t.numel() * t.element_size()
+    if src is not None and dst is not None and dst.numel() * dst.element_size() != nbytes:
+        raise ValueError("src and dst differ in size")
+    n = lib().cudadma_probe_memory(mode, _p(src) if src is not None else None, _p(dst) if dst is not None else None,
+                                   nbytes, int(workgroups), _stream())
+    if n < 0:
+        check(int(n))
+    return int(n)
+
+
 def gemm_bf16(a, b, c, variant=0):
     """a: (m, k) and b: (k, n) torch.bfloat16, c: (m, n) float32; returns c = a @ b with fp32 accumulation."""
     _need(a, torch.bfloat16, "a")

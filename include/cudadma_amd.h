@@ -254,6 +254,27 @@ enum {
 long long cudadma_perf_sequential(const void* d_src, size_t src_bytes, unsigned* d_sums, int elmt_bytes,
                                   int dma_wavefronts, int buffering, int loop_iters, int workgroups, void* stream);
 
+/* ---- memory-system probes --------------------------------------------------------------
+ * Kernels without LDS and without a DMA object that show what a copy-shaped kernel reaches on the
+ * device and what the placement of the blocks costs: the yardsticks for config 2.  No counterpart
+ * in the reference.  `bytes` is the size of each buffer (a multiple of 16); the block modes view
+ * the buffers as n x n float matrices (bytes = 4 n^2, n a power of two >= 64) cut into blocks of
+ * 64 rows x 256 B, one block per wavefront and step.  Write-only modes store the float 1.0.
+ * Returns the bytes read plus the bytes written, or a negative CUDADMA_E* code. */
+enum {
+  CUDADMA_PROBE_READ                 = 0,  /* d_dst may be NULL                                    */
+  CUDADMA_PROBE_WRITE                = 1,  /* d_src may be NULL                                    */
+  CUDADMA_PROBE_WRITE_NONTEMPORAL    = 2,
+  CUDADMA_PROBE_COPY                 = 3,  /* grid-stride dwordx4                                  */
+  CUDADMA_PROBE_COPY_NONTEMPORAL     = 4,
+  CUDADMA_PROBE_BLOCKS_IN_PLACE      = 5,  /* block (r, c) -> block (r, c)                         */
+  CUDADMA_PROBE_BLOCKS_SWAPPED       = 6,  /* block (r, c) -> block (c, r), contents not transposed */
+  CUDADMA_PROBE_BLOCKS_PERMUTED      = 7,  /* in place, blocks visited in a scattered order        */
+  CUDADMA_PROBE_WRITE_BLOCKS_SWAPPED = 8,  /* mode 6 without its loads                             */
+  CUDADMA_PROBE_MODES                = 9
+};
+long long cudadma_probe_memory(int mode, const void* d_src, void* d_dst, size_t bytes, int workgroups, void* stream);
+
 /* ---- known-answer cases for the first-generation class names -------------------------
  * One transfer per case by cudaDMASequential / cudaDMAStrided / cudaDMAIndirect as declared in
  * include/cudaDMA.h:644-3580 (every constructor form), into a 16 KiB LDS window that holds the

@@ -341,6 +341,42 @@ def test_gemm_rejects_ragged_shapes(device):
         wl.gemm_bf16(a, b, c)
 
 
+# ------------------------------------------------------------------ memory-system probes
+@pytest.mark.parametrize("workgroups", [1, 7, 512])
+def test_memory_probes_move_what_they_say(device, workgroups):
+    n = 256                                                     # 256 x 256 floats: 4 x 4 blocks of 64 rows x 256 B
+    src = wl.fill_uniform(torch.empty(n * n, dtype=torch.float32, device=device), 77)
+    nbytes = src.numel() * 4
+    want_blocks = src.view(n // 64, 64, n // 64, 64)            # [block row][row][block column][column]
+    for mode, label in enumerate(wl.PROBE_MODES):
+        dst = torch.full_like(src, -3.0)
+        print(f"probe {label} workgroups {workgroups}", flush=True)
+        moved = wl.probe_memory(mode, None if label.startswith("write") else src, None if label == "read" else dst, workgroups)
+        torch.cuda.synchronize()
+        assert moved == nbytes * ((0 if label.startswith("write") else 1) + (0 if label == "read" else 1))
+        if label == "read":
+            continue
+        if label.startswith("write"):
+            assert bool((dst == 1.0).all())
+        elif label == "blocks_swapped":
+            got = dst.view(n // 64, 64, n // 64, 64)
+            assert torch.equal(got.view(torch.int32), want_blocks.permute(2, 1, 0, 3).contiguous().view(torch.int32))
+        else:
+            assert torch.equal(dst.view(torch.int32), src.view(torch.int32))
+
+
+def test_memory_probe_argument_checks(device):
+    t = torch.zeros(64 * 64, dtype=torch.float32, device=device)
+    with pytest.raises(cd.CudaDMAError):
+        wl.probe_memory(len(wl.PROBE_MODES), t, t.clone(), 4)
+    with pytest.raises(cd.CudaDMAError):
+        wl.probe_memory("copy", t, t.clone(), 0)
+    with pytest.raises(cd.CudaDMAError, match="power of two"):
+        wl.probe_memory("blocks_swapped", t[:3 * 64 * 64 // 4], t.clone()[:3 * 64 * 64 // 4], 4)
+    with pytest.raises(cd.CudaDMAError, match="NULL"):
+        wl.probe_memory("copy", t, None, 4)
+
+
 # ------------------------------------------------------------------ read-bandwidth probe (perf_sequential)
 @pytest.mark.parametrize("buffering", range(4))
 @pytest.mark.parametrize("elmt,waves,loops,groups", [(32, 1, 1, 3), (48, 2, 5, 7), (4096, 2, 8, 64), (16384, 4, 3, 33),
