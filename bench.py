@@ -166,7 +166,15 @@ def main():
     # yardstick on the same buffers: plain dwordx4 copy
     copy_ms, _ = time_launches(lambda: wl.plain_copy(src, dst), steps, warmup, SETTLE_MS)
     report("plain_copy", copy_ms, strided_bytes, "grid-stride dwordx4 copy of 1 GiB, no LDS, no DMA object")
-    del src, dst
+    # two more yardsticks on the same buffers: the copy at its best launch shape, and the blocks of the
+    # transposition moved through registers to their transposed position (no LDS, contents not transposed)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    flat_src, flat_dst = src.view(-1), dst.view(-1)
+    ms, _ = time_launches(lambda: wl.probe_memory("copy_nontemporal", flat_src, flat_dst, 4 * cus), steps, warmup, SETTLE_MS)
+    report("copy_best_shape", ms, strided_bytes, "the same copy with non-temporal stores at 4 workgroups per compute unit, its best launch shape")
+    ms, _ = time_launches(lambda: wl.probe_memory("blocks_swapped", flat_src, flat_dst, 8 * cus), steps, warmup, SETTLE_MS)
+    report("blocks_swapped", ms, strided_bytes, "64 x 256 B blocks through registers to the transposed block position: the placement cost of config 2 without LDS")
+    del src, dst, flat_src, flat_dst
 
     # ---- config 1: sequential copy, 64 MiB in 16 KiB tiles ----
     m = 64 * 1024 * 1024 // 4
