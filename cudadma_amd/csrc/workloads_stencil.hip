@@ -370,15 +370,19 @@ stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int
       ring.get<(I)>().template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(&plane[(I) % kBufs][kOrigin]); \
       if constexpr (SYNC != kBarrierOnly) guard.get<(I) % kBufs>().finish_async_dma();                       \
     }
-    // planes 0 .. kRingAhead-1 are requested up front; plane 0 lands before the first barrier
+    // With the handshake the ring lands two planes ahead of its use instead of one: the compute
+    // wavefronts then find the `full` word of a plane set when they first look, and never poll.
+    constexpr int kLand = (SYNC == kBarrierOnly) ? 1 : 2;
+    // planes 0 .. kRingAhead-1 are requested up front; planes 0 .. kLand-1 land before the first barrier
     HIPDMA_ISSUE(0, 0) HIPDMA_ISSUE(1, 1) HIPDMA_ISSUE(2, 2) HIPDMA_ISSUE(3, 3)
     HIPDMA_ISSUE(4, 4) HIPDMA_ISSUE(5, 5) HIPDMA_ISSUE(6, 6)
     HIPDMA_LAND(0, 0)
-    // iteration z: request plane z + kRingAhead, meet the compute wavefronts, land plane z + 1
+    if constexpr (kLand == 2) { HIPDMA_LAND(1, 1) }
+    // iteration z: request plane z + kRingAhead, meet the compute wavefronts, land plane z + kLand
     HIPDMA_FOR_RING(w.planes, {
       HIPDMA_ISSUE((S + kRingAhead) % kRingObjs, z + kRingAhead)
       if constexpr (SYNC != kHandshakeAndGroupBarrier) __syncthreads();
-      HIPDMA_LAND((S + 1) % kRingObjs, z + 1)
+      HIPDMA_LAND((S + kLand) % kRingObjs, z + kLand)
     })
 #undef HIPDMA_ISSUE
 #undef HIPDMA_LAND
@@ -414,11 +418,13 @@ stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int
       if constexpr (SYNC == kHandshakeAndGroupBarrier) compute_barrier.sync();
       else __syncthreads();
       const f32x4_t r = stencil_cells4<ROT>(plane[B], lx, ly, q, k);
-      if constexpr (SYNC != kBarrierOnly) cur_halo.start_async_dma();
       if constexpr (SYNC != kBarrierOnly) seen = guard.get<(B + 1) % kBufs>().peek_dma_finish();
       *(f32x4_t*)(&plane[(B + 1) % kBufs][kOrigin] + ly * kPitch + lx) = q[HIPDMA_QSLOT(ROT, kR + 1)];
       *(f32x4_t*)o = r;
       o += out_plane;
+      // The plane is released last: the store above already had to wait for every LDS read of the
+      // plane, so the release fence finds nothing left to wait for.
+      if constexpr (SYNC != kBarrierOnly) cur_halo.start_async_dma();
     })
   }
 }
