@@ -128,12 +128,13 @@ extern "C" int cudadma_scatter_copy(const float* d_records, const int32_t* d_idx
   const long long tiles = (long long)(n_idx / kRecsPerTile);
   hipStream_t s = (hipStream_t)stream;
   const dim3 block(kDmaThreads + kComputeThreads);
-  const dim3 grid(workloads::persistent_grid(tiles, 8));
+  // workgroups per compute unit: four where several tiles are buffered, eight where one is
+  const dim3 few(workloads::persistent_grid(tiles, 4)), many(workloads::persistent_grid(tiles, 8));
   switch (variant) {
-    case 0: hipLaunchKernelGGL(scatter_manual<4>, grid, block, 0, s, d_records, d_idx, d_table, tiles); break;
-    case 1: hipLaunchKernelGGL(scatter_manual<1>, grid, block, 0, s, d_records, d_idx, d_table, tiles); break;
-    case 2: hipLaunchKernelGGL(scatter_manual<2>, grid, block, 0, s, d_records, d_idx, d_table, tiles); break;
-    default: hipLaunchKernelGGL(scatter_not_specialized, grid, block, 0, s, d_records, d_idx, d_table, tiles); break;
+    case 0: hipLaunchKernelGGL(scatter_manual<4>, few, block, 0, s, d_records, d_idx, d_table, tiles); break;
+    case 1: hipLaunchKernelGGL(scatter_manual<1>, many, block, 0, s, d_records, d_idx, d_table, tiles); break;
+    case 2: hipLaunchKernelGGL(scatter_manual<2>, few, block, 0, s, d_records, d_idx, d_table, tiles); break;
+    default: hipLaunchKernelGGL(scatter_not_specialized, many, block, 0, s, d_records, d_idx, d_table, tiles); break;
   }
   CUDADMA_HIP_CHECK(hipGetLastError());
   return CUDADMA_OK;
