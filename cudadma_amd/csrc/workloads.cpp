@@ -60,6 +60,8 @@ static const VariantInfo kStrided[] = {
   {"two DMA groups, unpadded 256 B LDS rows filled by global_load_lds_dwordx4 with XOR-swizzled chunks "
    "(STORE_LDS_DIRECT_SWIZZLE): no VGPR staging, no padding, no bank conflicts"},
   {"two DMA groups, unpadded 256 B LDS rows with XOR-swizzled chunks written from registers (STORE_LDS_SWIZZLE)"},
+  {"as variant 0, but the compute lanes transpose 4 x 4 words inside each quad (quad-permute moves) and write "
+   "dwordx4: one store covers four output rows of 256 contiguous bytes instead of one"},
 };
 static const VariantInfo kGather[] = {
   {"manual 4-stage buffering: one DMA group of 2 wavefronts, four CudaDMAIndirect objects"},

@@ -33,7 +33,26 @@ __device__ __forceinline__ void tile_coords(const int t, const int tiles_per_sid
   ty = band * band_rows + (in_band - tx * band_rows);
 }
 
-template<int LDS_ROW_BYTES, bool SWIZZLED = false, typename Dma>
+// 4 x 4 transposition among the four lanes of a quad: lane i of the quad gives word k to lane k and
+// ends up holding word i of lanes 0..3 (two butterfly stages of quad-permute moves).
+template<int CTRL>
+__device__ __forceinline__ unsigned quad_move(const unsigned v)
+{ return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false); }
+
+__device__ __forceinline__ vec4_t quad_transpose(const vec4_t a, const int lane)
+{
+  constexpr int kSwapPairs = 0x4E;     // quad_perm [2, 3, 0, 1]
+  constexpr int kSwapLanes = 0xB1;     // quad_perm [1, 0, 3, 2]
+  const bool upper = (lane & 2) != 0, odd = (lane & 1) != 0;
+  const unsigned p0 = quad_move<kSwapPairs>(a[0]), p1 = quad_move<kSwapPairs>(a[1]);
+  const unsigned p2 = quad_move<kSwapPairs>(a[2]), p3 = quad_move<kSwapPairs>(a[3]);
+  const vec4_t b = {upper ? p2 : a[0], upper ? p3 : a[1], upper ? a[2] : p0, upper ? a[3] : p1};
+  const unsigned q0 = quad_move<kSwapLanes>(b[0]), q1 = quad_move<kSwapLanes>(b[1]);
+  const unsigned q2 = quad_move<kSwapLanes>(b[2]), q3 = quad_move<kSwapLanes>(b[3]);
+  return vec4_t{odd ? q1 : b[0], odd ? b[1] : q0, odd ? q3 : b[2], odd ? b[3] : q2};
+}
+
+template<int LDS_ROW_BYTES, bool SWIZZLED = false, bool QUAD = false, typename Dma>
 __device__ __forceinline__ void write_tile_transposed(const char* lds_tile, float* __restrict__ out, const int n,
                                                       const int ty, const int tx, const Dma& dma)
 {
@@ -49,16 +68,25 @@ __device__ __forceinline__ void write_tile_transposed(const char* lds_tile, floa
   for (int j = 0; j < 8; ++j) v[j] = row[SWIZZLED ? hipdma::swizzled_chunk(lane, w * 8 + j, kRowBytes / 16) : (w * 8 + j)];
   dma.start_async_dma();
   // element (r = lane, c) of the tile goes to out[(tx*64 + c) * n + ty*64 + r]
-  float* o = out + (size_t)(tx * kTile + w * 32) * n + (size_t)ty * kTile + lane;
+  if constexpr (QUAD) {
+    // After the transposition inside each quad, lane 4q + i holds rows 4q .. 4q+3 of tile column
+    // 32w + 4j + i: four consecutive words of output row 32w + 4j + i.  One dwordx4 store per unit
+    // then covers four output rows with 256 contiguous bytes each.
+    float* o = out + (size_t)(tx * kTile + w * 32 + (lane & 3)) * n + (size_t)ty * kTile + (lane & ~3);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < 8; ++j) *(vec4_t*)(o + (size_t)(4 * j) * n) = quad_transpose(v[j], lane);
+  } else {
+    float* o = out + (size_t)(tx * kTile + w * 32) * n + (size_t)ty * kTile + lane;
 #pragma unroll
-    for (int k = 0; k < 4; ++k)
-      o[(size_t)(4 * j + k) * n] = __uint_as_float(v[j][k]);
+    for (int j = 0; j < 8; ++j) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        o[(size_t)(4 * j + k) * n] = __uint_as_float(v[j][k]);
+    }
   }
 }
 
-template<int LDS_ROW_BYTES>
+template<int LDS_ROW_BYTES, bool QUAD = false>
 __global__ void __launch_bounds__(kDmaThreads + kComputeThreads)
 transpose_manual_double(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles,
                         const int band)
@@ -110,11 +138,11 @@ transpose_manual_double(const float* __restrict__ in, float* __restrict__ out, c
       int ty, tx;
       tile_coords(t, tiles_per_side, band, ty, tx);
       dma0.wait_for_dma_finish();
-      write_tile_transposed<LDS_ROW_BYTES>(buf0, out, n, ty, tx, dma0);
+      write_tile_transposed<LDS_ROW_BYTES, false, QUAD>(buf0, out, n, ty, tx, dma0);
       if (t + stride < num_tiles) {
         tile_coords(t + stride, tiles_per_side, band, ty, tx);
         dma1.wait_for_dma_finish();
-        write_tile_transposed<LDS_ROW_BYTES>(buf1, out, n, ty, tx, dma1);
+        write_tile_transposed<LDS_ROW_BYTES, false, QUAD>(buf1, out, n, ty, tx, dma1);
       }
     }
   }
@@ -269,6 +297,7 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
     case 3: hipLaunchKernelGGL(transpose_double_groups<272>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 5: hipLaunchKernelGGL((transpose_double_groups<256, STORE_LDS_DIRECT_SWIZZLE>), dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 6: hipLaunchKernelGGL((transpose_double_groups<256, STORE_LDS_SWIZZLE>), dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 7: hipLaunchKernelGGL((transpose_manual_double<272, true>), dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
     default: hipLaunchKernelGGL(transpose_not_specialized, dim3(workloads::persistent_grid(tiles, 6)), block, 0, s, d_in, d_out, n, tiles, band); break;
   }
   CUDADMA_HIP_CHECK(hipGetLastError());
