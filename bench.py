@@ -5,7 +5,10 @@
 
 A step is one launch of the CudaDMAStrided tile-transpose kernel over the whole
 16384 x 16384 float32 matrix (benchmark config 2, the configuration the metric is
-quoted on); inputs are resident in HBM before the timed region.  The other three
+quoted on); inputs are resident in HBM before the timed region.  The kernel is the
+warp-specialised one with one LDS tile (the next tile waits in the DMA wavefronts'
+registers), one workgroup per compute unit; the kernel with two LDS tiles and two
+objects, which needs four workgroups per compute unit, is reported beside it.  The other three
 HBM-bound patterns (sequential copy, indirect gather, halo stencil), the scatter in
 the opposite direction and a plain copy kernel are timed the same way and reported
 under "patterns".  One JSON line goes to stdout; progress goes to stderr.
@@ -25,8 +28,9 @@ SETTLE_MS = 30.0                # wall time of untimed warm-up for the secondary
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # scaled by what the same counters read for the plain copy kernel (see profiles/).
-# profiles/bench_all_patterns_mi355x.md: FETCH_SIZE 524393 KiB x 1.99995 + WRITE_SIZE 1048576 KiB x 1.00000.
-MEASURED_TRAFFIC_BYTES = {"strided": 2147667896}
+# profiles/bench_all_patterns_mi355x.md: FETCH_SIZE 524323 KiB x 1.99996 + WRITE_SIZE 1048576 KiB x 1.00000.
+MEASURED_TRAFFIC_BYTES = {"strided": 2147534527}
+STRIDED_VARIANT = 1             # cudadma_strided_transpose variant timed as the headline
 
 
 def log(msg):
@@ -160,9 +164,13 @@ def main():
     n = 16384
     src = wl.fill_uniform(torch.empty(n * n, dtype=torch.float32, device=dev), 1002).view(n, n)
     dst = torch.empty_like(src)
-    strided_ms, strided_wall_ms = time_launches(lambda: wl.strided_transpose(src, dst, 0), steps, warmup)
+    strided_ms, strided_wall_ms = time_launches(lambda: wl.strided_transpose(src, dst, STRIDED_VARIANT), steps, warmup)
     strided_bytes = 2 * n * n * 4
-    report("strided", strided_ms, strided_bytes, "CudaDMAStrided 64x256B tiles of a 16384^2 f32 matrix, transposed out")
+    report("strided", strided_ms, strided_bytes, "CudaDMAStrided 64x256B tiles of a 16384^2 f32 matrix, transposed out: one LDS tile, "
+           "the next tile in the DMA wavefronts' registers, one workgroup per compute unit")
+    ms, _ = time_launches(lambda: wl.strided_transpose(src, dst, 0), steps, warmup, SETTLE_MS)
+    report("strided_two_lds_tiles", ms, strided_bytes, "the same transposition with two LDS tiles and two CudaDMAStrided objects "
+           "(manual double buffering), four workgroups per compute unit")
     # yardstick on the same buffers: plain dwordx4 copy
     copy_ms, _ = time_launches(lambda: wl.plain_copy(src, dst), steps, warmup, SETTLE_MS)
     report("plain_copy", copy_ms, strided_bytes, "grid-stride dwordx4 copy of 1 GiB, no LDS, no DMA object")
@@ -244,13 +252,14 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "CudaDMAStrided 2D tile extraction: 16384x16384 f32, 64 rows x 256 B tiles, "
-                               "double-buffered, transposed to output (benchmark config 2 of 5)",
+        "config": {"workload": "CudaDMAStrided 2D tile extraction: 16384x16384 f32, 64 rows x 256 B tiles at 65536 B stride, "
+                               "one tile in LDS and the next in the DMA wavefronts' registers, transposed to output "
+                               "(benchmark config 2 of 5)",
                    "tile_rows": 64, "tile_row_bytes": 256, "src_stride_bytes": 65536,
-                   "workgroup": "128 DMA + 128 compute threads"},
+                   "workgroup": "128 DMA + 128 compute threads", "workgroups": "one per compute unit"},
         "roofline": {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(value / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES["strided"],
-                     "kernel": "transpose_manual_double<272>", "kernel_ms": round(strided_ms, 4),
+                     "kernel": "transpose_single", "kernel_ms": round(strided_ms, 4),
                      "algorithmic_bytes_per_launch": strided_bytes},
         "patterns": patterns,
         "gemm": gemm,

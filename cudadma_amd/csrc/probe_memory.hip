@@ -7,6 +7,7 @@
 // the tile of config 2; a wavefront moves one block per step through registers (16 dwordx4 per
 // lane in flight) and the wavefronts walk the blocks grid-stride.
 #include "workloads.hpp"
+#include <type_traits>
 
 namespace {
 using workloads::vec4_t;
@@ -90,6 +91,55 @@ probe_blocks(const char* __restrict__ in, char* __restrict__ out, const size_t p
   }
 }
 
+// The transposition itself without a DMA object and without any synchronisation between wavefronts:
+// every wavefront brings its own block into a private LDS tile (rows padded to 272 B), reads it back
+// row per lane, transposes 4 x 4 words inside each quad of lanes and writes dwordx4.  out = in^T.
+__device__ __forceinline__ vec4_t probe_quad_transpose(const vec4_t a, const int lane)
+{
+  auto mv = [](const unsigned v, auto ctrl) { return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, decltype(ctrl)::value, 0xf, 0xf, false); };
+  typedef std::integral_constant<int, 0x4E> pairs;   // quad_perm [2, 3, 0, 1]
+  typedef std::integral_constant<int, 0xB1> lanes;   // quad_perm [1, 0, 3, 2]
+  const bool upper = (lane & 2) != 0, odd = (lane & 1) != 0;
+  const unsigned p0 = mv(a[0], pairs()), p1 = mv(a[1], pairs()), p2 = mv(a[2], pairs()), p3 = mv(a[3], pairs());
+  const vec4_t b = {upper ? p2 : a[0], upper ? p3 : a[1], upper ? a[2] : p0, upper ? a[3] : p1};
+  const unsigned q0 = mv(b[0], lanes()), q1 = mv(b[1], lanes()), q2 = mv(b[2], lanes()), q3 = mv(b[3], lanes());
+  return vec4_t{odd ? q1 : b[0], odd ? b[1] : q0, odd ? q3 : b[2], odd ? b[3] : q2};
+}
+
+__global__ void __launch_bounds__(kThreads)
+probe_transpose_private(const char* __restrict__ in, char* __restrict__ out, const size_t pitch, const size_t num_blocks,
+                        const int blocks_per_row)
+{
+  constexpr int kLdsRow = kSegBytes + 16;
+  __shared__ __attribute__((aligned(16))) char tiles[kThreads / 64][kBlockRows * kLdsRow];
+  const int lane = threadIdx.x & 63;
+  char* tile = tiles[threadIdx.x >> 6];
+  const size_t wave = (size_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+  const size_t waves = (size_t)gridDim.x * (kThreads / 64);
+  const int seg = lane >> 4, off = (lane & 15) * 16;
+  for (size_t b = wave; b < num_blocks; b += waves) {
+    const size_t brow = b / blocks_per_row, bcol = b % blocks_per_row;
+    const char* src = in + brow * kBlockRows * pitch + bcol * kSegBytes;
+    vec4_t v[kBlockRows / 4];
+#pragma unroll
+    for (int i = 0; i < kBlockRows / 4; ++i) v[i] = *(const vec4_t*)(src + (size_t)(i * 4 + seg) * pitch + off);
+#pragma unroll
+    for (int i = 0; i < kBlockRows / 4; ++i) *(vec4_t*)(tile + (i * 4 + seg) * kLdsRow + off) = v[i];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const vec4_t* row = (const vec4_t*)(tile + lane * kLdsRow);
+#pragma unroll
+    for (int j = 0; j < kBlockRows / 4; ++j) v[j] = row[j];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    // lane 4q + i now gets rows 4q .. 4q+3 of block column 4j + i: four words of output row 4j + i
+    char* dst = out + (bcol * kBlockRows + (lane & 3)) * pitch + brow * kSegBytes + (size_t)(lane & ~3) * 4;
+#pragma unroll
+    for (int j = 0; j < kBlockRows / 4; ++j) *(vec4_t*)(dst + (size_t)(4 * j) * pitch) = probe_quad_transpose(v[j], lane);
+  }
+}
+
 }  // namespace
 
 extern "C" long long cudadma_probe_memory(int mode, const void* d_src, void* d_dst, size_t bytes, int workgroups,
@@ -133,7 +183,8 @@ extern "C" long long cudadma_probe_memory(int mode, const void* d_src, void* d_d
     case CUDADMA_PROBE_BLOCKS_IN_PLACE: hipLaunchKernelGGL(probe_blocks<kInPlace>, grid, block, 0, s, in, out, pitch, num_blocks, blocks_per_row); break;
     case CUDADMA_PROBE_BLOCKS_SWAPPED: hipLaunchKernelGGL(probe_blocks<kSwapped>, grid, block, 0, s, in, out, pitch, num_blocks, blocks_per_row); break;
     case CUDADMA_PROBE_BLOCKS_PERMUTED: hipLaunchKernelGGL(probe_blocks<kPermuted>, grid, block, 0, s, in, out, pitch, num_blocks, blocks_per_row); break;
-    default: hipLaunchKernelGGL(probe_blocks<kWriteOnlySwapped>, grid, block, 0, s, in, out, pitch, num_blocks, blocks_per_row); break;
+    case CUDADMA_PROBE_WRITE_BLOCKS_SWAPPED: hipLaunchKernelGGL(probe_blocks<kWriteOnlySwapped>, grid, block, 0, s, in, out, pitch, num_blocks, blocks_per_row); break;
+    default: hipLaunchKernelGGL(probe_transpose_private, grid, block, 0, s, in, out, pitch, num_blocks, blocks_per_row); break;
   }
   CUDADMA_HIP_CHECK(hipGetLastError());
   return (long long)((reads ? bytes : 0) + (writes ? bytes : 0));

@@ -28,7 +28,7 @@ struct Knob {
   const char* name;
   std::atomic<int> value;
 };
-static Knob g_knobs[] = {{"transpose_band", {0}}, {"stencil_zchunk", {0}}, {"stencil_xcd_remap", {0}}};
+static Knob g_knobs[] = {{"transpose_band", {0}}, {"transpose_workgroups", {0}}, {"stencil_zchunk", {0}}, {"stencil_xcd_remap", {0}}};
 
 static Knob* find_knob(const char* name)
 {
@@ -53,7 +53,8 @@ static const VariantInfo kSequential[] = {
 };
 static const VariantInfo kStrided[] = {
   {"manual double buffer: one DMA group of 2 wavefronts, two CudaDMAStrided objects, padded LDS rows (272 B)"},
-  {"single buffer: one object, execute_dma"},
+  {"single buffer: one object and one LDS tile, execute_dma (the next tile waits in the DMA wavefronts' registers); one "
+   "workgroup per compute unit, tiles walked down the columns: the fastest shape"},
   {"manual double buffer, unpadded LDS rows (256 B): shows the bank-conflict cost"},
   {"double buffer: two DMA groups of 1 wavefront, one CudaDMAStrided object and one padded LDS tile each"},
   {"not warp-specialised: all four wavefronts move the tile and write it out, next tile requested two-phase"},
@@ -62,6 +63,9 @@ static const VariantInfo kStrided[] = {
   {"two DMA groups, unpadded 256 B LDS rows with XOR-swizzled chunks written from registers (STORE_LDS_SWIZZLE)"},
   {"as variant 0, but the compute lanes transpose 4 x 4 words inside each quad (quad-permute moves) and write "
    "dwordx4: one store covers four output rows of 256 contiguous bytes instead of one"},
+  {"one DMA wavefront and one compute wavefront per workgroup, two objects of a whole tile each on the DMA "
+   "wavefront, two LDS tiles; dword stores"},
+  {"as variant 8 with the quad transposition and dwordx4 stores of variant 7"},
 };
 static const VariantInfo kGather[] = {
   {"manual 4-stage buffering: one DMA group of 2 wavefronts, four CudaDMAIndirect objects"},

@@ -102,7 +102,8 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
   // One DMA wavefront: tiles kt and kt+1 are requested up front, then every landed tile is
   // followed by the request for the tile two steps on (clamped past the end so that no load
   // sits behind a branch and s_waitcnt can leave the younger tile in flight).
-  auto stage_tiles = [&](auto& d0, auto& d1, char* s0, char* s1, const unsigned short* src, const size_t step) {
+  auto stage_tiles = [&](auto& d0, auto& d1, char* s0, char* s1, const unsigned short* src, const size_t step)
+      __attribute__((always_inline)) {
     d0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src);
     d1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src + step);
     for (int kt = 0; kt < ksteps; kt += 2) {
@@ -273,7 +274,8 @@ gemm_bf16_ws_direct(const unsigned short* __restrict__ a, const unsigned short* 
   // One DMA wavefront: tile t lands in stage t % 3.  Tiles t+1 and t+2 are in flight while the
   // compute wavefronts work on tile t: the wavefront waits for tile t (leaving the younger
   // loads in flight), reports it, and then requests tile t+2 as soon as its stage is free.
-  auto feed = [&](auto& dma, char* lds, auto stage_bytes, const unsigned short* src, const size_t step) {
+  auto feed = [&](auto& dma, char* lds, auto stage_bytes, const unsigned short* src, const size_t step)
+      __attribute__((always_inline)) {
     constexpr int kStageBytes = decltype(stage_bytes)::value;
     constexpr int kLoads = std::remove_reference<decltype(dma)>::type::loads_per_thread();
     stage.a0.wait_for_dma_start_direct();

@@ -123,7 +123,8 @@ stencil_warp_specialized(const float* __restrict__ in, float* __restrict__ out, 
     const float* next = col + (size_t)(2 * kR) * in_plane;
     float* o = w.out_origin + (size_t)ly * nx + lx;
 
-    auto one_plane = [&](const float* cur_plane, float* other_origin, const halo_ws_t& cur_halo, const bool last) {
+    auto one_plane = [&](const float* cur_plane, float* other_origin, const halo_ws_t& cur_halo, const bool last)
+        __attribute__((always_inline)) {
       // slide the queue and fetch the newest plane
 #pragma unroll
       for (int i = 0; i < kCells; ++i) {

@@ -148,6 +148,74 @@ transpose_manual_double(const float* __restrict__ in, float* __restrict__ out, c
   }
 }
 
+// The smallest warp-specialised shape: one DMA wavefront and one compute wavefront per workgroup, two
+// objects on the DMA wavefront (each holds a whole tile, 16 dwordx4 per lane), two LDS tiles.  The
+// handshake then runs between two wavefronts only.
+template<bool QUAD>
+__global__ void __launch_bounds__(128)
+transpose_pairs(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles, const int band)
+{
+  constexpr int kLdsRow = 272;
+  __shared__ __attribute__((aligned(16))) char buf0[kTile * kLdsRow];
+  __shared__ __attribute__((aligned(16))) char buf1[kTile * kLdsRow];
+  typedef CudaDMAStrided<true, 16, kTile * kRowBytes / 64, kRowBytes, 64, kTile> dma_t;
+  dma_t dma0(0, 64, 64, n * 4, kLdsRow);
+  dma_t dma1(1, 64, 64, n * 4, kLdsRow);
+  const int tiles_per_side = n / kTile;
+  const int stride = gridDim.x;
+  auto src_of = [&](const int t) {
+    int ty, tx;
+    tile_coords(t, tiles_per_side, band, ty, tx);
+    return (const void*)(in + (size_t)ty * kTile * n + (size_t)tx * kTile);
+  };
+  if (dma0.owns_this_thread()) {
+    int t = blockIdx.x;
+    if (t < num_tiles) dma0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t));
+    if (t + stride < num_tiles) dma1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t + stride));
+    for (; t < num_tiles; t += 2 * stride) {
+      dma0.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf0);
+      if (t + 2 * stride < num_tiles) dma0.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t + 2 * stride));
+      if (t + stride < num_tiles) {
+        dma1.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf1);
+        if (t + 3 * stride < num_tiles) dma1.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(src_of(t + 3 * stride));
+      }
+    }
+  } else {
+    const int lane = threadIdx.x;
+    auto write_out = [&](const char* lds_tile, const int t, const dma_t& dma) __attribute__((always_inline)) {
+      int ty, tx;
+      tile_coords(t, tiles_per_side, band, ty, tx);
+      vec4_t v[16];
+      const vec4_t* row = (const vec4_t*)(lds_tile + lane * kLdsRow);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) v[j] = row[j];
+      dma.start_async_dma();
+      if constexpr (QUAD) {
+        float* o = out + (size_t)(tx * kTile + (lane & 3)) * n + (size_t)ty * kTile + (lane & ~3);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) *(vec4_t*)(o + (size_t)(4 * j) * n) = quad_transpose(v[j], lane);
+      } else {
+        float* o = out + (size_t)(tx * kTile) * n + (size_t)ty * kTile + lane;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) o[(size_t)(4 * j + k) * n] = __uint_as_float(v[j][k]);
+        }
+      }
+    };
+    dma0.start_async_dma();
+    dma1.start_async_dma();
+    for (int t = blockIdx.x; t < num_tiles; t += 2 * stride) {
+      dma0.wait_for_dma_finish();
+      write_out(buf0, t, dma0);
+      if (t + stride < num_tiles) {
+        dma1.wait_for_dma_finish();
+        write_out(buf1, t + stride, dma1);
+      }
+    }
+  }
+}
+
 // Two DMA groups of one wavefront, one object and one LDS tile each
 // (src/perf/sequential/perf_sequential.cu:116-173).  A wavefront's loads complete in
 // issue order and s_waitcnt counts them in that order, so a wavefront that owns a
@@ -171,7 +239,9 @@ transpose_double_groups(const float* __restrict__ in, float* __restrict__ out, c
     tile_coords(t, tiles_per_side, band, ty, tx);
     return (const void*)(in + (size_t)ty * kTile * n + (size_t)tx * kTile);
   };
-  auto dma_loop = [&](dma_t& dma, char* buf, int t) {
+  // always inlined: called once per DMA group, and an object that is passed to a real function
+  // lives in scratch memory
+  auto dma_loop = [&](dma_t& dma, char* buf, int t) __attribute__((always_inline)) {
     if (t < num_tiles) dma.template start_xfer_async<true, LOAD_CACHE_ALL, SQ>(src_of(t));
     for (; t + 2 * stride < num_tiles; t += 2 * stride) {
       dma.template wait_xfer_finish<true, LOAD_CACHE_ALL, SQ>(buf);
@@ -277,8 +347,6 @@ transpose_single(const float* __restrict__ in, float* __restrict__ out, const in
 extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n, int variant, void* stream)
 {
   CUDADMA_REQUIRE(n >= 0 && (n % kTile) == 0, "n (%d) must be a multiple of %d", n, kTile);
-  int band = workloads::tuning("transpose_band", kDefaultBand);
-  while (band > 1 && (n / kTile) % band != 0) band /= 2;      // bands must tile the matrix
   CUDADMA_REQUIRE((long long)n * 4 <= 0x7fffffffLL, "row pitch must fit an int");
   if (variant < 0 || variant >= cudadma_num_variants(CUDADMA_WORKLOAD_STRIDED)) {
     cudadma_host::set_error("strided transpose has no variant %d", variant);
@@ -287,18 +355,32 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
   if (n == 0) return CUDADMA_OK;
   CUDADMA_REQUIRE(d_in != nullptr && d_out != nullptr && d_in != d_out, "NULL or aliased pointers");
   CUDADMA_REQUIRE(cudadma_host::aligned_to(d_in, 16) && cudadma_host::aligned_to(d_out, 16), "pointers must be 16-byte aligned");
-  const int tiles = (n / kTile) * (n / kTile);
+  const int tiles_per_side = n / kTile;
+  const int tiles = tiles_per_side * tiles_per_side;
+  // The kernels with one LDS tile (variants 1 and 4) run best with exactly one workgroup per compute unit, i.e. one
+  // 16 KB tile of loads in flight per compute unit, and with the tiles walked down the columns (the workgroups that
+  // run together then write whole output rows); the others with four workgroups and bands of 16 tile rows.
+  const bool one_tile = variant == 1 || variant == 4;
+  int band = workloads::tuning("transpose_band", one_tile ? tiles_per_side : kDefaultBand);
+  if (band > tiles_per_side) band = tiles_per_side;
+  while (band > 1 && tiles_per_side % band != 0) band /= 2;      // bands must tile the matrix
+  const int forced = workloads::tuning("transpose_workgroups", 0);
+  auto grid_for = [&](const int per_cu) {
+    return dim3((unsigned)(forced > 0 ? (forced < tiles ? forced : tiles) : workloads::persistent_grid(tiles, per_cu)));
+  };
   hipStream_t s = (hipStream_t)stream;
   const dim3 block(kDmaThreads + kComputeThreads);
   switch (variant) {
-    case 0: hipLaunchKernelGGL(transpose_manual_double<272>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
-    case 1: hipLaunchKernelGGL(transpose_single, dim3(workloads::persistent_grid(tiles, 8)), block, 0, s, d_in, d_out, n, tiles, band); break;
-    case 2: hipLaunchKernelGGL(transpose_manual_double<256>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
-    case 3: hipLaunchKernelGGL(transpose_double_groups<272>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
-    case 5: hipLaunchKernelGGL((transpose_double_groups<256, STORE_LDS_DIRECT_SWIZZLE>), dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
-    case 6: hipLaunchKernelGGL((transpose_double_groups<256, STORE_LDS_SWIZZLE>), dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
-    case 7: hipLaunchKernelGGL((transpose_manual_double<272, true>), dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, d_in, d_out, n, tiles, band); break;
-    default: hipLaunchKernelGGL(transpose_not_specialized, dim3(workloads::persistent_grid(tiles, 6)), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 0: hipLaunchKernelGGL(transpose_manual_double<272>, grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 1: hipLaunchKernelGGL(transpose_single, grid_for(1), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 2: hipLaunchKernelGGL(transpose_manual_double<256>, grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 3: hipLaunchKernelGGL(transpose_double_groups<272>, grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 5: hipLaunchKernelGGL((transpose_double_groups<256, STORE_LDS_DIRECT_SWIZZLE>), grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 6: hipLaunchKernelGGL((transpose_double_groups<256, STORE_LDS_SWIZZLE>), grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 7: hipLaunchKernelGGL((transpose_manual_double<272, true>), grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 8: hipLaunchKernelGGL(transpose_pairs<false>, grid_for(4), dim3(128), 0, s, d_in, d_out, n, tiles, band); break;
+    case 9: hipLaunchKernelGGL(transpose_pairs<true>, grid_for(4), dim3(128), 0, s, d_in, d_out, n, tiles, band); break;
+    default: hipLaunchKernelGGL(transpose_not_specialized, grid_for(1), block, 0, s, d_in, d_out, n, tiles, band); break;
   }
   CUDADMA_HIP_CHECK(hipGetLastError());
   return CUDADMA_OK;

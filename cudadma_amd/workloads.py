@@ -158,7 +158,7 @@ def perf_sequential(src, elmt_bytes, dma_wavefronts, buffering, loop_iters, work
 
 
 PROBE_MODES = ("read", "write", "write_nontemporal", "copy", "copy_nontemporal", "blocks_in_place", "blocks_swapped",
-               "blocks_permuted", "write_blocks_swapped")
+               "blocks_permuted", "write_blocks_swapped", "transpose_private")
 
 
 def probe_memory(mode, src, dst, workgroups):

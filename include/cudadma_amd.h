@@ -169,6 +169,7 @@ int cudadma_set_workgroups_per_cu(int value);
 /* Further integer knobs by name (0 restores the default); returns the previous
  * value or CUDADMA_EINVAL for an unknown name:
  *   "transpose_band"  tile rows per band of the config 2 tile order
+ *   "transpose_workgroups"  workgroups to launch for config 2, whatever the per-CU knob says
  *   "stencil_zchunk"     output planes one workgroup marches through in config 4
  *   "stencil_xcd_remap"  config 4 numbers its workgroups so that each XCD gets a contiguous part of the grid; 2 turns that off */
 int cudadma_set_tuning(const char* name, int value);
@@ -271,7 +272,9 @@ enum {
   CUDADMA_PROBE_BLOCKS_SWAPPED       = 6,  /* block (r, c) -> block (c, r), contents not transposed */
   CUDADMA_PROBE_BLOCKS_PERMUTED      = 7,  /* in place, blocks visited in a scattered order        */
   CUDADMA_PROBE_WRITE_BLOCKS_SWAPPED = 8,  /* mode 6 without its loads                             */
-  CUDADMA_PROBE_MODES                = 9
+  CUDADMA_PROBE_TRANSPOSE_PRIVATE    = 9,  /* d_dst = transpose(d_src): every wavefront transposes its blocks
+                                              through an LDS tile of its own, no DMA object, no handshake    */
+  CUDADMA_PROBE_MODES                = 10
 };
 long long cudadma_probe_memory(int mode, const void* d_src, void* d_dst, size_t bytes, int workgroups, void* stream);
 

@@ -358,6 +358,8 @@ def test_memory_probes_move_what_they_say(device, workgroups):
             continue
         if label.startswith("write"):
             assert bool((dst == 1.0).all())
+        elif label == "transpose_private":
+            assert torch.equal(dst.view(n, n).view(torch.int32), src.view(n, n).t().contiguous().view(torch.int32))
         elif label == "blocks_swapped":
             got = dst.view(n // 64, 64, n // 64, 64)
             assert torch.equal(got.view(torch.int32), want_blocks.permute(2, 1, 0, 3).contiguous().view(torch.int32))
