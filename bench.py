@@ -7,7 +7,7 @@ A step is one launch of the CudaDMAStrided tile-transpose kernel over the whole
 16384 x 16384 float32 matrix (benchmark config 2, the configuration the metric is
 quoted on); inputs are resident in HBM before the timed region.  The kernel is the
 warp-specialised one with one LDS tile (the next tile waits in the DMA wavefronts'
-registers), one workgroup per compute unit; the kernel with two LDS tiles and two
+registers), one workgroup per compute unit, streaming loads and stores; the kernel with two LDS tiles and two
 objects, which needs four workgroups per compute unit, is reported beside it.  The other three
 HBM-bound patterns (sequential copy, indirect gather, halo stencil), the scatter in
 the opposite direction and a plain copy kernel are timed the same way and reported
@@ -28,8 +28,8 @@ SETTLE_MS = 30.0                # wall time of untimed warm-up for the secondary
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # scaled by what the same counters read for the plain copy kernel (see profiles/).
-# profiles/bench_all_patterns_mi355x.md: FETCH_SIZE 524323 KiB x 1.99996 + WRITE_SIZE 1048576 KiB x 1.00000.
-MEASURED_TRAFFIC_BYTES = {"strided": 2147534527}
+# profiles/bench_all_patterns_mi355x.md: FETCH_SIZE 524328 KiB x 1.99996 + WRITE_SIZE 1048622 KiB x 1.00000.
+MEASURED_TRAFFIC_BYTES = {"strided": 2147590335}
 STRIDED_VARIANT = 1             # cudadma_strided_transpose variant timed as the headline
 
 
@@ -259,7 +259,7 @@ def main():
                    "workgroup": "128 DMA + 128 compute threads", "workgroups": "one per compute unit"},
         "roofline": {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(value / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES["strided"],
-                     "kernel": "transpose_single", "kernel_ms": round(strided_ms, 4),
+                     "kernel": "transpose_single<true, true>", "kernel_ms": round(strided_ms, 4),
                      "algorithmic_bytes_per_launch": strided_bytes},
         "patterns": patterns,
         "gemm": gemm,

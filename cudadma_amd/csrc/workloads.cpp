@@ -54,7 +54,8 @@ static const VariantInfo kSequential[] = {
 static const VariantInfo kStrided[] = {
   {"manual double buffer: one DMA group of 2 wavefronts, two CudaDMAStrided objects, padded LDS rows (272 B)"},
   {"single buffer: one object and one LDS tile, execute_dma (the next tile waits in the DMA wavefronts' registers); one "
-   "workgroup per compute unit, tiles walked down the columns: the fastest shape"},
+   "workgroup per compute unit, tiles walked down the columns, streaming loads (LOAD_CACHE_STREAMING), the consumer "
+   "transposes 4 x 4 words inside each quad and writes non-temporal dwordx4: the fastest shape"},
   {"manual double buffer, unpadded LDS rows (256 B): shows the bank-conflict cost"},
   {"double buffer: two DMA groups of 1 wavefront, one CudaDMAStrided object and one padded LDS tile each"},
   {"not warp-specialised: all four wavefronts move the tile and write it out, next tile requested two-phase"},

@@ -52,7 +52,8 @@ __device__ __forceinline__ vec4_t quad_transpose(const vec4_t a, const int lane)
   return vec4_t{odd ? q1 : b[0], odd ? b[1] : q0, odd ? q3 : b[2], odd ? b[3] : q2};
 }
 
-template<int LDS_ROW_BYTES, bool SWIZZLED = false, bool QUAD = false, typename Dma>
+// NT: the stores carry the non-temporal hint (the output is not read again by this kernel).
+template<int LDS_ROW_BYTES, bool SWIZZLED = false, bool QUAD = false, bool NT = false, typename Dma>
 __device__ __forceinline__ void write_tile_transposed(const char* lds_tile, float* __restrict__ out, const int n,
                                                       const int ty, const int tx, const Dma& dma)
 {
@@ -74,14 +75,20 @@ __device__ __forceinline__ void write_tile_transposed(const char* lds_tile, floa
     // then covers four output rows with 256 contiguous bytes each.
     float* o = out + (size_t)(tx * kTile + w * 32 + (lane & 3)) * n + (size_t)ty * kTile + (lane & ~3);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) *(vec4_t*)(o + (size_t)(4 * j) * n) = quad_transpose(v[j], lane);
+    for (int j = 0; j < 8; ++j) {
+      const vec4_t t = quad_transpose(v[j], lane);
+      if constexpr (NT) __builtin_nontemporal_store(t, (vec4_t*)(o + (size_t)(4 * j) * n));
+      else *(vec4_t*)(o + (size_t)(4 * j) * n) = t;
+    }
   } else {
     float* o = out + (size_t)(tx * kTile + w * 32) * n + (size_t)ty * kTile + lane;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
-        o[(size_t)(4 * j + k) * n] = __uint_as_float(v[j][k]);
+      for (int k = 0; k < 4; ++k) {
+        if constexpr (NT) __builtin_nontemporal_store(__uint_as_float(v[j][k]), o + (size_t)(4 * j + k) * n);
+        else o[(size_t)(4 * j + k) * n] = __uint_as_float(v[j][k]);
+      }
     }
   }
 }
@@ -317,9 +324,13 @@ transpose_not_specialized(const float* __restrict__ in, float* __restrict__ out,
   }
 }
 
+// STREAM: the loads and the stores carry the streaming / non-temporal hints.  At one workgroup per compute unit, where
+// a tile takes one trip to memory, they are worth 5 %; with more in flight they change nothing.
+template<bool STREAM, bool QUAD = false>
 __global__ void __launch_bounds__(kDmaThreads + kComputeThreads)
 transpose_single(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles, const int band)
 {
+  constexpr int kLoadQual = STREAM ? LOAD_CACHE_STREAMING : LOAD_CACHE_ALL;
   constexpr int kLdsRow = 272;
   __shared__ __attribute__((aligned(16))) char buf[kTile * kLdsRow];
   CudaDMAStrided<true, 16, kBytesPerThread, kRowBytes, kDmaThreads, kTile>
@@ -329,7 +340,7 @@ transpose_single(const float* __restrict__ in, float* __restrict__ out, const in
     for (int t = blockIdx.x; t < num_tiles; t += gridDim.x) {
       int ty, tx;
       tile_coords(t, tiles_per_side, band, ty, tx);
-      dma.template execute_dma<true, LOAD_CACHE_ALL, STORE_LDS>(in + (size_t)ty * kTile * n + (size_t)tx * kTile, buf);
+      dma.template execute_dma<true, kLoadQual, STORE_LDS>(in + (size_t)ty * kTile * n + (size_t)tx * kTile, buf);
     }
   } else {
     dma.start_async_dma();
@@ -337,7 +348,7 @@ transpose_single(const float* __restrict__ in, float* __restrict__ out, const in
       int ty, tx;
       tile_coords(t, tiles_per_side, band, ty, tx);
       dma.wait_for_dma_finish();
-      write_tile_transposed<kLdsRow>(buf, out, n, ty, tx, dma);
+      write_tile_transposed<kLdsRow, false, QUAD, STREAM>(buf, out, n, ty, tx, dma);
     }
   }
 }
@@ -372,7 +383,7 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
   const dim3 block(kDmaThreads + kComputeThreads);
   switch (variant) {
     case 0: hipLaunchKernelGGL(transpose_manual_double<272>, grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
-    case 1: hipLaunchKernelGGL(transpose_single, grid_for(1), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 1: hipLaunchKernelGGL((transpose_single<true, true>), grid_for(1), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 2: hipLaunchKernelGGL(transpose_manual_double<256>, grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 3: hipLaunchKernelGGL(transpose_double_groups<272>, grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 5: hipLaunchKernelGGL((transpose_double_groups<256, STORE_LDS_DIRECT_SWIZZLE>), grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
