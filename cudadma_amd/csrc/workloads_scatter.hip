@@ -64,7 +64,7 @@ scatter_manual(const float* __restrict__ records, const int* __restrict__ idx, f
         const long long tt = t + s * stride;
         if (tt < num_tiles) {
           g.wait_for_dma_start();                       // the producers have filled buf[s]
-          dma.template execute_dma<false, LOAD_CACHE_ALL, STORE_WRITE_BACK>(idx + tt * kRecsPerTile, buf[s], table);
+          dma.template execute_dma<false, LOAD_CACHE_ALL, STORE_CACHE_STREAMING>(idx + tt * kRecsPerTile, buf[s], table);
           g.finish_async_dma();                         // its contents are in registers or on their way
         }
       })
