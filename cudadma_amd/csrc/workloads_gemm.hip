@@ -231,7 +231,7 @@ gemm_bf16_ws(const unsigned short* __restrict__ a, const unsigned short* __restr
         for (int e = 0; e < 16; ++e) {
           const int row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
           const int col = j * 32 + (lane & 31);
-          cbase[(size_t)row * n + col] = acc[i][j][e];
+          __builtin_nontemporal_store(acc[i][j][e], &cbase[(size_t)row * n + col]);
         }
   }
 }
@@ -395,7 +395,7 @@ gemm_bf16_ws_direct(const unsigned short* __restrict__ a, const unsigned short* 
         for (int e = 0; e < 16; ++e) {
           const int row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
           const int col = j * 32 + (lane & 31);
-          cbase[(size_t)row * n + col] = acc[i][j][e];
+          __builtin_nontemporal_store(acc[i][j][e], &cbase[(size_t)row * n + col]);
         }
   }
 }
