@@ -28,8 +28,8 @@ SETTLE_MS = 30.0                # wall time of untimed warm-up for the secondary
 
 # HBM bytes per launch of the headline kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
 # scaled by what the same counters read for the plain copy kernel (see profiles/).
-# profiles/bench_all_patterns_mi355x.md: FETCH_SIZE 524328 KiB x 1.99996 + WRITE_SIZE 1048622 KiB x 1.00000.
-MEASURED_TRAFFIC_BYTES = {"strided": 2147590335}
+# profiles/bench_all_patterns_mi355x.md: FETCH_SIZE 524328 KiB x 1.99996 + WRITE_SIZE 1048598 KiB x 1.00000.
+MEASURED_TRAFFIC_BYTES = {"strided": 2147566719}
 STRIDED_VARIANT = 1             # cudadma_strided_transpose variant timed as the headline
 
 
