@@ -87,7 +87,7 @@ def test_plain_copy(device):
 
 # ------------------------------------------------------------------ config 2
 @pytest.mark.parametrize("variant", _variants(wl.STRIDED))
-@pytest.mark.parametrize("n", [1024, 2048])
+@pytest.mark.parametrize("n", [64, 192, 1024, 2048, 2112])       # 1, 3, 16, 32 and 33 tiles per side
 def test_strided_transpose_small(device, variant, n):
     host = ol.uniform(n * n, 1002).reshape(n, n)
     want = np.empty_like(host)
@@ -100,11 +100,31 @@ def test_strided_transpose_small(device, variant, n):
     assert np.array_equal(dst.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
-def test_strided_transpose_full_size(device):
+@pytest.mark.parametrize("variant", [1, 4, 0])
+@pytest.mark.parametrize("band,workgroups", [(0, 0), (1, 0), (3, 7), (5, 300), (256, 255), (1000, 100000)])
+def test_strided_transpose_under_every_tuning(device, variant, band, workgroups):
+    """The tile order and the number of workgroups are tuning knobs: the result does not depend on them."""
+    n = 1344                                                     # 21 tiles per side
+    host = ol.uniform(n * n, 77).reshape(n, n)
+    src = torch.from_numpy(host).to(device)
+    dst = torch.full_like(src, float("nan"))
+    try:
+        wl.set_tuning("transpose_band", band)
+        wl.set_tuning("transpose_workgroups", workgroups)
+        wl.strided_transpose(src, dst, variant)
+        torch.cuda.synchronize()
+    finally:
+        wl.set_tuning("transpose_band", 0)
+        wl.set_tuning("transpose_workgroups", 0)
+    assert np.array_equal(dst.cpu().numpy().view(np.uint32), np.ascontiguousarray(host.T).view(np.uint32))
+
+
+@pytest.mark.parametrize("variant", [1, 0])                       # the reported kernel and the one with two LDS tiles
+def test_strided_transpose_full_size(device, variant):
     n = 16384
     src = wl.fill_uniform(torch.empty(n * n, dtype=torch.float32, device=device), 1002).view(n, n)
     dst = torch.empty_like(src)
-    wl.strided_transpose(src, dst, 0)
+    wl.strided_transpose(src, dst, variant)
     torch.cuda.synchronize()
     # rows of the oracle's statement on a sample of the output, then transpose twice = identity
     host_rows = ol.uniform(n * n, 1002).reshape(n, n)
@@ -112,7 +132,7 @@ def test_strided_transpose_full_size(device):
         assert np.array_equal(dst[c].cpu().numpy(), host_rows[:, c])
     del host_rows
     back = torch.empty_like(src)
-    wl.strided_transpose(dst, back, 0)
+    wl.strided_transpose(dst, back, variant)
     torch.cuda.synchronize()
     assert torch.equal(back.view(torch.int32), src.view(torch.int32))
 
