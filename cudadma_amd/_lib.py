@@ -131,6 +131,7 @@ _WORKLOAD_SIGNATURES = {
     "cudadma_gemm_bf16": [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cudadma_selftest_bounded_wait": [_vp, _vp],
     "cudadma_selftest_split_wait": [_vp, _ci, _vp],
+    "cudadma_selftest_all_ids": [_vp, _ci, _vp],
     "cudadma_v1_num_cases": [],
     "cudadma_v1_run_case": [_ci, _vp, _vp, _vp, _vp],
     "cudadma_example_num_variants": [_ci],

@@ -120,6 +120,11 @@ int cudadma_selftest_bounded_wait(int* d_flags, void* stream);
  * which the peek already found the buffer full. */
 int cudadma_selftest_split_wait(int* d_out, int phases, void* stream);
 
+/* All sixteen dmaIDs at once: sixteen sync-only objects guard sixteen LDS slots, two DMA wavefronts
+ * fill slot (phase mod 16) with the phase's token and may run sixteen phases ahead, one compute
+ * wavefront checks every token.  d_out (one zeroed int) receives the number of wrong tokens. */
+int cudadma_selftest_all_ids(int* d_out, int phases, void* stream);
+
 /* ------------------------------------------------------------------------
  * Host-side planner.  cudadma_diagnose prints what the static diagnose()
  * members of the objects print (include/cudaDMAv2.h:1402-1458, :3208-3493,

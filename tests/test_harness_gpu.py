@@ -207,3 +207,14 @@ def test_split_wait_sees_every_phase(device):
     wrong, early = out.tolist()
     assert wrong == 0
     assert 0 < early < phases, f"both branches of the split wait should have run ({early} early of {phases})"
+
+
+@pytest.mark.parametrize("phases", [1, 16, 17, 1000])
+def test_all_sixteen_ids_keep_their_own_counts(device, phases):
+    """Sixteen sync-only objects, one per dmaID, used round-robin with the DMA side up to sixteen phases
+    ahead: no id may see another id's signals."""
+    import ctypes
+    out = torch.zeros(1, dtype=torch.int32, device=device)
+    cd._lib.check(cd.lib().cudadma_selftest_all_ids(ctypes.c_void_p(out.data_ptr()), phases, None))
+    torch.cuda.synchronize()
+    assert out.item() == 0
