@@ -400,6 +400,161 @@ gemm_bf16_ws_direct(const unsigned short* __restrict__ a, const unsigned short* 
   }
 }
 
+// ---- 256 x 256 tile, K step 32, four unpadded swizzled stages filled by global_load_lds_dwordx4 ----
+// Eight compute wavefronts (2 x 4, 128 x 64 each, two per SIMD) and four DMA wavefronts.  A stage is
+// 32 KB (A: 256 rows x 64 B, B: 32 rows x 512 B); each DMA wavefront keeps three transfers in flight.
+template<typename T>
+struct Four4 {
+  T a0, a1, a2, a3;
+  template<int I> __device__ __forceinline__ T& get() { if constexpr (I == 0) return a0; else if constexpr (I == 1) return a1; else if constexpr (I == 2) return a2; else return a3; }
+};
+
+constexpr int kDirect4DmaThreads = 128;    // DMA threads per operand
+constexpr int kDirect4Ahead = 3;           // transfers in flight per DMA wavefront (2: 3 % slower; 4 stages allow no more)
+__global__ void __launch_bounds__(512 + 2 * kDirect4DmaThreads)
+gemm_bf16_ws_direct4(const unsigned short* __restrict__ a, const unsigned short* __restrict__ b, float* __restrict__ c,
+                     const int m, const int n, const int k)
+{
+  constexpr int WI = 4, WJ = 2, WN = 4, kStages = 4, kBK4 = 32, kCompute = 512, kDmaWave = kDirect4DmaThreads;
+  constexpr int kBM = 256, kBN = 256;
+  constexpr int kARow = kBK4 * 2, kBRow = kBN * 2;                 // 64 B and 512 B, unpadded
+  constexpr int kAStage = kBM * kARow, kBStage = kBK4 * kBRow;     // 16 KB and 16 KB
+  typedef CudaDMAStrided<false, 16, 16, kARow, kDmaWave, kBM> dma_a_t;
+  typedef CudaDMAStrided<false, 16, 16, kBRow, kDmaWave, kBK4> dma_b_t;
+  __shared__ __attribute__((aligned(1024))) char lds_a[kStages][kAStage];
+  __shared__ __attribute__((aligned(1024))) char lds_b[kStages][kBStage];
+  dma_a_t dma_a(k * 2, kARow, kCompute);
+  dma_b_t dma_b(n * 2, kBRow, kCompute + kDmaWave);
+  Four4<cudaDMACustom> stage{cudaDMACustom(0, 2 * kDmaWave, kCompute, kCompute), cudaDMACustom(1, 2 * kDmaWave, kCompute, kCompute),
+                             cudaDMACustom(2, 2 * kDmaWave, kCompute, kCompute), cudaDMACustom(3, 2 * kDmaWave, kCompute, kCompute)};
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, m / kBM, n / kBN, tile_m, tile_n);
+  const int ksteps = k / kBK4;            // a multiple of four: k is a multiple of 128
+
+  // One DMA wavefront: tile t lands in stage t % 4; tiles t+1 .. t+3 are in flight while the compute
+  // wavefronts work on tile t.
+  auto feed = [&](auto& dma, char* lds, auto stage_bytes, const unsigned short* src, const size_t step)
+      __attribute__((always_inline)) {
+    constexpr int kStageBytes = decltype(stage_bytes)::value;
+    constexpr int kLoads = std::remove_reference<decltype(dma)>::type::loads_per_thread();
+    constexpr int kAhead = kDirect4Ahead;       // transfers in flight per DMA wavefront
+    stage.a0.wait_for_dma_start_direct();
+    dma.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src, lds);
+    if constexpr (kAhead > 1) {
+      stage.a1.wait_for_dma_start_direct();
+      dma.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src + step, lds + kStageBytes);
+    }
+    if constexpr (kAhead > 2) {
+      stage.a2.wait_for_dma_start_direct();
+      dma.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src + 2 * step, lds + 2 * kStageBytes);
+    }
+    auto land = [&](auto cur, const int t) __attribute__((always_inline)) {
+      constexpr int kCur = decltype(cur)::value, kNext = (kCur + kAhead) % kStages;
+      // the younger transfers stay in flight (fewer at the end)
+      if (t + kAhead - 1 < ksteps) hipdma::wait_direct_loads<(kAhead - 1) * kLoads>();
+      else if (kAhead > 2 && t + 1 < ksteps) hipdma::wait_direct_loads<kLoads>();
+      else hipdma::wait_direct_loads<0>();
+      stage.template get<kCur>().finish_async_dma_direct();
+      if (t + kAhead < ksteps) {
+        stage.template get<kNext>().wait_for_dma_start_direct();
+        dma.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src + (size_t)(t + kAhead) * step, lds + kNext * kStageBytes);
+      }
+    };
+    typedef std::integral_constant<int, 0> s0;
+    typedef std::integral_constant<int, 1> s1;
+    typedef std::integral_constant<int, 2> s2;
+    typedef std::integral_constant<int, 3> s3;
+    for (int t = 0; t < ksteps; t += 4) {
+      land(s0(), t);
+      land(s1(), t + 1);
+      land(s2(), t + 2);
+      land(s3(), t + 3);
+    }
+  };
+  if (dma_a.owns_this_thread()) {
+    feed(dma_a, &lds_a[0][0], std::integral_constant<int, kAStage>(), a + (size_t)tile_m * kBM * k, (size_t)kBK4);
+  } else if (dma_b.owns_this_thread()) {
+    feed(dma_b, &lds_b[0][0], std::integral_constant<int, kBStage>(), b + (size_t)tile_n * kBN, (size_t)kBK4 * n);
+  } else {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = (wave / WN) * 32 * WI, wn = (wave % WN) * 32 * WJ;
+    f32x16_t acc[WI][WJ];
+#pragma unroll
+    for (int i = 0; i < WI; ++i)
+#pragma unroll
+      for (int j = 0; j < WJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+    stage.a0.start_async_dma();
+    stage.a1.start_async_dma();
+    stage.a2.start_async_dma();
+    stage.a3.start_async_dma();
+    // A fragment of slice ks: row wm + 32*i + lane%32, chunk 2*ks + lane/32 of the 4 chunks of the row, found at
+    // chunk position (2*ks + lane/32) ^ key(row); the key only depends on lane%32 (wm and 32*i are multiples of 32).
+    int a_lane[kBK4 / 16];
+    {
+      const int row = wm + (lane & 31);
+#pragma unroll
+      for (int ks = 0; ks < kBK4 / 16; ++ks)
+        a_lane[ks] = row * kARow + hipdma::swizzled_chunk(row, 2 * ks + (lane >> 5), kARow / 16) * 16;
+    }
+    // B fragment through the transposing read; adding 16 rows (the next slice) does not change a row's key.
+    int b_lo[WJ], b_hi[WJ];
+    {
+      const int j16 = lane & 15;
+      const int row = (lane >> 5) * 8 + (j16 >> 2);
+#pragma unroll
+      for (int j = 0; j < WJ; ++j) {
+        const int col_bytes = (wn + j * 32 + ((lane >> 4) & 1) * 16 + (j16 & 3) * 4) * 2;
+        b_lo[j] = row * kBRow + hipdma::swizzled_chunk(row, col_bytes >> 4, kBRow / 16) * 16 + (col_bytes & 15);
+        b_hi[j] = (row + 4) * kBRow + hipdma::swizzled_chunk(row + 4, col_bytes >> 4, kBRow / 16) * 16 + (col_bytes & 15);
+      }
+    }
+    auto k_stage = [&](const cudaDMACustom& cur, const int s) __attribute__((always_inline)) {
+      const char* sa = lds_a[s]; const char* sb = lds_b[s];
+      cur.wait_for_dma_finish();
+#pragma unroll
+      for (int ks = 0; ks < kBK4 / 16; ++ks) {
+        bf16x8_t fa[WI], fb[WJ];
+#pragma unroll
+        for (int i = 0; i < WI; ++i) fa[i] = *(const bf16x8_t*)(sa + i * 32 * kARow + a_lane[ks]);
+#pragma unroll
+        for (int j = 0; j < WJ; ++j) {
+          const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+              (__attribute__((address_space(3))) bf16x4_t*)(sb + ks * 16 * kBRow + b_lo[j]));
+          const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+              (__attribute__((address_space(3))) bf16x4_t*)(sb + ks * 16 * kBRow + b_hi[j]));
+          fb[j] = bf16x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+#pragma unroll
+        for (int i = 0; i < WI; ++i)
+#pragma unroll
+          for (int j = 0; j < WJ; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+      cur.start_async_dma();
+    };
+    for (int kt = 0; kt < ksteps; kt += 4) {
+      k_stage(stage.a0, 0);
+      k_stage(stage.a1, 1);
+      k_stage(stage.a2, 2);
+      k_stage(stage.a3, 3);
+    }
+    float* cbase = c + (size_t)(tile_m * kBM + wm) * n + (size_t)tile_n * kBN + wn;
+#pragma unroll
+    for (int i = 0; i < WI; ++i)
+#pragma unroll
+      for (int j = 0; j < WJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
+          const int col = j * 32 + (lane & 31);
+          __builtin_nontemporal_store(acc[i][j][e], &cbase[(size_t)row * n + col]);
+        }
+  }
+}
+
 template<int WI, int WJ, int WM = 2, int WN = 2>
 int launch_gemm(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k, hipStream_t stream)
 {
@@ -435,7 +590,7 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
     // the largest tile that divides the problem and still gives every compute unit a tile; the small one otherwise
     const long long cus = workloads::device_cus();
     const bool m256 = (m % 256) == 0, n256 = (n % 256) == 0;
-    if (m256 && n256 && (long long)(m / 256) * (n / 256) >= cus) variant = 5;
+    if (m256 && n256 && (long long)(m / 256) * (n / 256) >= cus) variant = 6;
     else if (m256 && (long long)(m / 256) * (n / 128) >= cus) variant = 3;
     else if (n256 && (long long)(m / 128) * (n / 256) >= cus) variant = 2;
     else variant = 1;
@@ -445,6 +600,14 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
     case 2: return launch_gemm<2, 4>(d_a, d_b, d_c, m, n, k, s);
     case 3: return launch_gemm<4, 2>(d_a, d_b, d_c, m, n, k, s);
     case 5: return launch_gemm<4, 2, 2, 4>(d_a, d_b, d_c, m, n, k, s);
+    case 6: {
+      CUDADMA_REQUIRE((m % 256) == 0 && (n % 256) == 0, "this variant needs m and n multiples of 256 (got %d x %d)", m, n);
+      const long long grid = (long long)(m / 256) * (n / 256);
+      CUDADMA_REQUIRE(grid <= 0x7fffffffLL, "grid too large");
+      hipLaunchKernelGGL(gemm_bf16_ws_direct4, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
+      CUDADMA_HIP_CHECK(hipGetLastError());
+      return CUDADMA_OK;
+    }
     default: {
       CUDADMA_REQUIRE((m % 256) == 0, "this variant needs m a multiple of 256 (got %d)", m);
       const long long grid = (long long)(m / 256) * (n / 128);

@@ -238,7 +238,8 @@ int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz
  * problem and leaves no compute unit without a tile; 1: 128 x 128; 2: 128 x 256 (n a multiple of
  * 256); 3: 256 x 128 (m a multiple of 256); 4: 256 x 128 with the tiles brought in by
  * global_load_lds into swizzled LDS rows; 5: 256 x 256 with eight compute wavefronts (m and n
- * multiples of 256). */
+ * multiples of 256); 6: the same tile with K steps of 32 brought into four swizzled LDS stages by
+ * global_load_lds. */
 int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k,
                       int variant, void* stream);
 
