@@ -232,9 +232,10 @@ def main():
     flops = 2.0 * dim ** 3
     gemm = {"TFLOP/s": round(flops / ms / 1e9, 1), "frac_of_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4),
             "ms": round(ms, 4), "flop": flops,
-            "workload": "C = A*B, bf16 4096^3, fp32 accumulate, 256x256 workgroup tile: 256x32 / 32x256 operand tiles "
-                        "brought into four swizzled LDS stages by CudaDMAStrided::issue_direct (global_load_lds) in "
-                        "four DMA wavefronts, v_mfma_f32_32x32x16_bf16 on 128x64 tiles in eight compute wavefronts"}
+            "workload": "C = A*B, bf16 4096^3, fp32 accumulate, 256x256 workgroup tile: 256x64 A tiles (two buffers) and "
+                        "32x256 B tiles (four stages) brought into swizzled LDS by CudaDMAStrided::issue_direct "
+                        "(global_load_lds) in four DMA wavefronts, v_mfma_f32_32x32x16_bf16 on 128x64 tiles in eight "
+                        "compute wavefronts"}
     log(f"gemm         {ms:9.4f} ms  {gemm['TFLOP/s']:8.1f} TFLOP/s  {100 * gemm['frac_of_mfma_peak']:5.1f}% of 2.5 PFLOP/s")
     del ga, gb, gc
 

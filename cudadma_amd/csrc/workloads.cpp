@@ -86,7 +86,7 @@ static const VariantInfo kHalo[] = {
 };
 
 static const VariantInfo kGemm[] = {
-  {"the largest workgroup tile that divides the problem and gives every compute unit a tile: variant 6, 3 or 2, else "
+  {"the largest workgroup tile that divides the problem and gives every compute unit a tile: variant 7, 3 or 2, else "
    "variant 1"},
   {"warp-specialised: two DMA wavefronts per operand with two CudaDMAStrided objects each (two LDS stages, tile two K "
    "steps ahead in flight), four compute wavefronts with v_mfma_f32_32x32x16_bf16, B fragments through "
@@ -99,6 +99,8 @@ static const VariantInfo kGemm[] = {
    "four DMA wavefronts; twelve wavefronts leave 168 registers each"},
   {"256 x 256 workgroup tile, K step 32, four unpadded swizzled LDS stages filled by global_load_lds_dwordx4 "
    "(three transfers in flight per DMA wavefront), eight compute wavefronts"},
+  {"variant 6 with A transfers of two K steps (256 rows x 128 B, whole cache lines) into two 32 KB buffers with guards "
+   "of their own; B keeps four stages of one K step"},
 };
 
 static const VariantInfo kScatter[] = {

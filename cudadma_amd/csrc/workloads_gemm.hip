@@ -555,6 +555,172 @@ gemm_bf16_ws_direct4(const unsigned short* __restrict__ a, const unsigned short*
   }
 }
 
+// ---- the same kernel with A rows of 128 B: an A transfer covers two K steps ----
+// A K step of 32 takes 64 B of every A row, half a cache line: the L1 fetches each line of the A
+// panel twice, a step apart, and the compute wavefronts wait for the DMA wavefronts (measured with
+// s_memtime stamps: 900 of 2350 cycles per step).  Here an A transfer brings 256 rows x 128 B
+// (two K steps, whole lines) into one of two 32 KB buffers with its own guard; B keeps the four
+// 16 KB stages of one K step each.  The compute wavefronts wait for a B stage every step and for
+// an A buffer every other step.
+__global__ void __launch_bounds__(512 + 2 * kDirect4DmaThreads)
+gemm_bf16_ws_direct4_a64(const unsigned short* __restrict__ a, const unsigned short* __restrict__ b, float* __restrict__ c,
+                         const int m, const int n, const int k)
+{
+  constexpr int WI = 4, WJ = 2, WN = 4, kBStages = 4, kBK4 = 32, kCompute = 512, kDmaWave = kDirect4DmaThreads;
+  constexpr int kBM = 256, kBN = 256;
+  constexpr int kARow = 4 * kBK4, kBRow = kBN * 2;                 // 128 B (two K steps) and 512 B, unpadded
+  constexpr int kABuf = kBM * kARow, kBStage = kBK4 * kBRow;       // 32 KB and 16 KB
+  typedef CudaDMAStrided<false, 16, 16, kARow, kDmaWave, kBM> dma_a_t;
+  typedef CudaDMAStrided<false, 16, 16, kBRow, kDmaWave, kBK4> dma_b_t;
+  __shared__ __attribute__((aligned(1024))) char lds_a[2][kABuf];
+  __shared__ __attribute__((aligned(1024))) char lds_b[kBStages][kBStage];
+  dma_a_t dma_a(k * 2, kARow, kCompute);
+  dma_b_t dma_b(n * 2, kBRow, kCompute + kDmaWave);
+  Four4<cudaDMACustom> gb{cudaDMACustom(0, kDmaWave, kCompute, kCompute + kDmaWave), cudaDMACustom(1, kDmaWave, kCompute, kCompute + kDmaWave),
+                          cudaDMACustom(2, kDmaWave, kCompute, kCompute + kDmaWave), cudaDMACustom(3, kDmaWave, kCompute, kCompute + kDmaWave)};
+  cudaDMACustom ga0(4, kDmaWave, kCompute, kCompute);
+  cudaDMACustom ga1(5, kDmaWave, kCompute, kCompute);
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, m / kBM, n / kBN, tile_m, tile_n);
+  const int ksteps = k / kBK4;            // a multiple of four: k is a multiple of 128
+
+  if (dma_a.owns_this_thread()) {
+    // Transfer p (K steps 2p and 2p+1) lands in buffer p % 2; transfer p+1 is requested as soon as
+    // p has landed (its buffer was released when the compute wavefronts left transfer p-1).
+    const unsigned short* src = a + (size_t)tile_m * kBM * k;
+    const int transfers = ksteps / 2;     // even
+    ga0.wait_for_dma_start_direct();
+    dma_a.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src, lds_a[0]);
+    for (int p = 0; p < transfers; p += 2) {
+      hipdma::wait_direct_loads<0>();
+      ga0.finish_async_dma_direct();
+      ga1.wait_for_dma_start_direct();
+      dma_a.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src + (size_t)(p + 1) * (2 * kBK4), lds_a[1]);
+      hipdma::wait_direct_loads<0>();
+      ga1.finish_async_dma_direct();
+      if (p + 2 < transfers) {
+        ga0.wait_for_dma_start_direct();
+        dma_a.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src + (size_t)(p + 2) * (2 * kBK4), lds_a[0]);
+      }
+    }
+  } else if (dma_b.owns_this_thread()) {
+    // Tile t lands in stage t % 4; tiles t+1 .. t+3 are in flight while the compute wavefronts work on tile t.
+    const unsigned short* src = b + (size_t)tile_n * kBN;
+    const size_t step = (size_t)kBK4 * n;
+    constexpr int kLoads = dma_b_t::loads_per_thread();
+    constexpr int kAhead = kDirect4Ahead;
+    gb.a0.wait_for_dma_start_direct();
+    dma_b.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src, lds_b[0]);
+    gb.a1.wait_for_dma_start_direct();
+    dma_b.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src + step, lds_b[1]);
+    gb.a2.wait_for_dma_start_direct();
+    dma_b.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src + 2 * step, lds_b[2]);
+    auto land = [&](auto cur, const int t) __attribute__((always_inline)) {
+      constexpr int kCur = decltype(cur)::value, kNext = (kCur + kAhead) % kBStages;
+      if (t + kAhead - 1 < ksteps) hipdma::wait_direct_loads<(kAhead - 1) * kLoads>();
+      else if (t + 1 < ksteps) hipdma::wait_direct_loads<kLoads>();
+      else hipdma::wait_direct_loads<0>();
+      gb.template get<kCur>().finish_async_dma_direct();
+      if (t + kAhead < ksteps) {
+        gb.template get<kNext>().wait_for_dma_start_direct();
+        dma_b.template issue_direct<STORE_LDS_DIRECT_SWIZZLE>(src + (size_t)(t + kAhead) * step, lds_b[kNext]);
+      }
+    };
+    for (int t = 0; t < ksteps; t += 4) {
+      land(std::integral_constant<int, 0>(), t);
+      land(std::integral_constant<int, 1>(), t + 1);
+      land(std::integral_constant<int, 2>(), t + 2);
+      land(std::integral_constant<int, 3>(), t + 3);
+    }
+  } else {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wm = (wave / WN) * 32 * WI, wn = (wave % WN) * 32 * WJ;
+    f32x16_t acc[WI][WJ];
+#pragma unroll
+    for (int i = 0; i < WI; ++i)
+#pragma unroll
+      for (int j = 0; j < WJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+    gb.a0.start_async_dma();
+    gb.a1.start_async_dma();
+    gb.a2.start_async_dma();
+    gb.a3.start_async_dma();
+    ga0.start_async_dma();
+    ga1.start_async_dma();
+    // A fragment of slice ks (0..3 inside a buffer): row wm + 32*i + lane%32, chunk 2*ks + lane/32 of the 8 chunks
+    // of the row, found at chunk position (2*ks + lane/32) ^ key(row); the key only depends on lane%32.
+    int a_lane[4];
+    {
+      const int row = wm + (lane & 31);
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+        a_lane[ks] = row * kARow + hipdma::swizzled_chunk(row, 2 * ks + (lane >> 5), kARow / 16) * 16;
+    }
+    // B fragment through the transposing read; adding 16 rows (the next slice) does not change a row's key.
+    int b_lo[WJ], b_hi[WJ];
+    {
+      const int j16 = lane & 15;
+      const int row = (lane >> 5) * 8 + (j16 >> 2);
+#pragma unroll
+      for (int j = 0; j < WJ; ++j) {
+        const int col_bytes = (wn + j * 32 + ((lane >> 4) & 1) * 16 + (j16 & 3) * 4) * 2;
+        b_lo[j] = row * kBRow + hipdma::swizzled_chunk(row, col_bytes >> 4, kBRow / 16) * 16 + (col_bytes & 15);
+        b_hi[j] = (row + 4) * kBRow + hipdma::swizzled_chunk(row + 4, col_bytes >> 4, kBRow / 16) * 16 + (col_bytes & 15);
+      }
+    }
+    // One K step: B stage s, slices 2*half and 2*half+1 of A buffer `abuf`.
+    auto k_step = [&](const cudaDMACustom& gbs, const int s, const cudaDMACustom& gas, const int abuf, auto half)
+        __attribute__((always_inline)) {
+      constexpr int kHalf = decltype(half)::value;
+      const char* sa = lds_a[abuf]; const char* sb = lds_b[s];
+      if constexpr (kHalf == 0) gas.wait_for_dma_finish();
+      gbs.wait_for_dma_finish();
+#pragma unroll
+      for (int ks = 0; ks < kBK4 / 16; ++ks) {
+        bf16x8_t fa[WI], fb[WJ];
+#pragma unroll
+        for (int i = 0; i < WI; ++i) fa[i] = *(const bf16x8_t*)(sa + i * 32 * kARow + a_lane[2 * kHalf + ks]);
+#pragma unroll
+        for (int j = 0; j < WJ; ++j) {
+          const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+              (__attribute__((address_space(3))) bf16x4_t*)(sb + ks * 16 * kBRow + b_lo[j]));
+          const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+              (__attribute__((address_space(3))) bf16x4_t*)(sb + ks * 16 * kBRow + b_hi[j]));
+          fb[j] = bf16x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+#pragma unroll
+        for (int i = 0; i < WI; ++i)
+#pragma unroll
+          for (int j = 0; j < WJ; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+      gbs.start_async_dma();
+      if constexpr (kHalf == 1) gas.start_async_dma();
+    };
+    typedef std::integral_constant<int, 0> h0;
+    typedef std::integral_constant<int, 1> h1;
+    for (int kt = 0; kt < ksteps; kt += 4) {
+      k_step(gb.a0, 0, ga0, 0, h0());
+      k_step(gb.a1, 1, ga0, 0, h1());
+      k_step(gb.a2, 2, ga1, 1, h0());
+      k_step(gb.a3, 3, ga1, 1, h1());
+    }
+    float* cbase = c + (size_t)(tile_m * kBM + wm) * n + (size_t)tile_n * kBN + wn;
+#pragma unroll
+    for (int i = 0; i < WI; ++i)
+#pragma unroll
+      for (int j = 0; j < WJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
+          const int col = j * 32 + (lane & 31);
+          __builtin_nontemporal_store(acc[i][j][e], &cbase[(size_t)row * n + col]);
+        }
+  }
+}
+
 template<int WI, int WJ, int WM = 2, int WN = 2>
 int launch_gemm(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k, hipStream_t stream)
 {
@@ -590,7 +756,7 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
     // the largest tile that divides the problem and still gives every compute unit a tile; the small one otherwise
     const long long cus = workloads::device_cus();
     const bool m256 = (m % 256) == 0, n256 = (n % 256) == 0;
-    if (m256 && n256 && (long long)(m / 256) * (n / 256) >= cus) variant = 6;
+    if (m256 && n256 && (long long)(m / 256) * (n / 256) >= cus) variant = 7;
     else if (m256 && (long long)(m / 256) * (n / 128) >= cus) variant = 3;
     else if (n256 && (long long)(m / 128) * (n / 256) >= cus) variant = 2;
     else variant = 1;
@@ -600,11 +766,12 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
     case 2: return launch_gemm<2, 4>(d_a, d_b, d_c, m, n, k, s);
     case 3: return launch_gemm<4, 2>(d_a, d_b, d_c, m, n, k, s);
     case 5: return launch_gemm<4, 2, 2, 4>(d_a, d_b, d_c, m, n, k, s);
-    case 6: {
+    case 6: case 7: {
       CUDADMA_REQUIRE((m % 256) == 0 && (n % 256) == 0, "this variant needs m and n multiples of 256 (got %d x %d)", m, n);
       const long long grid = (long long)(m / 256) * (n / 256);
       CUDADMA_REQUIRE(grid <= 0x7fffffffLL, "grid too large");
-      hipLaunchKernelGGL(gemm_bf16_ws_direct4, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
+      if (variant == 6) hipLaunchKernelGGL(gemm_bf16_ws_direct4, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
+      else hipLaunchKernelGGL(gemm_bf16_ws_direct4_a64, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
       CUDADMA_HIP_CHECK(hipGetLastError());
       return CUDADMA_OK;
     }

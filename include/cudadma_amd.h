@@ -239,7 +239,8 @@ int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz
  * 256); 3: 256 x 128 (m a multiple of 256); 4: 256 x 128 with the tiles brought in by
  * global_load_lds into swizzled LDS rows; 5: 256 x 256 with eight compute wavefronts (m and n
  * multiples of 256); 6: the same tile with K steps of 32 brought into four swizzled LDS stages by
- * global_load_lds. */
+ * global_load_lds; 7: variant 6 with A transfers of two K steps (rows of 128 B, whole cache
+ * lines) into two buffers of their own. */
 int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k,
                       int variant, void* stream);
 

@@ -128,27 +128,45 @@ __device__ __forceinline__ void acquire_lds()
 #endif
 }
 
+// The lowest active lane of the calling wavefront adds the number of active lanes to `word`.
+// The election is scalar work (s_ff1 on exec, exec narrowed to that lane around the ds_add, one
+// v_mov for the count): a vector ALU instruction of a wavefront that shares its SIMD with
+// wavefronts issuing matrix instructions back to back waits for a gap between those, so every
+// one saved in a hand-off shortens it by tens of cycles (measured in the GEMM workload: a DMA
+// wavefront with three vector ALU instructions per load issued a load every 175 cycles).
+__device__ __forceinline__ void add_active_lanes(lds_word_t* word)
+{
+  const unsigned addr = (unsigned)(size_t)word;
+  const unsigned count = (unsigned)__builtin_popcountll(__builtin_amdgcn_ballot_w64(true));
+  unsigned long long saved;
+  unsigned first;
+  asm volatile("s_mov_b64 %0, exec\n\t"
+               "s_ff1_i32_b64 %1, exec\n\t"
+               "s_lshl_b64 exec, 1, %1\n\t"
+               "ds_add_u32 %2, %3\n\t"
+               "s_mov_b64 exec, %0"
+               : "=&s"(saved), "=&s"(first) : "v"(addr), "v"(count) : "memory", "scc");     // s_lshl_b64 writes SCC
+}
+
 // All active lanes of the calling wavefront arrive at `word`.
 __device__ __forceinline__ void signal_word(lds_word_t* word)
 {
   release_lds();
-  const unsigned long long active = __builtin_amdgcn_ballot_w64(true);
-  const unsigned lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-  if (lane == (unsigned)__builtin_ctzll(active))
-    __hip_atomic_fetch_add(word, (unsigned)__builtin_popcountll(active),
-                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  add_active_lanes(word);
 }
 
-// Block until `word` has reached `target` (wrap-around safe).
+// Block until `word` has reached `target` (wrap-around safe).  Every lane reads the same word with
+// the same instruction, so the comparison and the loop are scalar.
 __device__ __forceinline__ void wait_word(lds_word_t* word, unsigned target)
 {
+  const unsigned want = __builtin_amdgcn_readfirstlane(target);
 #if HIPDMA_SPIN_LIMIT > 0
   int polls = 0;
-  while ((int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - target) < 0 &&
+  while ((int)(__builtin_amdgcn_readfirstlane(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) - want) < 0 &&
          ++polls < HIPDMA_SPIN_LIMIT)
     __builtin_amdgcn_s_sleep(HIPDMA_SPIN_SLEEP);
 #else
-  while ((int)(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - target) < 0)
+  while ((int)(__builtin_amdgcn_readfirstlane(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) - want) < 0)
     __builtin_amdgcn_s_sleep(HIPDMA_SPIN_SLEEP);
 #endif
   acquire_lds();
@@ -163,18 +181,13 @@ __device__ __forceinline__ void wait_word(lds_word_t* word, unsigned target)
 // after the wait for that buffer has returned (a control dependence the hardware honours).
 __device__ __forceinline__ void signal_word_unfenced(lds_word_t* word)
 {
-  const unsigned long long active = __builtin_amdgcn_ballot_w64(true);
-  const unsigned lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-  if (lane == (unsigned)__builtin_ctzll(active)) {
-    const unsigned addr = (unsigned)(size_t)word;
-    const unsigned count = (unsigned)__builtin_popcountll(active);
-    asm volatile("ds_add_u32 %0, %1" : : "v"(addr), "v"(count) : "memory");
-  }
+  add_active_lanes(word);
 }
 
 __device__ __forceinline__ void wait_word_unfenced(lds_word_t* word, unsigned target)
 {
   const unsigned addr = (unsigned)(size_t)word;
+  const unsigned want = __builtin_amdgcn_readfirstlane(target);
   unsigned seen;
 #if HIPDMA_SPIN_LIMIT > 0
   for (int polls = 0; polls < HIPDMA_SPIN_LIMIT; ++polls) {
@@ -182,7 +195,7 @@ __device__ __forceinline__ void wait_word_unfenced(lds_word_t* word, unsigned ta
   for (;;) {
 #endif
     asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : "v"(addr) : "memory");
-    if ((int)(seen - target) >= 0) break;
+    if ((int)(__builtin_amdgcn_readfirstlane(seen) - want) >= 0) break;
     __builtin_amdgcn_s_sleep(HIPDMA_SPIN_SLEEP);
   }
 }
@@ -314,7 +327,9 @@ public:
   {
     if (m_has_sync) {
       m_wait_target += m_wait_unit;
-      if ((int)(peeked - m_wait_target) < 0) hipdma::detail::wait_word(m_full, m_wait_target);
+      // every lane peeked at the same word with the same instruction: a scalar comparison
+      if ((int)(__builtin_amdgcn_readfirstlane(peeked) - __builtin_amdgcn_readfirstlane(m_wait_target)) < 0)
+        hipdma::detail::wait_word(m_full, m_wait_target);
       else hipdma::detail::acquire_lds();
     }
   }

@@ -156,6 +156,36 @@ __device__ __forceinline__ void load_to_lds(const char* global_lane_ptr, char* l
                                      (HIPDMA_LDS_AS void*)lds_wave_base, 4, 0, 0);
 }
 
+// The same move with the source address split into a part that is the same in every lane, held
+// in scalar registers, and a 32-bit offset per lane: no vector ALU instruction is needed to form
+// the address.  Written as assembly because the compiler only picks this form of the instruction
+// when it finds the zero-extension of the lane offset in the same basic block as the load, and it
+// moves a loop-invariant one out of the loop.  It does not count the load among the LDS writes it
+// tracks: the caller waits with wait_lds_direct() / wait_lds_direct_but<N>(), as for load_to_lds().
+// `scalar_base` and `lds_wave_base` must come out of scalar_u32() / scalar_ptr() or scalar
+// arithmetic on such values.
+__device__ __forceinline__ unsigned scalar_u32(const unsigned v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ const char* scalar_ptr(const char* p)
+{
+  const unsigned long long bits = (unsigned long long)p;
+  return (const char*)(((unsigned long long)scalar_u32((unsigned)(bits >> 32)) << 32) | (unsigned long long)scalar_u32((unsigned)bits));
+}
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"      // m0 is a reserved register: naming it keeps the compiler from merging its own writes across this one
+template<int BYTES>
+__device__ __forceinline__ void load_to_lds_scalar_base(const char* scalar_base, const unsigned lane_offset,
+                                                        const unsigned lds_wave_base)
+{
+  static_assert(BYTES == 4 || BYTES == 16, "global_load_lds moves 4 or 16 bytes per lane here");
+  if constexpr (BYTES == 16)
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 : : "v"(lane_offset), "s"(scalar_base), "s"(lds_wave_base) : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
+                 : : "v"(lane_offset), "s"(scalar_base), "s"(lds_wave_base) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+
 // Wait until every global -> LDS move of this wavefront has landed.
 __device__ __forceinline__ void wait_lds_direct()
 {

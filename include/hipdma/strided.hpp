@@ -301,6 +301,34 @@ private:
   {
     using namespace hipdma::detail;
     const int lane = lane_id();
+    // When a round moves every thread down whole rows and a round's rows span less than 4 GiB of the
+    // source, a load is written as "scalar base + 32-bit lane offset": the base (source, rows of the
+    // round) and the LDS address are scalar arithmetic, the lane offsets do not change from one transfer
+    // to the next, and no vector ALU instruction is left between two loads.  It matters next to compute
+    // wavefronts that issue matrix instructions back to back: a vector ALU instruction of the DMA
+    // wavefront then waits for a gap between those.
+    if (m_grid.dcol == 0 && m_src_stride >= 0 &&
+        (long long)m_grid.drow * (long long)m_src_stride + (long long)m_grid.W * ALIGNMENT <= 0xffffffffLL) {
+      const unsigned lane_row = (unsigned)(m_grid.row0 * m_src_stride);
+      // The pointers, strides and rows per round are the same in every lane by the contract of the call;
+      // the compiler cannot always tell, so they are pinned to scalar registers once per transfer.
+      const char* const base = scalar_ptr(m_src);
+      const long long round_src = (long long)(int)scalar_u32((unsigned)m_grid.drow) * (long long)(int)scalar_u32((unsigned)m_src_stride);
+      const unsigned round_lds = scalar_u32((unsigned)(m_grid.drow * m_dst_stride));
+      // where lane 0 of this wavefront lands in round 0 (lane L lands L chunks further on)
+      const unsigned lds0 = scalar_u32((unsigned)(size_t)(HIPDMA_LDS_AS char*)dst) +
+                            scalar_u32((unsigned)(m_grid.row0 * m_dst_stride + (m_grid.col0 - lane) * ALIGNMENT));
+      GridCursor cur = m_grid.begin();
+      for (int r = 0; r < m_grid.rounds; ++r) {
+        if (m_grid.live(r, cur)) {
+          const unsigned lane_off = lane_row + (unsigned)(lds_col<SWIZZLE>(cur) * ALIGNMENT);
+          if constexpr (ALIGNMENT == 16 || ALIGNMENT == 4)
+            load_to_lds_scalar_base<ALIGNMENT>(base + r * round_src, lane_off, lds0 + r * round_lds);
+        }
+        m_grid.advance(cur);
+      }
+      return;
+    }
     GridCursor cur = m_grid.begin();
     for (int r = 0; r < m_grid.rounds; ++r) {
       if (m_grid.live(r, cur)) {
