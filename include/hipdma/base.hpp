@@ -280,7 +280,8 @@ public:
     HIPDMA_ASSERT(num_dma_threads > 0 && (num_dma_threads % HIPDMA_WAVE_SIZE) == 0);
     HIPDMA_ASSERT((dma_threadIdx_start % HIPDMA_WAVE_SIZE) == 0);
     HIPDMA_ASSERT(num_compute_threads > 0);
-    m_wait_unit = m_is_dma_thread ? unsigned(num_compute_threads) : unsigned(num_dma_threads);
+    // the same in every lane (a wavefront holds one role): pinned to a scalar register, and with it the targets
+    m_wait_unit = __builtin_amdgcn_readfirstlane(m_is_dma_thread ? unsigned(num_compute_threads) : unsigned(num_dma_threads));
     if (threadIdx.x == 0) {
       *m_full = 0u;
       *m_empty = 0u;
