@@ -101,6 +101,8 @@ static const VariantInfo kGemm[] = {
    "(three transfers in flight per DMA wavefront), eight compute wavefronts"},
   {"variant 6 with A transfers of two K steps (256 rows x 128 B, whole cache lines) into two 32 KB buffers with guards "
    "of their own; B keeps four stages of one K step"},
+  {"not warp-specialised: 256 x 256 tile, four wavefronts that each issue their share of the direct-to-LDS loads and "
+   "multiply a 128 x 128 block; one s_barrier per K step"},
 };
 
 static const VariantInfo kScatter[] = {

@@ -721,6 +721,164 @@ gemm_bf16_ws_direct4_a64(const unsigned short* __restrict__ a, const unsigned sh
   }
 }
 
+// ---- 256 x 256 tile without warp specialisation: four wavefronts that each fetch and multiply ----
+// The objects are the form of CudaDMAStrided that is not warp-specialised (all 256 threads issue their
+// share of a stage with issue_direct; src/examples/stencil/non_warp_specialized_single_buffer.h:47-57 is
+// the reference's use of that form).  A wavefront owns a SIMD and a 128 x 128 block of C: 256 accumulator
+// registers, 0.5 KB of fragments read per matrix instruction instead of 0.75, no DMA wavefronts to share the
+// register file with.  Four stages of one K step (32); a K step starts with one s_barrier: by then every
+// wavefront has waited for its own loads of the next stage, so that stage is complete, and every wavefront has
+// left the previous stage, so that buffer takes the loads of the stage three steps on.  Those eight loads per
+// thread are issued one at a time between groups of four products (issued back to back they hold the wavefront,
+// and with it its matrix core, for 550 cycles: the address unit takes one 16-byte load of a wavefront per
+// sixteen cycles); the fragments of the next slice, in the second half those of the next stage, are requested
+// under the products of the current one.
+__global__ void __launch_bounds__(256)
+gemm_bf16_all_direct(const unsigned short* __restrict__ a, const unsigned short* __restrict__ b, float* __restrict__ c,
+                     const int m, const int n, const int k)
+{
+  constexpr int WI = 4, WJ = 4, kStages = 4, kBK4 = 32, kThreads = 256;
+  constexpr int kBM = 256, kBN = 256;
+  constexpr int kARow = kBK4 * 2, kBRow = kBN * 2;                 // 64 B and 512 B, unpadded
+  constexpr int kAStage = kBM * kARow, kBStage = kBK4 * kBRow;     // 16 KB and 16 KB
+  typedef CudaDMAStrided<false, 16, 16, kARow, kThreads, kBM> dma_a_t;
+  typedef CudaDMAStrided<false, 16, 16, kBRow, kThreads, kBK4> dma_b_t;
+  constexpr int kLoads = dma_a_t::loads_per_thread() + dma_b_t::loads_per_thread();     // per stage and thread
+  __shared__ __attribute__((aligned(1024))) char lds_a[kStages][kAStage];
+  __shared__ __attribute__((aligned(1024))) char lds_b[kStages][kBStage];
+  dma_a_t dma_a(k * 2, kARow);
+  dma_b_t dma_b(n * 2, kBRow);
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, m / kBM, n / kBN, tile_m, tile_n);
+  const int ksteps = k / kBK4;            // a multiple of four
+  const int klast = ksteps - 1;
+  const unsigned short* const src_a = a + (size_t)tile_m * kBM * k;
+  const unsigned short* const src_b = b + (size_t)tile_n * kBN;
+  const size_t step_b = (size_t)kBK4 * n;
+  // Stage t of the K loop into buffer t % 4: round g of the A loads (g < 4) or round g - 4 of the B loads.  Past
+  // the end the last stage is requested again (into a buffer nobody reads any more): the loop keeps one shape and
+  // one wait count.
+  static_assert(dma_a_t::loads_per_thread() == 4 && dma_b_t::loads_per_thread() == 4, "eight loads per thread and stage");
+  auto issue = [&](const int t, const int buf, const int g) __attribute__((always_inline)) {
+    const int tt = t < klast ? t : klast;
+    if (g < 4) dma_a.template issue_direct_part<STORE_LDS_DIRECT_SWIZZLE, true>(src_a + (size_t)tt * kBK4, lds_a[buf], g, 1);
+    else dma_b.template issue_direct_part<STORE_LDS_DIRECT_SWIZZLE, true>(src_b + (size_t)tt * step_b, lds_b[buf], g - 4, 1);
+  };
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = (wave >> 1) * 32 * WI, wn = (wave & 1) * 32 * WJ;
+  f32x16_t acc[WI][WJ];
+#pragma unroll
+  for (int i = 0; i < WI; ++i)
+#pragma unroll
+    for (int j = 0; j < WJ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  int a_lane[kBK4 / 16];
+  {
+    const int row = wm + (lane & 31);
+#pragma unroll
+    for (int ks = 0; ks < kBK4 / 16; ++ks)
+      a_lane[ks] = row * kARow + hipdma::swizzled_chunk(row, 2 * ks + (lane >> 5), kARow / 16) * 16;
+  }
+  int b_lo[WJ], b_hi[WJ];
+  {
+    const int j16 = lane & 15;
+    const int row = (lane >> 5) * 8 + (j16 >> 2);
+#pragma unroll
+    for (int j = 0; j < WJ; ++j) {
+      const int col_bytes = (wn + j * 32 + ((lane >> 4) & 1) * 16 + (j16 & 3) * 4) * 2;
+      b_lo[j] = row * kBRow + hipdma::swizzled_chunk(row, col_bytes >> 4, kBRow / 16) * 16 + (col_bytes & 15);
+      b_hi[j] = (row + 4) * kBRow + hipdma::swizzled_chunk(row + 4, col_bytes >> 4, kBRow / 16) * 16 + (col_bytes & 15);
+    }
+  }
+  auto load_frags = [&](bf16x8_t (&fa)[WI], bf16x8_t (&fb)[WJ], const int buf, const int ks) __attribute__((always_inline)) {
+    const char* sa = lds_a[buf]; const char* sb = lds_b[buf];
+#pragma unroll
+    for (int i = 0; i < WI; ++i) fa[i] = *(const bf16x8_t*)(sa + i * 32 * kARow + a_lane[ks]);
+#pragma unroll
+    for (int j = 0; j < WJ; ++j) {
+      const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+          (__attribute__((address_space(3))) bf16x4_t*)(sb + ks * 16 * kBRow + b_lo[j]));
+      const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+          (__attribute__((address_space(3))) bf16x4_t*)(sb + ks * 16 * kBRow + b_hi[j]));
+      fb[j] = bf16x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+  };
+  // Half a K step: the sixteen products of the slice in (fa, fb) in four groups of four.  Under the first three
+  // groups the fragments of the slice (nbuf, nks) are requested into (na, nb): the four A blocks, then two B blocks
+  // twice.  Behind every group goes one load of stage t + 3.  Nothing moves across the ends of a group.
+  auto half_step = [&](const bf16x8_t (&fa)[WI], const bf16x8_t (&fb)[WJ], bf16x8_t (&na)[WI], bf16x8_t (&nb)[WJ],
+                       const int nbuf, const int nks, const int t, const int buf, const int first_load)
+      __attribute__((always_inline)) {
+    const char* sa = lds_a[nbuf]; const char* sb = lds_b[nbuf];
+#pragma unroll
+    for (int i = 0; i < WI; ++i) {
+      if (i == 0) {
+#pragma unroll
+        for (int q = 0; q < WI; ++q) na[q] = *(const bf16x8_t*)(sa + q * 32 * kARow + a_lane[nks]);
+      } else if (i < 3) {
+#pragma unroll
+        for (int j = 2 * (i - 1); j < 2 * i; ++j) {
+          const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+              (__attribute__((address_space(3))) bf16x4_t*)(sb + nks * 16 * kBRow + b_lo[j]));
+          const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+              (__attribute__((address_space(3))) bf16x4_t*)(sb + nks * 16 * kBRow + b_hi[j]));
+          nb[j] = bf16x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < WJ; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      // product, request, product, request, ...
+#pragma unroll
+      for (int q = 0; q < WJ; ++q) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      issue(t + 3, (buf + 3) % kStages, first_load + i);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  bf16x8_t fa0[WI], fb0[WJ], fa1[WI], fb1[WJ];
+#pragma unroll
+  for (int g = 0; g < 8; ++g) issue(0, 0, g);
+#pragma unroll
+  for (int g = 0; g < 8; ++g) issue(1, 1, g);
+#pragma unroll
+  for (int g = 0; g < 8; ++g) issue(2, 2, g);
+  hipdma::wait_direct_loads<2 * kLoads>();
+  __builtin_amdgcn_s_barrier();
+  load_frags(fa0, fb0, 0, 0);
+  // One K step on buffer `buf`: on entry fa0/fb0 hold its first slice and stages t + 1, t + 2 are in flight; on
+  // exit fa0/fb0 hold the first slice of the next step.
+  auto k_step = [&](const int t, const int buf) __attribute__((always_inline)) {
+    hipdma::wait_direct_loads<kLoads>();          // this thread's part of stage t + 1 (stage t + 2 stays in flight)
+    __builtin_amdgcn_s_barrier();
+    half_step(fa0, fb0, fa1, fb1, buf, 1, t, buf, 0);
+    half_step(fa1, fb1, fa0, fb0, (buf + 1) % kStages, 0, t, buf, 4);
+  };
+  for (int kt = 0; kt < ksteps; kt += 4) {
+    k_step(kt, 0);
+    k_step(kt + 1, 1);
+    k_step(kt + 2, 2);
+    k_step(kt + 3, 3);
+  }
+  hipdma::wait_direct_loads<0>();
+  float* cbase = c + (size_t)(tile_m * kBM + wm) * n + (size_t)tile_n * kBN + wn;
+#pragma unroll
+  for (int i = 0; i < WI; ++i)
+#pragma unroll
+    for (int j = 0; j < WJ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
+        const int col = j * 32 + (lane & 31);
+        __builtin_nontemporal_store(acc[i][j][e], &cbase[(size_t)row * n + col]);
+      }
+}
+
 template<int WI, int WJ, int WM = 2, int WN = 2>
 int launch_gemm(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k, hipStream_t stream)
 {
@@ -766,12 +924,13 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
     case 2: return launch_gemm<2, 4>(d_a, d_b, d_c, m, n, k, s);
     case 3: return launch_gemm<4, 2>(d_a, d_b, d_c, m, n, k, s);
     case 5: return launch_gemm<4, 2, 2, 4>(d_a, d_b, d_c, m, n, k, s);
-    case 6: case 7: {
+    case 6: case 7: case 8: {
       CUDADMA_REQUIRE((m % 256) == 0 && (n % 256) == 0, "this variant needs m and n multiples of 256 (got %d x %d)", m, n);
       const long long grid = (long long)(m / 256) * (n / 256);
       CUDADMA_REQUIRE(grid <= 0x7fffffffLL, "grid too large");
       if (variant == 6) hipLaunchKernelGGL(gemm_bf16_ws_direct4, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
-      else hipLaunchKernelGGL(gemm_bf16_ws_direct4_a64, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
+      else if (variant == 7) hipLaunchKernelGGL(gemm_bf16_ws_direct4_a64, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
+      else hipLaunchKernelGGL(gemm_bf16_all_direct, dim3((unsigned)grid), dim3(256), 0, s, d_a, d_b, d_c, m, n, k);
       CUDADMA_HIP_CHECK(hipGetLastError());
       return CUDADMA_OK;
     }

@@ -193,6 +193,23 @@ public:
     m_src = (const char*)src_ptr;
     issue_direct_rounds<hipdma::detail::store_is_swizzled(DMA_STORE_QUAL)>((char*)dst_ptr);
   }
+  // A part of the same transfer: the loads of rounds [first_round, first_round + num_rounds) of the
+  // loads_per_thread() a thread issues for it, for callers that spread the loads of a transfer between other
+  // instructions (a wavefront that also computes holds up its own work while it issues loads back to back:
+  // the address unit takes a wavefront's 16-byte loads at one per sixteen cycles).
+  // With WHOLE_ROWS the caller vouches for the shape the scalar-base loads need (the DMA threads cover whole rows,
+  // a non-negative source stride, a round's rows within 4 GiB): only that form is compiled, and the few scalar
+  // instructions of a load fit under one matrix instruction.
+  template<int DMA_STORE_QUAL = STORE_LDS_DIRECT, bool WHOLE_ROWS = false>
+  __device__ __forceinline__ void issue_direct_part(const void* __restrict__ src_ptr, void* __restrict__ dst_ptr,
+                                                    const int first_round, const int num_rounds)
+  {
+    static_assert(hipdma::detail::store_is_direct(DMA_STORE_QUAL), "issue_direct_part takes one of the STORE_LDS_DIRECT qualifiers");
+    static_assert(ALIGNMENT == 16 || ALIGNMENT == 4, "global_load_lds moves 4 or 16 bytes per lane");
+    HIPDMA_ASSERT(direct_ready());
+    m_src = (const char*)src_ptr;
+    issue_direct_rounds<hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), WHOLE_ROWS>((char*)dst_ptr, first_round, first_round + num_rounds);
+  }
   // True when this object's shape can use global_load_lds (whole chunks, whole wavefronts, rows of
   // at least a wavefront of chunks or unpadded power-of-two rows).
   __device__ __forceinline__ bool direct_ready() const { return use_direct<STORE_LDS_DIRECT>(); }
@@ -296,8 +313,8 @@ private:
     hipdma::detail::wait_lds_direct();
   }
 
-  template<bool SWIZZLE>
-  __device__ __forceinline__ void issue_direct_rounds(char* dst)
+  template<bool SWIZZLE, bool WHOLE_ROWS = false>
+  __device__ __forceinline__ void issue_direct_rounds(char* dst, const int first = 0, const int end = 0x7fffffff)
   {
     using namespace hipdma::detail;
     const int lane = lane_id();
@@ -307,8 +324,10 @@ private:
     // to the next, and no vector ALU instruction is left between two loads.  It matters next to compute
     // wavefronts that issue matrix instructions back to back: a vector ALU instruction of the DMA
     // wavefront then waits for a gap between those.
-    if (m_grid.dcol == 0 && m_src_stride >= 0 &&
-        (long long)m_grid.drow * (long long)m_src_stride + (long long)m_grid.W * ALIGNMENT <= 0xffffffffLL) {
+    const bool whole_rows = (m_grid.dcol == 0) && (m_src_stride >= 0) &&
+        ((long long)m_grid.drow * (long long)m_src_stride + (long long)m_grid.W * ALIGNMENT <= 0xffffffffLL);
+    if constexpr (WHOLE_ROWS) HIPDMA_ASSERT(whole_rows);
+    if (WHOLE_ROWS || whole_rows) {
       const unsigned lane_row = (unsigned)(m_grid.row0 * m_src_stride);
       // The pointers, strides and rows per round are the same in every lane by the contract of the call;
       // the compiler cannot always tell, so they are pinned to scalar registers once per transfer.
@@ -320,7 +339,7 @@ private:
                             scalar_u32((unsigned)(m_grid.row0 * m_dst_stride + (m_grid.col0 - lane) * ALIGNMENT));
       GridCursor cur = m_grid.begin();
       for (int r = 0; r < m_grid.rounds; ++r) {
-        if (m_grid.live(r, cur)) {
+        if (r >= first && r < end && m_grid.live(r, cur)) {
           const unsigned lane_off = lane_row + (unsigned)(lds_col<SWIZZLE>(cur) * ALIGNMENT);
           if constexpr (ALIGNMENT == 16 || ALIGNMENT == 4)
             load_to_lds_scalar_base<ALIGNMENT>(base + r * round_src, lane_off, lds0 + r * round_lds);
@@ -331,7 +350,7 @@ private:
     }
     GridCursor cur = m_grid.begin();
     for (int r = 0; r < m_grid.rounds; ++r) {
-      if (m_grid.live(r, cur)) {
+      if (r >= first && r < end && m_grid.live(r, cur)) {
         const int lds_off = cur.row * m_dst_stride + cur.col * ALIGNMENT;
         if constexpr (ALIGNMENT == 16 || ALIGNMENT == 4)
           load_to_lds<ALIGNMENT>(m_src + cur.row * m_src_stride + lds_col<SWIZZLE>(cur) * ALIGNMENT,
