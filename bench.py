@@ -232,11 +232,16 @@ def main():
     flops = 2.0 * dim ** 3
     gemm = {"TFLOP/s": round(flops / ms / 1e9, 1), "frac_of_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4),
             "ms": round(ms, 4), "flop": flops,
-            "workload": "C = A*B, bf16 4096^3, fp32 accumulate, 256x256 workgroup tile: 256x64 A tiles (two buffers) and "
-                        "32x256 B tiles (four stages) brought into swizzled LDS by CudaDMAStrided::issue_direct "
-                        "(global_load_lds) in four DMA wavefronts, v_mfma_f32_32x32x16_bf16 on 128x64 tiles in eight "
-                        "compute wavefronts"}
+            "workload": "C = A*B, bf16 4096^3, fp32 accumulate, 256x256 workgroup tile in four stages of K=32 brought "
+                        "into swizzled LDS by CudaDMAStrided::issue_direct_part (global_load_lds) from the same four "
+                        "wavefronts that multiply (v_mfma_f32_32x32x16_bf16, 128x128 per wavefront), one load between "
+                        "every four matrix instructions"}
+    ms_ws, _ = time_launches(lambda: wl.gemm_bf16(ga, gb, gc, 7), max(steps, 50), warmup, SETTLE_MS)
+    gemm["warp_specialised"] = {"TFLOP/s": round(flops / ms_ws / 1e9, 1), "ms": round(ms_ws, 4),
+                                "workload": "the same tile with four DMA wavefronts feeding eight compute wavefronts "
+                                            "(128x64 per wavefront), variant 7"}
     log(f"gemm         {ms:9.4f} ms  {gemm['TFLOP/s']:8.1f} TFLOP/s  {100 * gemm['frac_of_mfma_peak']:5.1f}% of 2.5 PFLOP/s")
+    log(f"gemm_ws      {ms_ws:9.4f} ms  {gemm['warp_specialised']['TFLOP/s']:8.1f} TFLOP/s  (warp-specialised, variant 7)")
     del ga, gb, gc
 
     value = patterns["strided"]["GB/s"]

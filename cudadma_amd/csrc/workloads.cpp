@@ -86,7 +86,7 @@ static const VariantInfo kHalo[] = {
 };
 
 static const VariantInfo kGemm[] = {
-  {"the largest workgroup tile that divides the problem and gives every compute unit a tile: variant 7, 3 or 2, else "
+  {"the largest workgroup tile that divides the problem and gives every compute unit a tile: variant 8, 3 or 2, else "
    "variant 1"},
   {"warp-specialised: two DMA wavefronts per operand with two CudaDMAStrided objects each (two LDS stages, tile two K "
    "steps ahead in flight), four compute wavefronts with v_mfma_f32_32x32x16_bf16, B fragments through "

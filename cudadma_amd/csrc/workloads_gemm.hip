@@ -914,7 +914,7 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
     // the largest tile that divides the problem and still gives every compute unit a tile; the small one otherwise
     const long long cus = workloads::device_cus();
     const bool m256 = (m % 256) == 0, n256 = (n % 256) == 0;
-    if (m256 && n256 && (long long)(m / 256) * (n / 256) >= cus) variant = 7;
+    if (m256 && n256 && (long long)(m / 256) * (n / 256) >= cus) variant = 8;
     else if (m256 && (long long)(m / 256) * (n / 128) >= cus) variant = 3;
     else if (n256 && (long long)(m / 128) * (n / 256) >= cus) variant = 2;
     else variant = 1;

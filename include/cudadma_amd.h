@@ -233,14 +233,16 @@ int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz
 /* Config 5 (no GEMM in the reference; nearest: src/examples/sgemv/sgemv_dma.cu:329-388):
  * C = A * B with A m x k and B k x n row-major bf16 (as uint16 bit patterns), C m x n
  * float, fp32 accumulation on the matrix cores.  m, n and k multiples of 128.
- * Four DMA wavefronts stage the A and B tiles of one K step (64) through CudaDMAStrided, four
- * compute wavefronts multiply.  variant 0 picks the largest workgroup tile that divides the
+ * In the warp-specialised variants four DMA wavefronts stage the A and B tiles of one K step
+ * through CudaDMAStrided and four or eight compute wavefronts multiply.  variant 0 picks the largest workgroup tile that divides the
  * problem and leaves no compute unit without a tile; 1: 128 x 128; 2: 128 x 256 (n a multiple of
  * 256); 3: 256 x 128 (m a multiple of 256); 4: 256 x 128 with the tiles brought in by
  * global_load_lds into swizzled LDS rows; 5: 256 x 256 with eight compute wavefronts (m and n
  * multiples of 256); 6: the same tile with K steps of 32 brought into four swizzled LDS stages by
  * global_load_lds; 7: variant 6 with A transfers of two K steps (rows of 128 B, whole cache
- * lines) into two buffers of their own. */
+ * lines) into two buffers of their own; 8: the 256 x 256 tile without warp specialisation: four
+ * wavefronts that each issue their share of the direct-to-LDS loads (the form of CudaDMAStrided
+ * that is not warp-specialised) between the matrix instructions of their 128 x 128 block. */
 int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k,
                       int variant, void* stream);
 
