@@ -79,12 +79,19 @@ template<bool ONE, int A, int BPT, int E, int T, int N> struct Make<false, 4, ON
 // through issue_direct() + wait_direct_loads<0>() with the hand-off done by hand around them
 // (the form a kernel uses to keep several direct transfers in flight); otherwise through the
 // ordinary calls, which fall back to registers when the shape does not fit.
+// Every other repetition issues the transfer in two parts (its first load, then the rest) through
+// issue_direct_part().
 template<bool WS, int SQ, typename Obj>
-__device__ __forceinline__ void direct_transfer(Obj& dma, const int two_phase, const void* src, void* dst)
+__device__ __forceinline__ void direct_transfer(Obj& dma, const int two_phase, const void* src, void* dst, const int rep)
 {
   if (two_phase && dma.direct_ready()) {
     if constexpr (WS) dma.wait_for_dma_start();
-    dma.template issue_direct<SQ>(src, dst);
+    if (rep & 1) {
+      dma.template issue_direct_part<SQ>(src, dst, 0, 1);
+      dma.template issue_direct_part<SQ>(src, dst, 1, 0x3fffffff);
+    } else {
+      dma.template issue_direct<SQ>(src, dst);
+    }
     hipdma::wait_direct_loads<0>();
     if constexpr (WS) dma.finish_async_dma();
   } else {
@@ -104,12 +111,12 @@ __global__ void __launch_bounds__(1024) strided_kernel(const Args a)
     const char* src = a.reverse ? (const char*)lds + a.src_offset : a.in + a.src_offset + (size_t)rep * a.rep_src_bytes;
     char* dst = a.reverse ? a.out + (size_t)rep * a.out_bytes + a.dst_offset : (char*)lds + a.dst_offset;
     if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
-      if constexpr (A == 16 || A == 4) direct_transfer<WS, STORE_LDS_DIRECT>(dma, a.two_phase, src, dst);
+      if constexpr (A == 16 || A == 4) direct_transfer<WS, STORE_LDS_DIRECT>(dma, a.two_phase, src, dst, rep);
     } else if (a.call_style == CUDADMA_CALL_LDS_SWIZZLE) {
       if constexpr (kWholeChunks) harness::do_transfer_direct<STORE_LDS_SWIZZLE>(dma, a.two_phase, src, dst);
     } else if (a.call_style == CUDADMA_CALL_LDS_DIRECT_SWIZZLE) {
       if constexpr ((A == 16 || A == 4) && kWholeChunks)
-        direct_transfer<WS, STORE_LDS_DIRECT_SWIZZLE>(dma, a.two_phase, src, dst);
+        direct_transfer<WS, STORE_LDS_DIRECT_SWIZZLE>(dma, a.two_phase, src, dst, rep);
     } else {
       harness::do_transfer(dma, a.call_style, a.two_phase, src, dst);
     }
