@@ -14,6 +14,18 @@
 //     start the DMA threads at a multiple of 64;
 //   * construct every warp-specialised object in all threads of the workgroup,
 //     before the code branches on owns_this_thread().
+//
+// What exists here and not in the CUDA header:
+//   * store qualifiers STORE_LDS, STORE_LDS_DIRECT, STORE_LDS_SWIZZLE, STORE_LDS_DIRECT_SWIZZLE and
+//     hipdma::swizzled_chunk() for readers of swizzled rows (base.hpp, strided.hpp);
+//   * CudaDMAHalo with the v2 template parameters and two-phase calls (halo.hpp);
+//   * peek_dma_finish() + wait_for_dma_finish(peeked), the wait in two halves (base.hpp);
+//   * CudaDMAStrided::issue_direct() / issue_direct_part() + hipdma::wait_direct_loads<N>() and the
+//     wait_for_dma_start_direct() / finish_async_dma_direct() hand-off, for kernels that keep several
+//     direct-to-LDS transfers in flight or spread the loads of one between other instructions
+//     (strided.hpp, base.hpp);
+//   * hipdma::GroupBarrier, a barrier among some of the workgroup's wavefronts (base.hpp);
+//   * HIPDMA_SPIN_LIMIT, HIPDMA_FULL_FENCE, DEBUG_CUDADMA build switches (base.hpp).
 #pragma once
 
 #include "hipdma/base.hpp"
