@@ -111,13 +111,13 @@ def main(argv=None):
             src = wl.fill_uniform(torch.empty(n * n, device=dev), 1002)
             dst = torch.empty_like(src)
             cus = torch.cuda.get_device_properties(0).multi_processor_count
-            print("# memory probes on 2 x 1 GiB; GB/s of bytes read + written; columns: workgroups per CU 2 / 4 / 8 / 16")
+            print("# memory probes on 2 x 1 GiB; GB/s of bytes read + written; columns: workgroups per CU 0.5 / 1 / 1.5 / 2 / 3 / 4 / 8 / 16")
             for mode, label in enumerate(wl.PROBE_MODES):
                 cells = []
-                for wg in (2, 4, 8, 16):
+                for wg in (0.5, 1, 1.5, 2, 3, 4, 8, 16):
                     s_, d_ = (None if label.startswith("write") else src), (None if label == "read" else dst)
-                    nbytes = wl.probe_memory(mode, s_, d_, cus * wg)
-                    ms = _time(lambda: wl.probe_memory(mode, s_, d_, cus * wg), args.steps, settle_ms=10.0)
+                    nbytes = wl.probe_memory(mode, s_, d_, int(cus * wg))
+                    ms = _time(lambda: wl.probe_memory(mode, s_, d_, int(cus * wg)), args.steps, settle_ms=10.0)
                     cells.append(f"{ms:7.4f} ms {nbytes / ms / 1e6:6.0f}")
                 print(f"{label:22s} " + "   ".join(cells), flush=True)
         elif name == "scatter":
