@@ -237,7 +237,10 @@ def main():
                         "wavefronts that multiply (v_mfma_f32_32x32x16_bf16, 128x128 per wavefront), one load between "
                         "every four matrix instructions"}
     ms_ws, _ = time_launches(lambda: wl.gemm_bf16(ga, gb, gc, 7), max(steps, 50), warmup, SETTLE_MS)
-    gemm["warp_specialised"] = {"TFLOP/s": round(flops / ms_ws / 1e9, 1), "ms": round(ms_ws, 4),
+    gemm["note"] = ("config 5 names the warp-specialised kernel: it is reported under warp_specialised; the figures at "
+                    "this level are the form of the same objects that is not warp-specialised, the faster one")
+    gemm["warp_specialised"] = {"TFLOP/s": round(flops / ms_ws / 1e9, 1),
+                                "frac_of_mfma_peak": round(flops / ms_ws / 1e9 / 2500.0, 4), "ms": round(ms_ws, 4),
                                 "workload": "the same tile with four DMA wavefronts feeding eight compute wavefronts "
                                             "(128x64 per wavefront), variant 7"}
     log(f"gemm         {ms:9.4f} ms  {gemm['TFLOP/s']:8.1f} TFLOP/s  {100 * gemm['frac_of_mfma_peak']:5.1f}% of 2.5 PFLOP/s")
