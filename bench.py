@@ -232,10 +232,10 @@ def main():
     flops = 2.0 * dim ** 3
     gemm = {"TFLOP/s": round(flops / ms / 1e9, 1), "frac_of_mfma_peak": round(flops / ms / 1e9 / 2500.0, 4),
             "ms": round(ms, 4), "flop": flops,
-            "workload": "C = A*B, bf16 4096^3, fp32 accumulate, 256x256 workgroup tile in four stages of K=32 brought "
-                        "into swizzled LDS by CudaDMAStrided::issue_direct_part (global_load_lds) from the same four "
-                        "wavefronts that multiply (v_mfma_f32_32x32x16_bf16, 128x128 per wavefront), one load between "
-                        "every four matrix instructions"}
+            "workload": "C = A*B, bf16 4096^3, fp32 accumulate, 256x256 workgroup tile: B in four stages of K=32, A in "
+                        "three buffers of K=64, brought into swizzled LDS by CudaDMAStrided::issue_direct_part "
+                        "(global_load_lds) from the same four wavefronts that multiply (v_mfma_f32_32x32x16_bf16, "
+                        "128x128 per wavefront), one load between every four matrix instructions"}
     ms_ws, _ = time_launches(lambda: wl.gemm_bf16(ga, gb, gc, 7), max(steps, 50), warmup, SETTLE_MS)
     gemm["note"] = ("config 5 names the warp-specialised kernel: it is reported under warp_specialised; the figures at "
                     "this level are the form of the same objects that is not warp-specialised, the faster one")

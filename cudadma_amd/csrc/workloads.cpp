@@ -86,7 +86,7 @@ static const VariantInfo kHalo[] = {
 };
 
 static const VariantInfo kGemm[] = {
-  {"the largest workgroup tile that divides the problem and gives every compute unit a tile: variant 8, 3 or 2, else "
+  {"the largest workgroup tile that divides the problem and gives every compute unit a tile: variant 9, 3 or 2, else "
    "variant 1"},
   {"warp-specialised: two DMA wavefronts per operand with two CudaDMAStrided objects each (two LDS stages, tile two K "
    "steps ahead in flight), four compute wavefronts with v_mfma_f32_32x32x16_bf16, B fragments through "
@@ -103,6 +103,8 @@ static const VariantInfo kGemm[] = {
    "of their own; B keeps four stages of one K step"},
   {"not warp-specialised: 256 x 256 tile, four wavefronts that each issue their share of the direct-to-LDS loads and "
    "multiply a 128 x 128 block; one s_barrier per K step"},
+  {"variant 8 with A transfers of two K steps (rows of 128 B, whole cache lines) into a ring of three buffers: with the "
+   "four B stages all of the 160 KB of LDS"},
 };
 
 static const VariantInfo kScatter[] = {

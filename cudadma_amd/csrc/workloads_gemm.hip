@@ -879,6 +879,175 @@ gemm_bf16_all_direct(const unsigned short* __restrict__ a, const unsigned short*
       }
 }
 
+// ---- the same kernel with A transfers of two K steps (rows of 128 B) ----
+// A K step of 32 takes 64 B of an A row, half a cache line, and the L1 asks the L2 for every line of the A panel
+// twice (TCP_TCC_READ_REQ: 12.8 M requests per 4096^3 launch instead of 8.4 M).  Here an A transfer is 256 rows x
+// 128 B for two K steps.  Three A buffers (96 KB) and the four B stages (64 KB) are all of the LDS: an A buffer is
+// free two K steps after its last read and its next transfer has to be complete a step before its first, so two
+// buffers would leave it one K step to land.  The A buffers form a ring indexed at run time (three does not divide
+// the K steps of every problem); a K step still issues eight loads, four of B and half an A transfer.
+__global__ void __launch_bounds__(256)
+gemm_bf16_all_direct_a64(const unsigned short* __restrict__ a, const unsigned short* __restrict__ b, float* __restrict__ c,
+                         const int m, const int n, const int k)
+{
+  constexpr int WI = 4, WJ = 4, kBStages = 4, kABufs = 3, kBK4 = 32, kThreads = 256;
+  constexpr int kBM = 256, kBN = 256;
+  constexpr int kARow = 4 * kBK4, kBRow = kBN * 2;                 // 128 B (two K steps) and 512 B, unpadded
+  constexpr int kABuf = kBM * kARow, kBStage = kBK4 * kBRow;       // 32 KB and 16 KB
+  typedef CudaDMAStrided<false, 16, 16, kARow, kThreads, kBM> dma_a_t;
+  typedef CudaDMAStrided<false, 16, 16, kBRow, kThreads, kBK4> dma_b_t;
+  static_assert(dma_a_t::loads_per_thread() == 8 && dma_b_t::loads_per_thread() == 4, "eight loads per thread and K step");
+  constexpr int kLoads = 8;
+  __shared__ __attribute__((aligned(1024))) char lds_a[kABufs * kABuf];
+  __shared__ __attribute__((aligned(1024))) char lds_b[kBStages][kBStage];
+  dma_a_t dma_a(k * 2, kARow);
+  dma_b_t dma_b(n * 2, kBRow);
+  int tile_m, tile_n;
+  tile_of_workgroup(blockIdx.x, m / kBM, n / kBN, tile_m, tile_n);
+  const int ksteps = k / kBK4;            // a multiple of four
+  const int klast = ksteps - 1, dlast = ksteps / 2 - 1;
+  const unsigned short* const src_a = a + (size_t)tile_m * kBM * k;
+  const unsigned short* const src_b = b + (size_t)tile_n * kBN;
+  const size_t step_b = (size_t)kBK4 * n;
+  // Round r of the B stage of K step t into B buffer `buf`; round r of A transfer d (K steps 2d, 2d+1) into A
+  // buffer `buf`.  Past the end the last one is requested again, into a buffer nobody reads any more.
+  auto issue_b = [&](const int t, const int buf, const int r) __attribute__((always_inline)) {
+    const int tt = t < klast ? t : klast;
+    dma_b.template issue_direct_part<STORE_LDS_DIRECT_SWIZZLE, true>(src_b + (size_t)tt * step_b, lds_b[buf], r, 1);
+  };
+  auto issue_a = [&](const int d, const int buf, const int r) __attribute__((always_inline)) {
+    const int dd = d < dlast ? d : dlast;
+    dma_a.template issue_direct_part<STORE_LDS_DIRECT_SWIZZLE, true>(src_a + (size_t)dd * (2 * kBK4), lds_a + buf * kABuf, r, 1);
+  };
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wm = (wave >> 1) * 32 * WI, wn = (wave & 1) * 32 * WJ;
+  f32x16_t acc[WI][WJ];
+#pragma unroll
+  for (int i = 0; i < WI; ++i)
+#pragma unroll
+    for (int j = 0; j < WJ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  // A fragment of slice q (0..3 inside a buffer): row wm + 32*i + lane%32, chunk 2*q + lane/32 of the 8 chunks of the row
+  int a_lane[4];
+  {
+    const int row = wm + (lane & 31);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      a_lane[q] = row * kARow + hipdma::swizzled_chunk(row, 2 * q + (lane >> 5), kARow / 16) * 16;
+  }
+  int b_lo[WJ], b_hi[WJ];
+  {
+    const int j16 = lane & 15;
+    const int row = (lane >> 5) * 8 + (j16 >> 2);
+#pragma unroll
+    for (int j = 0; j < WJ; ++j) {
+      const int col_bytes = (wn + j * 32 + ((lane >> 4) & 1) * 16 + (j16 & 3) * 4) * 2;
+      b_lo[j] = row * kBRow + hipdma::swizzled_chunk(row, col_bytes >> 4, kBRow / 16) * 16 + (col_bytes & 15);
+      b_hi[j] = (row + 4) * kBRow + hipdma::swizzled_chunk(row + 4, col_bytes >> 4, kBRow / 16) * 16 + (col_bytes & 15);
+    }
+  }
+  // Half a K step: sixteen products in four groups; under the first three the fragments of slice q of A buffer
+  // `abuf` and of slice ks of B stage `bbuf` are requested into (na, nb); `after_group(i)` places the loads.
+  auto half_step = [&](const bf16x8_t (&fa)[WI], const bf16x8_t (&fb)[WJ], bf16x8_t (&na)[WI], bf16x8_t (&nb)[WJ],
+                       const int abuf, const int q, const int bbuf, const int ks, auto after_group)
+      __attribute__((always_inline)) {
+    const char* sa = lds_a + abuf * kABuf; const char* sb = lds_b[bbuf];
+#pragma unroll
+    for (int i = 0; i < WI; ++i) {
+      if (i == 0) {
+#pragma unroll
+        for (int r = 0; r < WI; ++r) na[r] = *(const bf16x8_t*)(sa + r * 32 * kARow + a_lane[q]);
+      } else if (i < 3) {
+#pragma unroll
+        for (int j = 2 * (i - 1); j < 2 * i; ++j) {
+          const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+              (__attribute__((address_space(3))) bf16x4_t*)(sb + ks * 16 * kBRow + b_lo[j]));
+          const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+              (__attribute__((address_space(3))) bf16x4_t*)(sb + ks * 16 * kBRow + b_hi[j]));
+          nb[j] = bf16x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < WJ; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < WJ; ++r) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      after_group(i);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  bf16x8_t fa0[WI], fb0[WJ], fa1[WI], fb1[WJ];
+  // Before the loop, in the order the loop's wait counts assume: (A transfer 0, B stage 0), then what K steps -2
+  // and -1 would have issued: (B stage 1, first half of A transfer 1), (B stage 2, second half of A transfer 1).
+#pragma unroll
+  for (int r = 0; r < 8; ++r) issue_a(0, 0, r);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) issue_b(0, 0, r);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) issue_b(1, 1, r);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) issue_a(1, 1, r);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) issue_b(2, 2, r);
+#pragma unroll
+  for (int r = 4; r < 8; ++r) issue_a(1, 1, r);
+  hipdma::wait_direct_loads<2 * kLoads>();
+  __builtin_amdgcn_s_barrier();
+  // first slice of K step 0
+  {
+#pragma unroll
+    for (int r = 0; r < WI; ++r) fa0[r] = *(const bf16x8_t*)(lds_a + r * 32 * kARow + a_lane[0]);
+#pragma unroll
+    for (int j = 0; j < WJ; ++j) {
+      const bf16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4_t*)(lds_b[0] + b_lo[j]));
+      const bf16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4_t*)(lds_b[0] + b_hi[j]));
+      fb0[j] = bf16x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+  }
+  // One K step t on B buffer bbuf and slices (2*h, 2*h+1) of A buffer abuf; the next step starts in A buffer nabuf
+  // at slice nq.  It issues B stage t + 3 and rounds [ar, ar + 4) of A transfer ad into A buffer aibuf.
+  auto k_step = [&](const int t, const int bbuf, const int abuf, const int h, const int nabuf, const int nq,
+                    const int ad, const int aibuf, const int ar) __attribute__((always_inline)) {
+    hipdma::wait_direct_loads<kLoads>();          // everything up to K step t - 2; what step t - 1 issued stays in flight
+    __builtin_amdgcn_s_barrier();
+    half_step(fa0, fb0, fa1, fb1, abuf, 2 * h + 1, bbuf, 1, [&](const int i) __attribute__((always_inline)) {
+      issue_b(t + 3, (bbuf + 3) % kBStages, i);
+    });
+    half_step(fa1, fb1, fa0, fb0, nabuf, nq, (bbuf + 1) % kBStages, 0, [&](const int i) __attribute__((always_inline)) {
+      issue_a(ad, aibuf, ar + i);
+    });
+  };
+  int ab0 = 0;                                // A buffer of transfer kt / 2
+  for (int kt = 0; kt < ksteps; kt += 4) {
+    const int ab1 = ab0 == 2 ? 0 : ab0 + 1;   // transfer kt / 2 + 1
+    const int ab2 = ab1 == 2 ? 0 : ab1 + 1;   // transfer kt / 2 + 2, requested during K steps kt and kt + 1
+    const int d = kt >> 1;
+    k_step(kt, 0, ab0, 0, ab0, 2, d + 2, ab2, 0);
+    k_step(kt + 1, 1, ab0, 1, ab1, 0, d + 2, ab2, 4);
+    k_step(kt + 2, 2, ab1, 0, ab1, 2, d + 3, ab0, 0);     // transfer kt / 2 + 3 takes the buffer transfer kt / 2 has left
+    k_step(kt + 3, 3, ab1, 1, ab2, 0, d + 3, ab0, 4);
+    ab0 = ab2;
+  }
+  hipdma::wait_direct_loads<0>();
+  float* cbase = c + (size_t)(tile_m * kBM + wm) * n + (size_t)tile_n * kBN + wn;
+#pragma unroll
+  for (int i = 0; i < WI; ++i)
+#pragma unroll
+    for (int j = 0; j < WJ; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = i * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
+        const int col = j * 32 + (lane & 31);
+        __builtin_nontemporal_store(acc[i][j][e], &cbase[(size_t)row * n + col]);
+      }
+}
+
 template<int WI, int WJ, int WM = 2, int WN = 2>
 int launch_gemm(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k, hipStream_t stream)
 {
@@ -914,7 +1083,7 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
     // the largest tile that divides the problem and still gives every compute unit a tile; the small one otherwise
     const long long cus = workloads::device_cus();
     const bool m256 = (m % 256) == 0, n256 = (n % 256) == 0;
-    if (m256 && n256 && (long long)(m / 256) * (n / 256) >= cus) variant = 8;
+    if (m256 && n256 && (long long)(m / 256) * (n / 256) >= cus) variant = 9;
     else if (m256 && (long long)(m / 256) * (n / 128) >= cus) variant = 3;
     else if (n256 && (long long)(m / 128) * (n / 256) >= cus) variant = 2;
     else variant = 1;
@@ -924,13 +1093,14 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
     case 2: return launch_gemm<2, 4>(d_a, d_b, d_c, m, n, k, s);
     case 3: return launch_gemm<4, 2>(d_a, d_b, d_c, m, n, k, s);
     case 5: return launch_gemm<4, 2, 2, 4>(d_a, d_b, d_c, m, n, k, s);
-    case 6: case 7: case 8: {
+    case 6: case 7: case 8: case 9: {
       CUDADMA_REQUIRE((m % 256) == 0 && (n % 256) == 0, "this variant needs m and n multiples of 256 (got %d x %d)", m, n);
       const long long grid = (long long)(m / 256) * (n / 256);
       CUDADMA_REQUIRE(grid <= 0x7fffffffLL, "grid too large");
       if (variant == 6) hipLaunchKernelGGL(gemm_bf16_ws_direct4, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
       else if (variant == 7) hipLaunchKernelGGL(gemm_bf16_ws_direct4_a64, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
-      else hipLaunchKernelGGL(gemm_bf16_all_direct, dim3((unsigned)grid), dim3(256), 0, s, d_a, d_b, d_c, m, n, k);
+      else if (variant == 8) hipLaunchKernelGGL(gemm_bf16_all_direct, dim3((unsigned)grid), dim3(256), 0, s, d_a, d_b, d_c, m, n, k);
+      else hipLaunchKernelGGL(gemm_bf16_all_direct_a64, dim3((unsigned)grid), dim3(256), 0, s, d_a, d_b, d_c, m, n, k);
       CUDADMA_HIP_CHECK(hipGetLastError());
       return CUDADMA_OK;
     }

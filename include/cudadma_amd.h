@@ -242,7 +242,8 @@ int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz
  * global_load_lds; 7: variant 6 with A transfers of two K steps (rows of 128 B, whole cache
  * lines) into two buffers of their own; 8: the 256 x 256 tile without warp specialisation: four
  * wavefronts that each issue their share of the direct-to-LDS loads (the form of CudaDMAStrided
- * that is not warp-specialised) between the matrix instructions of their 128 x 128 block. */
+ * that is not warp-specialised) between the matrix instructions of their 128 x 128 block; 9:
+ * variant 8 with A transfers of two K steps in a ring of three buffers. */
 int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int m, int n, int k,
                       int variant, void* stream);
 

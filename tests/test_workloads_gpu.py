@@ -303,12 +303,12 @@ def _bf16_inputs(m, n, k):
     return a.reshape(m, k), b.reshape(k, n)
 
 
-@pytest.mark.parametrize("variant", range(9))
+@pytest.mark.parametrize("variant", range(10))
 @pytest.mark.parametrize("shape", [(128, 128, 128), (256, 384, 256), (512, 512, 512), (768, 256, 384), (256, 128, 128),
                                    (1024, 256, 896), (256, 256, 128), (256, 512, 640)])
 def test_gemm_small(device, shape, variant):
     m, n, k = shape
-    tile_m, tile_n = {0: (128, 128), 1: (128, 128), 2: (128, 256), 3: (256, 128), 4: (256, 128), 5: (256, 256), 6: (256, 256), 7: (256, 256), 8: (256, 256)}[variant]
+    tile_m, tile_n = {0: (128, 128), 1: (128, 128), 2: (128, 256), 3: (256, 128), 4: (256, 128), 5: (256, 256), 6: (256, 256), 7: (256, 256), 8: (256, 256), 9: (256, 256)}[variant]
     if m % tile_m or n % tile_n:
         # a tile shape that does not divide the problem is refused, not rounded
         with pytest.raises(cd.CudaDMAError, match="this variant needs"):
@@ -333,7 +333,7 @@ def test_gemm_small(device, shape, variant):
     assert float(np.max(np.abs(got - want))) <= 1e-4 * scale * np.sqrt(k)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
 def test_gemm_full_size(device, variant):
     m = n = k = 4096
     a, b = _bf16_inputs(m, n, k)
