@@ -144,12 +144,17 @@ def main(argv=None):
                           flush=True)
             wl.set_tuning("stencil_zchunk", 0)
         elif name == "gemm":
-            n = 4096
-            a = torch.randn(n, n, device=dev).to(torch.bfloat16)
-            b = torch.randn(n, n, device=dev).to(torch.bfloat16)
-            c = torch.empty(n, n, device=dev)
-            ms = _time(lambda: wl.gemm_bf16(a, b, c), args.steps)
-            print(f"gemm       variant 0  {ms:9.4f} ms  {2.0 * n ** 3 / ms / 1e9:8.1f} TFLOP/s", flush=True)
+            # every variant at 4096^3 and 8192^3, torch.matmul (hipBLASLt) on the same tensors beside them
+            for n in (4096, 8192):
+                a = torch.randn(n, n, device=dev).to(torch.bfloat16)
+                b = torch.randn(n, n, device=dev).to(torch.bfloat16)
+                c = torch.empty(n, n, device=dev)
+                for v in range(1, wl.num_variants(wl.GEMM)):
+                    ms = _time(lambda: wl.gemm_bf16(a, b, c, v), args.steps, settle_ms=10.0)
+                    print(f"gemm {n}^3  variant {v}  {ms:9.4f} ms  {2.0 * n ** 3 / ms / 1e9:8.1f} TFLOP/s", flush=True)
+                ms = _time(lambda: torch.matmul(a, b), args.steps, settle_ms=10.0)
+                print(f"gemm {n}^3  torch.matmul  {ms:9.4f} ms  {2.0 * n ** 3 / ms / 1e9:8.1f} TFLOP/s", flush=True)
+                del a, b, c
         elif name == "perf_sequential":
             # src/perf/sequential/param_sweep.py:27-58: element size x DMA wavefronts x workgroups per CU x
             # buffering; a launch reads 1 GiB whatever the point (loop count follows from that)
