@@ -30,6 +30,9 @@ SETTLE_MS = 30.0                # wall time of untimed warm-up for the secondary
 # scaled by what the same counters read for the plain copy kernel (see profiles/).
 # profiles/bench_all_patterns_mi355x.md: FETCH_SIZE 524328 KiB x 1.99996 + WRITE_SIZE 1048598 KiB x 1.00000.
 MEASURED_TRAFFIC_BYTES = {"strided": 2147566719}
+# Matrix-core occupancy of the two GEMM kernels from rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_BUSY_CU_CYCLES
+# (busy cycles / 4 SIMDs / busy cycles per compute unit), same file.
+MEASURED_MFMA_BUSY = {"gemm": 0.744, "gemm_warp_specialised": 0.579}
 STRIDED_VARIANT = 1             # cudadma_strided_transpose variant timed as the headline
 
 
@@ -237,10 +240,12 @@ def main():
                         "(global_load_lds) from the same four wavefronts that multiply (v_mfma_f32_32x32x16_bf16, "
                         "128x128 per wavefront), one load between every four matrix instructions"}
     ms_ws, _ = time_launches(lambda: wl.gemm_bf16(ga, gb, gc, 7), max(steps, 50), warmup, SETTLE_MS)
+    gemm["mfma_busy_from_counters"] = MEASURED_MFMA_BUSY["gemm"]
     gemm["note"] = ("config 5 names the warp-specialised kernel: it is reported under warp_specialised; the figures at "
                     "this level are the form of the same objects that is not warp-specialised, the faster one")
     gemm["warp_specialised"] = {"TFLOP/s": round(flops / ms_ws / 1e9, 1),
                                 "frac_of_mfma_peak": round(flops / ms_ws / 1e9 / 2500.0, 4), "ms": round(ms_ws, 4),
+                                "mfma_busy_from_counters": MEASURED_MFMA_BUSY["gemm_warp_specialised"],
                                 "workload": "the same tile with four DMA wavefronts feeding eight compute wavefronts "
                                             "(128x64 per wavefront), variant 7"}
     log(f"gemm         {ms:9.4f} ms  {gemm['TFLOP/s']:8.1f} TFLOP/s  {100 * gemm['frac_of_mfma_peak']:5.1f}% of 2.5 PFLOP/s")
