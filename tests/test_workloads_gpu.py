@@ -305,7 +305,7 @@ def _bf16_inputs(m, n, k):
 
 @pytest.mark.parametrize("variant", range(10))
 @pytest.mark.parametrize("shape", [(128, 128, 128), (256, 384, 256), (512, 512, 512), (768, 256, 384), (256, 128, 128),
-                                   (1024, 256, 896), (256, 256, 128), (256, 512, 640)])
+                                   (1024, 256, 896), (256, 256, 128), (256, 512, 640), (768, 1280, 640)])
 def test_gemm_small(device, shape, variant):
     m, n, k = shape
     tile_m, tile_n = {0: (128, 128), 1: (128, 128), 2: (128, 256), 3: (256, 128), 4: (256, 128), 5: (256, 256), 6: (256, 256), 7: (256, 256), 8: (256, 256), 9: (256, 256)}[variant]
