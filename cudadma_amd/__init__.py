@@ -8,6 +8,10 @@ not been built: there is no CPU fallback.
 """
 from ._lib import (  # noqa: F401
     CALL_GLOBAL,
+    CALL_LDS_DIRECT_NT,
+    CALL_LDS_DIRECT_SC1,
+    CALL_MATRIX_GENERIC,
+    CALL_MATRIX_GLOBAL,
     CALL_LDS_DIRECT,
     CALL_LDS_DIRECT_SWIZZLE,
     CALL_LDS_SWIZZLE,
@@ -22,7 +26,9 @@ from ._lib import (  # noqa: F401
     CudaDMAError,
     PlanQuery,
     RunArgs,
+    STATUS_WAIT_GAVE_UP,
     V1Case,
+    device_status,
     lib,
     lib_path,
 )

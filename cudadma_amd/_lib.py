@@ -5,7 +5,14 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
 PATTERN_SEQUENTIAL, PATTERN_STRIDED, PATTERN_GATHER, PATTERN_SCATTER, PATTERN_HALO = range(5)
-CALL_UNQUALIFIED, CALL_GLOBAL, CALL_QUALIFIED, CALL_LDS_DIRECT, CALL_LDS_SWIZZLE, CALL_LDS_DIRECT_SWIZZLE = range(6)
+(CALL_UNQUALIFIED, CALL_GLOBAL, CALL_QUALIFIED, CALL_LDS_DIRECT, CALL_LDS_SWIZZLE, CALL_LDS_DIRECT_SWIZZLE,
+ CALL_Q_GLOBAL_CG, CALL_Q_LASTUSE_CS, CALL_Q_VOLATILE_WT, CALL_Q_STREAMING_WB,
+ CALL_QG_GLOBAL_CS, CALL_QG_STREAMING_WT, CALL_QG_LASTUSE_CG, CALL_QG_VOLATILE_WB,
+ CALL_LDS_DIRECT_SC1, CALL_LDS_DIRECT_NT) = range(16)
+# the qualifier matrix: source known to be global / generic source (the latter also run LDS -> global)
+STATUS_WAIT_GAVE_UP = 1
+CALL_MATRIX_GLOBAL = (CALL_Q_GLOBAL_CG, CALL_Q_LASTUSE_CS, CALL_Q_VOLATILE_WT, CALL_Q_STREAMING_WB)
+CALL_MATRIX_GENERIC = (CALL_QG_GLOBAL_CS, CALL_QG_STREAMING_WT, CALL_QG_LASTUSE_CG, CALL_QG_VOLATILE_WB)
 
 PATTERN_NAMES = {
     PATTERN_SEQUENTIAL: "sequential",
@@ -41,7 +48,8 @@ class PlanQuery(ctypes.Structure):
     """struct cudadma_plan_query"""
     _fields_ = [(n, ctypes.c_int) for n in (
         "pattern", "alignment", "bytes_per_thread", "bytes_per_elmt", "dma_threads", "num_elmts",
-        "src_stride", "dst_stride", "radius", "corners", "dimx", "dimy", "pitch")] + [("index", ctypes.c_void_p)]
+        "src_stride", "dst_stride", "radius", "corners", "dimx", "dimy", "pitch")] + [("index", ctypes.c_void_p),
+                                                                                       ("dst_pitch", ctypes.c_int)]
 
 
 class RunArgs(ctypes.Structure):
@@ -55,6 +63,8 @@ class RunArgs(ctypes.Structure):
         ("reverse", ctypes.c_int), ("out_bytes", ctypes.c_int),
         ("rt_bytes_per_elmt", ctypes.c_int), ("rt_dma_threads", ctypes.c_int), ("rt_num_elmts", ctypes.c_int),
         ("rt_dimx", ctypes.c_int), ("rt_dimy", ctypes.c_int),
+        ("dst_pitch", ctypes.c_int),
+        ("in_bytes", ctypes.c_size_t), ("out_capacity", ctypes.c_size_t), ("index_elmts", ctypes.c_int),
     ]
 
 
@@ -92,6 +102,8 @@ def lib():
     L.cudadma_plan_map.restype = ci
     L.cudadma_plan_map.argtypes = [ctypes.POINTER(PlanQuery), ctypes.c_longlong, ctypes.c_longlong, vp, cs,
                                    ctypes.POINTER(ci)]
+    L.cudadma_plan_extents.restype = ci
+    L.cudadma_plan_extents.argtypes = [ctypes.POINTER(PlanQuery), ctypes.POINTER(ctypes.c_longlong * 4)]
     L.cudadma_diagnose.restype = ci
     L.cudadma_diagnose.argtypes = [ci] * 8
     L.cudadma_set_tuning.restype = ci
@@ -118,6 +130,7 @@ _vp, _ci, _cs, _u64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_u
 _WORKLOAD_SIGNATURES = {
     "cudadma_fill_uniform": [_vp, _cs, _u64, _vp],
     "cudadma_fill_indices": [_vp, _cs, ctypes.c_uint32, _u64, _vp],
+    "cudadma_fill_normal_bf16": [_vp, _cs, _u64, _vp],
     "cudadma_plain_copy": [_vp, _vp, _cs, _vp],
     "cudadma_num_variants": [_ci],
     "cudadma_set_workgroups_per_cu": [_ci],
@@ -131,6 +144,10 @@ _WORKLOAD_SIGNATURES = {
     "cudadma_gemm_bf16": [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cudadma_selftest_bounded_wait": [_vp, _vp],
     "cudadma_selftest_split_wait": [_vp, _ci, _vp],
+    "cudadma_selftest_global_handoff": [_vp, _vp, _ci, _vp],
+    "cudadma_selftest_global_handoff_lds_only": [_vp, _vp, _ci, _vp],
+    "cudadma_device_status": [ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint), _ci, _vp],
+    "cudadma_device_status_sources": [],
     "cudadma_selftest_all_ids": [_vp, _ci, _vp],
     "cudadma_v1_num_cases": [],
     "cudadma_v1_run_case": [_ci, _vp, _vp, _vp, _vp],
@@ -146,8 +163,15 @@ def check(rc):
         raise CudaDMAError(f"libcudadma_amd error {rc}: {lib().cudadma_last_error().decode()}")
 
 
+def device_status(clear=True, stream=None):
+    """(status bits, wavefronts whose wait gave up) summed over the library's kernels since the last clear."""
+    bits, count = ctypes.c_uint(0), ctypes.c_uint(0)
+    check(lib().cudadma_device_status(ctypes.byref(bits), ctypes.byref(count), int(bool(clear)), ctypes.c_void_p(stream or 0)))
+    return bits.value, count.value
+
+
 def exported_symbols():
     """Every extern "C" symbol include/cudadma_amd.h declares."""
     return ["cudadma_last_error", "cudadma_device_cus", "cudadma_num_cases", "cudadma_get_case",
             "cudadma_run_case", "cudadma_variant_name", "cudadma_example_variant_name",
-            "cudadma_v1_get_case", "cudadma_v1_case_text", "cudadma_perf_sequential", "cudadma_probe_memory", "cudadma_plan_map", "cudadma_diagnose", "cudadma_set_tuning"] + list(_WORKLOAD_SIGNATURES)
+            "cudadma_v1_get_case", "cudadma_v1_case_text", "cudadma_perf_sequential", "cudadma_probe_memory", "cudadma_plan_map", "cudadma_plan_extents", "cudadma_diagnose", "cudadma_set_tuning"] + list(_WORKLOAD_SIGNATURES)

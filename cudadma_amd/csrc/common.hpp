@@ -29,4 +29,13 @@ void set_error(const char* fmt, ...);
 
 inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
+// The failure record of the DMA objects (hipdma::status_words_address in include/hipdma/base.hpp) exists once
+// per translation unit; status_word.hpp registers each unit's accessor here so that cudadma_device_status()
+// can read them all.  Called from static initialisers only.
+typedef hipError_t (*status_address_fn)(unsigned** words);
+void register_status_source(status_address_fn fn, const char* file);
+struct StatusRegistrar {
+  StatusRegistrar(status_address_fn fn, const char* file) { register_status_source(fn, file); }
+};
+
 }  // namespace cudadma_host

@@ -132,8 +132,10 @@ def write(name, lines):
     path = os.path.join(HERE, name)
     with open(path, "w") as f:
         f.write("// Generated by gen_cases.py; do not edit.\n")
-        for line in lines:
-            f.write(line + "\n")
+        f.write("// A harness source is compiled in HARNESS_SHARDS pieces (see the Makefile): piece HARNESS_SHARD\n")
+        f.write("// holds the cases whose number leaves that remainder.\n")
+        for i, line in enumerate(lines):
+            f.write(f"#if ({i} % HARNESS_SHARDS) == HARNESS_SHARD\n{line}\n#endif\n")
     print(f"{name}: {len(lines)} cases")
 
 

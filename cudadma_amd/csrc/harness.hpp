@@ -10,6 +10,14 @@
 
 #include "common.hpp"
 #include "../../include/hipDMA.h"
+#include "status_word.hpp"
+
+// The case lists are long and every case is a pair of kernels with a dozen call styles inlined: the Makefile
+// compiles each harness source HARNESS_SHARDS times, piece HARNESS_SHARD taking every HARNESS_SHARDS-th case.
+#ifndef HARNESS_SHARDS
+#define HARNESS_SHARDS 1
+#define HARNESS_SHARD 0
+#endif
 
 namespace harness {
 
@@ -28,6 +36,7 @@ struct Args {
   int reverse, out_bytes;
   // run-time copies of the template parameters, fed to the constructors of the lower levels
   int bytes_per_elmt, dma_threads, num_elmts, dimx, dimy;
+  int dst_pitch;       // halo: destination row pitch in cells, 0 = dimx + 2*radius
 };
 
 typedef int (*launch_fn)(const Args&, hipStream_t);
@@ -88,6 +97,65 @@ __device__ __forceinline__ void do_transfer_indexed(Obj& dma, const int call_sty
       dma.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_WRITE_BACK>(index, src);
       dma.template wait_xfer_finish<true, LOAD_CACHE_STREAMING, STORE_WRITE_BACK>(dst);
     } else dma.template execute_dma<true, LOAD_CACHE_STREAMING, STORE_WRITE_BACK>(index, src, dst);
+  }
+}
+
+// The qualifier matrix (enums of include/cudaDMAv2.h:50-63; the reference's tests run an assortment of the
+// combinations, src/tests/test_strided/cudaDMA_test_strided_v2.cu:693-812): every load qualifier once with a
+// source known to be global and once with a generic source, every store qualifier of the reference at least
+// twice, and the direct-to-LDS path with a load qualifier.  The kernels of these styles are instantiated
+// apart from those of the first six (template parameter MATRIX of the case kernels) to keep each kernel small.
+template<bool GL, int LQ, int SQ, typename Obj>
+__device__ __forceinline__ void transfer_as(Obj& dma, const int two_phase, const void* src, void* dst)
+{
+  if (two_phase) {
+    dma.template start_xfer_async<GL, LQ, SQ>(src);
+    dma.template wait_xfer_finish<GL, LQ, SQ>(dst);
+  } else dma.template execute_dma<GL, LQ, SQ>(src, dst);
+}
+template<bool GL, int LQ, int SQ, typename Obj>
+__device__ __forceinline__ void transfer_indexed_as(Obj& dma, const int two_phase, const int* index, const void* src, void* dst)
+{
+  if (two_phase) {
+    dma.template start_xfer_async<GL, LQ, SQ>(index, src);
+    dma.template wait_xfer_finish<GL, LQ, SQ>(dst);
+  } else dma.template execute_dma<GL, LQ, SQ>(index, src, dst);
+}
+
+// DIRECT: the object has a direct-to-LDS path for this case (otherwise the two direct styles are left out).
+#define HARNESS_QUALIFIER_MATRIX(CALL, ...)                                                                              \
+  switch (call_style) {                                                                                                  \
+    case CUDADMA_CALL_Q_GLOBAL_CG:     CALL<true, LOAD_CACHE_GLOBAL, STORE_CACHE_GLOBAL>(__VA_ARGS__); break;            \
+    case CUDADMA_CALL_Q_LASTUSE_CS:    CALL<true, LOAD_CACHE_LAST_USE, STORE_CACHE_STREAMING>(__VA_ARGS__); break;       \
+    case CUDADMA_CALL_Q_VOLATILE_WT:   CALL<true, LOAD_CACHE_VOLATILE, STORE_CACHE_WRITE_THROUGH>(__VA_ARGS__); break;   \
+    case CUDADMA_CALL_Q_STREAMING_WB:  CALL<true, LOAD_CACHE_STREAMING, STORE_WRITE_BACK>(__VA_ARGS__); break;           \
+    case CUDADMA_CALL_QG_GLOBAL_CS:    CALL<false, LOAD_CACHE_GLOBAL, STORE_CACHE_STREAMING>(__VA_ARGS__); break;        \
+    case CUDADMA_CALL_QG_STREAMING_WT: CALL<false, LOAD_CACHE_STREAMING, STORE_CACHE_WRITE_THROUGH>(__VA_ARGS__); break; \
+    case CUDADMA_CALL_QG_LASTUSE_CG:   CALL<false, LOAD_CACHE_LAST_USE, STORE_CACHE_GLOBAL>(__VA_ARGS__); break;         \
+    case CUDADMA_CALL_QG_VOLATILE_WB:  CALL<false, LOAD_CACHE_VOLATILE, STORE_WRITE_BACK>(__VA_ARGS__); break;           \
+    default: break;                                                                                                      \
+  }
+
+template<bool DIRECT, typename Obj>
+__device__ __forceinline__ void do_transfer_matrix(Obj& dma, const int call_style, const int two_phase,
+                                                   const void* src, void* dst)
+{
+  HARNESS_QUALIFIER_MATRIX(transfer_as, dma, two_phase, src, dst)
+  if constexpr (DIRECT) {
+    if (call_style == CUDADMA_CALL_LDS_DIRECT_SC1) transfer_as<true, LOAD_CACHE_GLOBAL, STORE_LDS_DIRECT>(dma, two_phase, src, dst);
+    else if (call_style == CUDADMA_CALL_LDS_DIRECT_NT) transfer_as<true, LOAD_CACHE_STREAMING, STORE_LDS_DIRECT>(dma, two_phase, src, dst);
+  }
+}
+template<bool DIRECT, typename Obj>
+__device__ __forceinline__ void do_transfer_indexed_matrix(Obj& dma, const int call_style, const int two_phase,
+                                                           const int* index, const void* src, void* dst)
+{
+  HARNESS_QUALIFIER_MATRIX(transfer_indexed_as, dma, two_phase, index, src, dst)
+  if constexpr (DIRECT) {
+    if (call_style == CUDADMA_CALL_LDS_DIRECT_SC1)
+      transfer_indexed_as<true, LOAD_CACHE_GLOBAL, STORE_LDS_DIRECT>(dma, two_phase, index, src, dst);
+    else if (call_style == CUDADMA_CALL_LDS_DIRECT_NT)
+      transfer_indexed_as<true, LOAD_CACHE_STREAMING, STORE_LDS_DIRECT>(dma, two_phase, index, src, dst);
   }
 }
 
@@ -155,11 +223,15 @@ __device__ __forceinline__ void run_body(Obj& dma, const Args& a, unsigned* lds,
   }
 }
 
+inline bool is_matrix_style(const int call_style) { return call_style >= CUDADMA_CALL_Q_GLOBAL_CG; }
+
+// `kernel` runs the first six call styles, `matrix_kernel` the qualifier matrix.
 template<typename Kernel>
-int launch_case(Kernel kernel, const bool ws, const Args& a, hipStream_t stream)
+int launch_case(Kernel kernel, Kernel matrix_kernel, const bool ws, const Args& a, hipStream_t stream)
 {
   const int threads = ws ? (kComputeThreads + a.dma_threads) : a.dma_threads;
-  hipLaunchKernelGGL(kernel, dim3(1), dim3(threads), (size_t)a.lds_bytes, stream, a);
+  hipLaunchKernelGGL(is_matrix_style(a.call_style) ? matrix_kernel : kernel, dim3(1), dim3(threads), (size_t)a.lds_bytes,
+                     stream, a);
   CUDADMA_HIP_CHECK(hipGetLastError());
   return CUDADMA_OK;
 }

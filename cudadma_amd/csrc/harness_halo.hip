@@ -23,32 +23,32 @@ template<int A, int BPT, int ES, int T, int R, bool C, int DX, int DY> struct Ma
 template<int A, int BPT, int ES, int T, int R, bool C, int DX, int DY> struct Make<true, 1, A, BPT, ES, T, R, C, DX, DY> {
   typedef CudaDMAHalo<true, A, BPT, ES, 0, R, C> type;
   static __device__ __forceinline__ type make(const Args& a)
-  { return type(1, a.dma_threads, kComputeThreads, kComputeThreads, a.dimx, a.dimy, a.pitch); }
+  { return type(1, a.dma_threads, kComputeThreads, kComputeThreads, a.dimx, a.dimy, a.pitch, a.dst_pitch); }
 };
 template<int A, int BPT, int ES, int T, int R, bool C, int DX, int DY> struct Make<true, 2, A, BPT, ES, T, R, C, DX, DY> {
   typedef CudaDMAHalo<true, A, BPT, ES, T, R, C> type;
   static __device__ __forceinline__ type make(const Args& a)
-  { return type(2, kComputeThreads, kComputeThreads, a.dimx, a.dimy, a.pitch); }
+  { return type(2, kComputeThreads, kComputeThreads, a.dimx, a.dimy, a.pitch, a.dst_pitch); }
 };
 template<int A, int BPT, int ES, int T, int R, bool C, int DX, int DY> struct Make<true, 3, A, BPT, ES, T, R, C, DX, DY> {
   typedef CudaDMAHalo<true, A, BPT, ES, T, R, C, DX, DY> type;
   static __device__ __forceinline__ type make(const Args& a)
-  { return type(3, kComputeThreads, kComputeThreads, a.pitch); }
+  { return type(3, kComputeThreads, kComputeThreads, a.pitch, a.dst_pitch); }
 };
 template<int A, int BPT, int ES, int T, int R, bool C, int DX, int DY> struct Make<false, 1, A, BPT, ES, T, R, C, DX, DY> {
   typedef CudaDMAHalo<false, A, BPT, ES, 0, R, C> type;
-  static __device__ __forceinline__ type make(const Args& a) { return type(a.dimx, a.dimy, a.pitch); }
+  static __device__ __forceinline__ type make(const Args& a) { return type(a.dimx, a.dimy, a.pitch, 0, 0, a.dst_pitch); }
 };
 template<int A, int BPT, int ES, int T, int R, bool C, int DX, int DY> struct Make<false, 2, A, BPT, ES, T, R, C, DX, DY> {
   typedef CudaDMAHalo<false, A, BPT, ES, T, R, C> type;
-  static __device__ __forceinline__ type make(const Args& a) { return type(a.dimx, a.dimy, a.pitch); }
+  static __device__ __forceinline__ type make(const Args& a) { return type(a.dimx, a.dimy, a.pitch, 0, a.dst_pitch); }
 };
 template<int A, int BPT, int ES, int T, int R, bool C, int DX, int DY> struct Make<false, 3, A, BPT, ES, T, R, C, DX, DY> {
   typedef CudaDMAHalo<false, A, BPT, ES, T, R, C, DX, DY> type;
-  static __device__ __forceinline__ type make(const Args& a) { return type(a.pitch); }
+  static __device__ __forceinline__ type make(const Args& a) { return type(a.pitch, 0, a.dst_pitch); }
 };
 
-template<bool WS, int LEVEL, int A, int BPT, int ES, int T, int R, bool C, int DX, int DY>
+template<bool WS, int LEVEL, int A, int BPT, int ES, int T, int R, bool C, int DX, int DY, bool MATRIX>
 __global__ void __launch_bounds__(1024) halo_kernel(const Args a)
 {
   extern __shared__ __attribute__((aligned(16))) unsigned lds[];
@@ -56,15 +56,17 @@ __global__ void __launch_bounds__(1024) halo_kernel(const Args a)
   harness::run_body<WS>(dma, a, lds, [&](const int rep) __attribute__((always_inline)) {
     const char* src = (a.reverse ? (const char*)lds + a.src_offset : a.in + a.src_offset + (size_t)rep * a.rep_src_bytes) +
                       (size_t)(R * a.pitch + R) * ES;
+    const int dst_pitch = a.dst_pitch > 0 ? a.dst_pitch : a.dimx + 2 * R;
     char* dst = (a.reverse ? a.out + (size_t)rep * a.out_bytes + a.dst_offset : (char*)lds + a.dst_offset) +
-                (size_t)(R * (a.dimx + 2 * R) + R) * ES;
-    harness::do_transfer(dma, a.call_style, a.two_phase, src, dst);
+                (size_t)(R * dst_pitch + R) * ES;
+    if constexpr (MATRIX) harness::do_transfer_matrix<false>(dma, a.call_style, a.two_phase, src, dst);
+    else harness::do_transfer(dma, a.call_style, a.two_phase, src, dst);
   });
 }
 
 template<bool WS, int LEVEL, int A, int BPT, int ES, int T, int R, bool C, int DX, int DY>
 int launch(const Args& a, hipStream_t s)
-{ return harness::launch_case(halo_kernel<WS, LEVEL, A, BPT, ES, T, R, C, DX, DY>, WS, a, s); }
+{ return harness::launch_case(halo_kernel<WS, LEVEL, A, BPT, ES, T, R, C, DX, DY, false>, halo_kernel<WS, LEVEL, A, BPT, ES, T, R, C, DX, DY, true>, WS, a, s); }
 
 #define HALO_CASE(ORDER, WS, LEVEL, A, BPT, ES, T, R, C, DX, DY)                                          \
   static harness::Registrar reg_halo_##ORDER(                                                              \

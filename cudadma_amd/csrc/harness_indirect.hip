@@ -49,7 +49,7 @@ template<bool G, int A, int BPT, int E, int T, int N> struct Make<G, false, 4, A
   static __device__ __forceinline__ type make(const Args& a) { return type(alt_stride<G>(a)); }
 };
 
-template<bool G, bool WS, int LEVEL, int A, int BPT, int E, int T, int N>
+template<bool G, bool WS, int LEVEL, int A, int BPT, int E, int T, int N, bool MATRIX>
 __global__ void __launch_bounds__(1024) indirect_kernel(const Args a)
 {
   extern __shared__ __attribute__((aligned(16))) unsigned lds[];
@@ -58,7 +58,9 @@ __global__ void __launch_bounds__(1024) indirect_kernel(const Args a)
     const char* src = a.reverse ? (const char*)lds + a.src_offset : a.in + a.src_offset + (size_t)rep * a.rep_src_bytes;
     const int* index = a.index + (size_t)rep * a.rep_index_elmts;
     char* dst = a.reverse ? a.out + (size_t)rep * a.out_bytes + a.dst_offset : (char*)lds + a.dst_offset;
-    if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
+    if constexpr (MATRIX) {
+      harness::do_transfer_indexed_matrix<(G && (A == 16 || A == 4))>(dma, a.call_style, a.two_phase, index, src, dst);
+    } else if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
       if constexpr (G && (A == 16 || A == 4)) {
         if (a.two_phase) {
           dma.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS_DIRECT>(index, src);
@@ -75,7 +77,7 @@ __global__ void __launch_bounds__(1024) indirect_kernel(const Args a)
 
 template<bool G, bool WS, int LEVEL, int A, int BPT, int E, int T, int N>
 int launch(const Args& a, hipStream_t s)
-{ return harness::launch_case(indirect_kernel<G, WS, LEVEL, A, BPT, E, T, N>, WS, a, s); }
+{ return harness::launch_case(indirect_kernel<G, WS, LEVEL, A, BPT, E, T, N, false>, indirect_kernel<G, WS, LEVEL, A, BPT, E, T, N, true>, WS, a, s); }
 
 #define INDIRECT_CASE(ORDER, G, WS, LEVEL, A, BPT, E, T, N)                                              \
   static harness::Registrar reg_indirect_##ORDER(                                                         \

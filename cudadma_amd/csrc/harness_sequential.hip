@@ -34,7 +34,7 @@ template<int A, int BPT, int E, int T> struct Make<false, 3, A, BPT, E, T> {
   static __device__ __forceinline__ type make(const Args&) { return type(); }
 };
 
-template<bool WS, int LEVEL, int A, int BPT, int E, int T>
+template<bool WS, int LEVEL, int A, int BPT, int E, int T, bool MATRIX>
 __global__ void __launch_bounds__(1024) seq_kernel(const Args a)
 {
   extern __shared__ __attribute__((aligned(16))) unsigned lds[];
@@ -42,7 +42,9 @@ __global__ void __launch_bounds__(1024) seq_kernel(const Args a)
   harness::run_body<WS>(dma, a, lds, [&](const int rep) __attribute__((always_inline)) {
     const char* src = a.reverse ? (const char*)lds + a.src_offset : a.in + a.src_offset + (size_t)rep * a.rep_src_bytes;
     char* dst = a.reverse ? a.out + (size_t)rep * a.out_bytes + a.dst_offset : (char*)lds + a.dst_offset;
-    if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
+    if constexpr (MATRIX) {
+      harness::do_transfer_matrix<(A == 16 || A == 4)>(dma, a.call_style, a.two_phase, src, dst);
+    } else if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
       if constexpr (A == 16 || A == 4) harness::do_transfer_direct(dma, a.two_phase, src, dst);
     } else {
       harness::do_transfer(dma, a.call_style, a.two_phase, src, dst);
@@ -51,7 +53,8 @@ __global__ void __launch_bounds__(1024) seq_kernel(const Args a)
 }
 
 template<bool WS, int LEVEL, int A, int BPT, int E, int T>
-int launch(const Args& a, hipStream_t s) { return harness::launch_case(seq_kernel<WS, LEVEL, A, BPT, E, T>, WS, a, s); }
+int launch(const Args& a, hipStream_t s)
+{ return harness::launch_case(seq_kernel<WS, LEVEL, A, BPT, E, T, false>, seq_kernel<WS, LEVEL, A, BPT, E, T, true>, WS, a, s); }
 
 #define SEQ_CASE(ORDER, WS, LEVEL, A, BPT, E, T)                                                         \
   static harness::Registrar reg_seq_##ORDER(                                                              \

@@ -99,7 +99,7 @@ __device__ __forceinline__ void direct_transfer(Obj& dma, const int two_phase, c
   }
 }
 
-template<bool WS, int LEVEL, bool ONE, int A, int BPT, int E, int T, int N>
+template<bool WS, int LEVEL, bool ONE, int A, int BPT, int E, int T, int N, bool MATRIX>
 __global__ void __launch_bounds__(1024) strided_kernel(const Args a)
 {
   extern __shared__ __attribute__((aligned(16))) unsigned lds[];
@@ -110,7 +110,9 @@ __global__ void __launch_bounds__(1024) strided_kernel(const Args a)
   harness::run_body<WS>(dma, a, lds, [&](const int rep) __attribute__((always_inline)) {
     const char* src = a.reverse ? (const char*)lds + a.src_offset : a.in + a.src_offset + (size_t)rep * a.rep_src_bytes;
     char* dst = a.reverse ? a.out + (size_t)rep * a.out_bytes + a.dst_offset : (char*)lds + a.dst_offset;
-    if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
+    if constexpr (MATRIX) {
+      harness::do_transfer_matrix<(A == 16 || A == 4)>(dma, a.call_style, a.two_phase, src, dst);
+    } else if (a.call_style == CUDADMA_CALL_LDS_DIRECT) {
       if constexpr (A == 16 || A == 4) direct_transfer<WS, STORE_LDS_DIRECT>(dma, a.two_phase, src, dst, rep);
     } else if (a.call_style == CUDADMA_CALL_LDS_SWIZZLE) {
       if constexpr (kWholeChunks) harness::do_transfer_direct<STORE_LDS_SWIZZLE>(dma, a.two_phase, src, dst);
@@ -130,7 +132,7 @@ int launch(const Args& a, hipStream_t s)
     cudadma_host::set_error("this case was built with the single-stride constructor: src_stride must equal dst_stride");
     return CUDADMA_EINVAL;
   }
-  return harness::launch_case(strided_kernel<WS, LEVEL, ONE, A, BPT, E, T, N>, WS, a, s);
+  return harness::launch_case(strided_kernel<WS, LEVEL, ONE, A, BPT, E, T, N, false>, strided_kernel<WS, LEVEL, ONE, A, BPT, E, T, N, true>, WS, a, s);
 }
 
 // dimx carries the ONE_STRIDE flag in the case description.

@@ -7,13 +7,22 @@
 namespace {
 
 struct MapWriter {
-  int* map;
+  int* map;               // NULL: only the extents are recorded
   size_t len;
   long long src_origin, dst_origin;
   int doubles;
   bool out_of_range;
+  bool any = false;
+  long long src_min = 0, src_end = 0, dst_min = 0, dst_end = 0;
   void move(long long src_off, long long dst_off, int nbytes)
   {
+    if (nbytes <= 0) return;
+    if (!any) { src_min = src_off; src_end = src_off + nbytes; dst_min = dst_off; dst_end = dst_off + nbytes; any = true; }
+    if (src_off < src_min) src_min = src_off;
+    if (src_off + nbytes > src_end) src_end = src_off + nbytes;
+    if (dst_off < dst_min) dst_min = dst_off;
+    if (dst_off + nbytes > dst_end) dst_end = dst_off + nbytes;
+    if (map == nullptr) return;
     for (int b = 0; b < nbytes; ++b) {
       const long long d = dst_origin + dst_off + b;
       if (d < 0 || (size_t)d >= len) { out_of_range = true; return; }
@@ -78,7 +87,7 @@ int replay_halo_t(const cudadma_plan_query_t& q, MapWriter& w, int* steps)
 {
   if ((2 * R * ES) % A != 0) return CUDADMA_EINVAL;
   hipdma::detail::HaloGeom<A, ES, R, C> g;
-  g.init(q.dimx, q.dimy, q.pitch);
+  g.init(q.dimx, q.dimy, q.pitch, q.dst_pitch);
   const int max_lds = q.bytes_per_thread / A;
   const int nsteps = hipdma::detail::ceil_div(hipdma::detail::ceil_div(g.total, q.dma_threads), max_lds);
   for (int tid = 0; tid < q.dma_threads; ++tid)
@@ -123,17 +132,18 @@ int replay_halo_es(const cudadma_plan_query_t& q, MapWriter& w, int* steps)
 
 }  // namespace
 
-extern "C" int cudadma_plan_map(const cudadma_plan_query_t* q, long long src_origin, long long dst_origin,
-                                int* map, size_t map_len, int* steps_out)
+// Replays the query into `w`; shared by cudadma_plan_map and cudadma_plan_extents.
+static int replay(const cudadma_plan_query_t* q, MapWriter& w, int* steps_out)
 {
-  CUDADMA_REQUIRE(q != nullptr && map != nullptr, "NULL argument");
   CUDADMA_REQUIRE(q->alignment == 4 || q->alignment == 8 || q->alignment == 16, "ALIGNMENT must be 4, 8 or 16");
   CUDADMA_REQUIRE(q->bytes_per_thread >= q->alignment && (q->bytes_per_thread % q->alignment) == 0,
                   "BYTES_PER_THREAD must be a positive multiple of ALIGNMENT");
   CUDADMA_REQUIRE(q->dma_threads > 0, "DMA_THREADS must be positive");
   CUDADMA_REQUIRE(q->bytes_per_elmt >= 0 && (q->bytes_per_elmt % 4) == 0, "sizes are multiples of 4 bytes");
-  for (size_t i = 0; i < map_len; ++i) map[i] = -1;
-  MapWriter w{map, map_len, src_origin, dst_origin, 0, false};
+  if (q->pattern == CUDADMA_PATTERN_HALO)
+    CUDADMA_REQUIRE(q->dimx > 0 && q->dimy > 0 && q->pitch >= q->dimx + 2 * q->radius &&
+                    (q->dst_pitch == 0 || q->dst_pitch >= q->dimx + 2 * q->radius),
+                    "halo: dimx, dimy positive, both pitches at least dimx + 2*radius");
   int steps = 0, rc = 0;
   switch (q->pattern) {
     case CUDADMA_PATTERN_SEQUENTIAL: rc = replay_sequential(*q, w, &steps); break;
@@ -152,12 +162,33 @@ extern "C" int cudadma_plan_map(const cudadma_plan_query_t* q, long long src_ori
     cudadma_host::set_error("plan replay rejected the query (pattern %d)", q->pattern);
     return rc;
   }
+  if (steps_out != nullptr) *steps_out = steps;
+  return CUDADMA_OK;
+}
+
+extern "C" int cudadma_plan_map(const cudadma_plan_query_t* q, long long src_origin, long long dst_origin,
+                                int* map, size_t map_len, int* steps_out)
+{
+  CUDADMA_REQUIRE(q != nullptr && map != nullptr, "NULL argument");
+  for (size_t i = 0; i < map_len; ++i) map[i] = -1;
+  MapWriter w{map, map_len, src_origin, dst_origin, 0, false};
+  const int rc = replay(q, w, steps_out);
+  if (rc != 0) return rc;
   if (w.out_of_range) {
     cudadma_host::set_error("plan replay: a thread steps outside the %zu-byte destination window", map_len);
     return CUDADMA_ERANGE;
   }
-  if (steps_out != nullptr) *steps_out = steps;
   return w.doubles;
+}
+
+extern "C" int cudadma_plan_extents(const cudadma_plan_query_t* q, long long extents[4])
+{
+  CUDADMA_REQUIRE(q != nullptr && extents != nullptr, "NULL argument");
+  MapWriter w{nullptr, 0, 0, 0, 0, false};
+  const int rc = replay(q, w, nullptr);
+  if (rc != 0) return rc;
+  extents[0] = w.src_min; extents[1] = w.src_end; extents[2] = w.dst_min; extents[3] = w.dst_end;
+  return CUDADMA_OK;
 }
 
 extern "C" int cudadma_diagnose(int pattern, int alignment, int bytes_per_thread, int bytes_per_elmt,

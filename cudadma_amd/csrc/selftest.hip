@@ -4,6 +4,7 @@
 #define HIPDMA_SPIN_LIMIT 256
 #include "common.hpp"
 #include "../../include/hipDMA.h"
+#include "status_word.hpp"
 
 namespace {
 

@@ -4,6 +4,7 @@
 // between two ids, or a lost count, shows up as a wrong token (the bounded wait turns a hang into one).
 #include "common.hpp"
 #include "../../include/hipDMA.h"
+#include "status_word.hpp"
 
 namespace {
 

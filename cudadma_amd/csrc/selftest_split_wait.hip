@@ -2,6 +2,7 @@
 // the bounded-wait test, which lowers the poll limit for its whole translation unit.
 #include "common.hpp"
 #include "../../include/hipDMA.h"
+#include "status_word.hpp"
 
 namespace {
 

@@ -4,6 +4,7 @@
 // was filled with a sentinel, and the whole window is copied out for comparison.
 #include "common.hpp"
 #include "../../include/cudaDMA.h"
+#include "status_word.hpp"
 
 namespace {
 

@@ -4,6 +4,7 @@
 
 #include "common.hpp"
 #include "../../include/hipDMA.h"
+#include "status_word.hpp"
 
 namespace workloads {
 

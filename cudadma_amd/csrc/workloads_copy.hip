@@ -171,6 +171,24 @@ fill_uniform_kernel(float* __restrict__ dst, const size_t n, const unsigned long
     dst[i] = (float)(workloads::hash32(seed, i) >> 8) * (1.0f / 8388608.0f) - 1.0f;
 }
 
+// normal(0,1) by Box-Muller on two hashes, in double precision, rounded to float and then to bf16 (nearest even):
+// the operations of the host statement in the same order.  Double-precision log, cos and sqrt may differ from the
+// host library's in their last bit; after the two roundings a difference survives in about one of 2^40 values.
+__global__ void __launch_bounds__(256)
+fill_normal_bf16_kernel(unsigned short* __restrict__ dst, const size_t n, const unsigned long long seed)
+{
+#pragma clang fp contract(off)
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const double u1 = ((double)(workloads::hash32(seed, 2ull * i) >> 8) + 1.0) / 16777216.0;
+    const double u2 = (double)(workloads::hash32(seed, 2ull * i + 1ull) >> 8) / 16777216.0;
+    const float v = (float)(sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925286766559 * u2));
+    unsigned u = __float_as_uint(v);
+    u += 0x7fffu + ((u >> 16) & 1u);          // the value is finite: u1 > 0
+    dst[i] = (unsigned short)(u >> 16);
+  }
+}
+
 __global__ void __launch_bounds__(256)
 fill_indices_kernel(int* __restrict__ dst, const size_t n, const unsigned n_records, const unsigned long long seed)
 {
@@ -221,6 +239,17 @@ extern "C" int cudadma_fill_uniform(float* d_dst, size_t n, uint64_t seed, void*
   if (n == 0) return CUDADMA_OK;
   const int grid = workloads::persistent_grid((long long)((n + 255) / 256), 8);
   hipLaunchKernelGGL(fill_uniform_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, d_dst, n,
+                     (unsigned long long)seed);
+  CUDADMA_HIP_CHECK(hipGetLastError());
+  return CUDADMA_OK;
+}
+
+extern "C" int cudadma_fill_normal_bf16(uint16_t* d_dst, size_t n, uint64_t seed, void* stream)
+{
+  CUDADMA_REQUIRE(d_dst != nullptr || n == 0, "d_dst is NULL");
+  if (n == 0) return CUDADMA_OK;
+  const int grid = workloads::persistent_grid((long long)((n + 255) / 256), 8);
+  hipLaunchKernelGGL(fill_normal_bf16_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, d_dst, n,
                      (unsigned long long)seed);
   CUDADMA_HIP_CHECK(hipGetLastError());
   return CUDADMA_OK;

@@ -53,6 +53,13 @@ def fill_uniform(out, seed):
     return out
 
 
+def fill_normal_bf16(out, seed):
+    """out: bfloat16 tensor; receives normal(0,1) values from the seeded generator (the GEMM inputs of config 5)."""
+    _need(out, torch.bfloat16, "out")
+    check(lib().cudadma_fill_normal_bf16(_p(out), out.numel(), seed, _stream()))
+    return out
+
+
 def fill_indices(out, n_records, seed):
     _need(out, torch.int32, "out")
     check(lib().cudadma_fill_indices(_p(out), out.numel(), n_records, seed, _stream()))

@@ -54,7 +54,22 @@ enum {
    * at position c ^ key(r) (hipdma::swizzled_chunk in include/hipdma/base.hpp: key = bit-reversed
    * low bits of the row number, as many bits as the row has aligned chunks, at most 256 bytes) */
   CUDADMA_CALL_LDS_SWIZZLE  = 4,  /* execute_dma<true,LOAD_CACHE_ALL,STORE_LDS_SWIZZLE>        */
-  CUDADMA_CALL_LDS_DIRECT_SWIZZLE = 5  /* execute_dma<true,LOAD_CACHE_ALL,STORE_LDS_DIRECT_SWIZZLE> */
+  CUDADMA_CALL_LDS_DIRECT_SWIZZLE = 5, /* execute_dma<true,LOAD_CACHE_ALL,STORE_LDS_DIRECT_SWIZZLE> */
+  /* The qualifier matrix (enums of include/cudaDMAv2.h:50-63): every load qualifier with a source known to be
+   * global (Q_) and with a generic source (QG_), every store qualifier of the reference.  The QG_ styles are also
+   * accepted with reverse = 1, where the store qualifier acts on global memory. */
+  CUDADMA_CALL_Q_GLOBAL_CG      = 6,   /* <true,  LOAD_CACHE_GLOBAL,    STORE_CACHE_GLOBAL>        */
+  CUDADMA_CALL_Q_LASTUSE_CS     = 7,   /* <true,  LOAD_CACHE_LAST_USE,  STORE_CACHE_STREAMING>     */
+  CUDADMA_CALL_Q_VOLATILE_WT    = 8,   /* <true,  LOAD_CACHE_VOLATILE,  STORE_CACHE_WRITE_THROUGH> */
+  CUDADMA_CALL_Q_STREAMING_WB   = 9,   /* <true,  LOAD_CACHE_STREAMING, STORE_WRITE_BACK>          */
+  CUDADMA_CALL_QG_GLOBAL_CS     = 10,  /* <false, LOAD_CACHE_GLOBAL,    STORE_CACHE_STREAMING>     */
+  CUDADMA_CALL_QG_STREAMING_WT  = 11,  /* <false, LOAD_CACHE_STREAMING, STORE_CACHE_WRITE_THROUGH> */
+  CUDADMA_CALL_QG_LASTUSE_CG    = 12,  /* <false, LOAD_CACHE_LAST_USE,  STORE_CACHE_GLOBAL>        */
+  CUDADMA_CALL_QG_VOLATILE_WB   = 13,  /* <false, LOAD_CACHE_VOLATILE,  STORE_WRITE_BACK>          */
+  /* the direct-to-LDS path with the load qualifier in the instruction's cache-policy bits */
+  CUDADMA_CALL_LDS_DIRECT_SC1   = 14,  /* <true,  LOAD_CACHE_GLOBAL,    STORE_LDS_DIRECT>          */
+  CUDADMA_CALL_LDS_DIRECT_NT    = 15,  /* <true,  LOAD_CACHE_STREAMING, STORE_LDS_DIRECT>          */
+  CUDADMA_CALL_STYLES           = 16
 };
 
 typedef struct cudadma_case {
@@ -89,8 +104,9 @@ typedef struct cudadma_run {
   int reverse;            /* 1: the object moves LDS -> global.  The workgroup first copies
                              lds_bytes from d_in (+ rep * rep_src_bytes) into LDS, the object then
                              moves from LDS + src_offset_bytes to d_out + rep * out_bytes +
-                             dst_offset_bytes.  Only CUDADMA_CALL_UNQUALIFIED (generic pointers on
-                             both sides, include/cudaDMAv2.h:107-114,553-558) makes sense here.   */
+                             dst_offset_bytes.  Needs generic pointers on both sides
+                             (include/cudaDMAv2.h:107-114,553-558): CUDADMA_CALL_UNQUALIFIED or one of
+                             the CUDADMA_CALL_QG_* styles.                                         */
   int out_bytes;          /* reverse only: bytes of d_out one rep may touch            */
   /* Other values for the parameters that the case's level hands to the constructor at run time
    * (0 keeps the case's own), so that one compiled case can be swept the way the reference's
@@ -101,6 +117,16 @@ typedef struct cudadma_run {
    *   rt_dimx, rt_dimy   levels 0-2 of halo
    * A value for a parameter that the case fixes at compile time is refused. */
   int rt_bytes_per_elmt, rt_dma_threads, rt_num_elmts, rt_dimx, rt_dimy;
+  /* halo: destination row pitch in cells handed to the constructor (0 = the reference's dimx + 2*radius,
+   * include/cudaDMA.h:3718-3719); at least dimx + 2*radius and a multiple of ALIGNMENT in bytes */
+  int dst_pitch;
+  /* Sizes of the caller's buffers, so that a wrong value above is refused on the host instead of turning
+   * into out-of-range accesses on the device: before the launch the transfer is replayed on the host with
+   * the device objects' own index arithmetic (gather / scatter: after copying the index list back), and
+   * the call fails with CUDADMA_ERANGE when any byte falls outside d_in, d_out or the LDS window. */
+  size_t in_bytes;        /* bytes readable at d_in                                        */
+  size_t out_capacity;    /* bytes writable at d_out: >= reps * (reverse ? out_bytes : lds_bytes) */
+  int index_elmts;        /* ints readable at d_index                                      */
 } cudadma_run_t;
 
 int cudadma_num_cases(void);
@@ -110,8 +136,30 @@ int cudadma_run_case(int case_id, const cudadma_run_t* run, void* stream);
 /* Failure handling of the handshake (the reference deadlocks on unbalanced calls,
  * include/cudaDMAv2.h:1329-1347): launches one workgroup whose DMA and compute threads wait for
  * signals that never come, with the poll limit lowered to 256.  Both sides must give up and the
- * kernel must end; d_flags[0] (DMA side) and d_flags[1] (compute side) are then 1. */
+ * kernel must end; d_flags[0] (DMA side) and d_flags[1] (compute side) are then 1 and
+ * cudadma_device_status() reports CUDADMA_STATUS_WAIT_GAVE_UP with a count of 2 wavefronts. */
 int cudadma_selftest_bounded_wait(int* d_flags, void* stream);
+
+/* The failure record of the handshake.  A wait that runs into the poll limit (HIPDMA_SPIN_LIMIT of
+ * include/hipdma/base.hpp; the reference's named barriers would hang instead, its DEBUG_CUDADMA build asserts,
+ * include/cudaDMAv2.h:1564-1576) lets its kernel finish and records the fact on the device.  This call waits
+ * for `stream` to drain and returns, summed over every kernel of the library that ran on the current device
+ * since the last clear: *status_bits = CUDADMA_STATUS_* bits, *waits_given_up = wavefronts whose wait gave up.
+ * clear != 0 resets the record.  Either pointer may be NULL.  Allocates nothing.  A non-zero record means the
+ * outputs of the kernels since the last clear are void. */
+#define CUDADMA_STATUS_WAIT_GAVE_UP 1u
+int cudadma_device_status(unsigned* status_bits, unsigned* waits_given_up, int clear, void* stream);
+/* Number of translation units whose record cudadma_device_status() reads. */
+int cudadma_device_status_sources(void);
+
+/* Global memory handed across the handshake in both directions (the reference's bar.sync / bar.arrive order
+ * all memory of the block, include/cudaDMAv2.h:65-75): per phase the compute wavefront writes 8 KiB to
+ * d_scratch, two DMA wavefronts move them to d_scratch + 8 KiB with CudaDMASequential's generic-pointer
+ * calls, the compute wavefront reads them back.  d_scratch: 16 KiB, 16-byte aligned; *d_wrong (zeroed)
+ * receives the number of words read back wrong.  The _lds_only twin is the same kernel built with
+ * HIPDMA_LDS_ONLY_FENCE. */
+int cudadma_selftest_global_handoff(unsigned* d_scratch, int* d_wrong, int phases, void* stream);
+int cudadma_selftest_global_handoff_lds_only(unsigned* d_scratch, int* d_wrong, int phases, void* stream);
 
 /* The split wait that only exists here (peek_dma_finish() + wait_for_dma_finish(peeked),
  * include/hipdma/base.hpp): one workgroup hands a 64-word buffer from a DMA wavefront to a
@@ -143,10 +191,15 @@ typedef struct cudadma_plan_query {
   int dst_stride;         /* strided; gather: dense-side stride                  */
   int radius, corners, dimx, dimy, pitch;   /* halo                              */
   const int* index;       /* gather / scatter: num_elmts element indices         */
+  int dst_pitch;          /* halo: destination row pitch in cells, 0 = dimx + 2*radius */
 } cudadma_plan_query_t;
 
 int cudadma_plan_map(const cudadma_plan_query_t* q, long long src_origin, long long dst_origin,
                      int* map, size_t map_len, int* steps_out);
+/* The same replay without the map: the lowest and highest byte offsets (relative to the transfer's pointers)
+ * that any DMA thread reads and writes; extents[0..3] = src_min, src_end, dst_min, dst_end (end = one past the
+ * last byte; all 0 for an empty transfer).  Returns 0 or a negative error. */
+int cudadma_plan_extents(const cudadma_plan_query_t* q, long long extents[4]);
 int cudadma_diagnose(int pattern, int alignment, int bytes_per_thread, int bytes_per_elmt, int dma_threads,
                      int num_elmts, int full_template, int verbose);
 
@@ -182,6 +235,10 @@ int cudadma_set_tuning(const char* name, int value);
 /* Seeded inputs generated on the device; bit-identical to the host statement
  * h(i) = splitmix64(seed + i) >> 32, value = (h >> 8) * 2^-23 - 1. */
 int cudadma_fill_uniform(float* d_dst, size_t n, uint64_t seed, void* stream);
+/* normal(0,1) values as bf16 bit patterns (the inputs of config 5): Box-Muller on the hashes 2i and 2i+1,
+ * sqrt(-2 ln u1) * cos(2 pi u2) with u1 = ((h(2i) >> 8) + 1) / 2^24 and u2 = (h(2i+1) >> 8) / 2^24 in double
+ * precision, rounded to float, then to bf16 (nearest even). */
+int cudadma_fill_normal_bf16(uint16_t* d_dst, size_t n, uint64_t seed, void* stream);
 /* Element indices uniform over [0, n_records), one in ten repeating an earlier draw. */
 int cudadma_fill_indices(int32_t* d_dst, size_t n, uint32_t n_records, uint64_t seed, void* stream);
 

@@ -16,10 +16,22 @@
 // phase * (threads in the signalling group).  The words only ever grow, so a
 // signal that nobody waits for (the "drain" wait_for_dma_start of
 // src/perf/sequential/perf_sequential.cu:139) is harmless either way.
-// Ordering is restricted to the LDS address space: a release before the add
-// (s_waitcnt lgkmcnt(0)), an acquire after the poll.  Outstanding global
-// stores of a consumer therefore do not delay its start_async_dma().
-// Define HIPDMA_FULL_FENCE to order every address space instead.
+// Ordering: a workgroup-scope release fence before the add, a workgroup-scope
+// acquire fence after the poll, over every address space, which is what
+// bar.sync / bar.arrive give CUDA code: global memory written by one side
+// before its signal is seen by the other side after its wait (LDS -> global
+// transfers, CudaDMAIndirect<false>, a source produced by the compute threads).
+// On gfx950 the wavefronts of a workgroup share one vector L1 that serves their
+// requests in issue order, so both fences come out as s_waitcnt lgkmcnt(0) and
+// cost what an LDS-only fence costs; what they add is that the compiler keeps
+// global accesses on their side of the hand-off.  HIPDMA_LDS_ONLY_FENCE
+// restricts both fences to the LDS address space for kernels that hand over
+// LDS contents only and want the compiler free to move global accesses across.
+// The *_direct forms of the DMA-side calls carry no fence at all (see below).
+//
+// A wait that gives up (HIPDMA_SPIN_LIMIT) records it: hipdma::status_words()
+// of the translation unit get the bit HIPDMA_STATUS_WAIT_GAVE_UP and a count,
+// which the host reads with hipdma::read_status() once the stream is idle.
 //
 // Requirements that differ from the CUDA original:
 //   * DMA and compute groups are made of whole 64-lane wavefronts:
@@ -41,11 +53,18 @@
 #define HIPDMA_SPIN_SLEEP 1
 #endif
 // A wait gives up after this many polls (about a second) and lets the wavefront
-// run on, so that unbalanced start_async_dma / execute_dma counts end in wrong
-// data and a finished kernel instead of a hung GPU.  0 = wait for ever.
+// run on, so that unbalanced start_async_dma / execute_dma counts end in a
+// finished kernel, wrong data and a recorded failure (HIPDMA_STATUS_WAIT_GAVE_UP)
+// instead of a hung GPU.  0 = wait for ever: the semantics of the reference's
+// named barriers (include/cudaDMAv2.h:65-75), for kernels whose stages between
+// two hand-offs can legitimately take longer than that.
 #ifndef HIPDMA_SPIN_LIMIT
 #define HIPDMA_SPIN_LIMIT (1 << 24)
 #endif
+
+// Bits of status word 0 (hipdma::read_status).
+#define HIPDMA_STATUS_OK            0u
+#define HIPDMA_STATUS_WAIT_GAVE_UP  1u   // a handshake wait ran into HIPDMA_SPIN_LIMIT: the kernel's results are void
 
 // DEBUG_CUDADMA (the reference's switch, include/cudaDMAv2.h:1564-1576) turns the
 // preconditions the objects rely on into device-side asserts: thread groups made of whole
@@ -101,6 +120,23 @@ namespace detail {
 
 typedef __attribute__((address_space(3))) unsigned lds_word_t;
 
+// Failure record of this translation unit's kernels: word 0 collects HIPDMA_STATUS_* bits, word 1
+// counts the waits that gave up.  File scope and internal linkage: every translation unit that
+// includes the header has its own pair (device code is linked per translation unit), read through
+// hipdma::read_status() compiled in that same translation unit.
+static __device__ __attribute__((used)) unsigned g_status_words[2];
+
+// Cold path of a wait that ran into HIPDMA_SPIN_LIMIT.
+__device__ __forceinline__ void record_wait_gave_up()
+{
+  // one lane per wavefront reports: the count is in wavefronts
+  const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  if (lane == __builtin_ctzll(__builtin_amdgcn_ballot_w64(true))) {
+    __hip_atomic_fetch_or(&g_status_words[0], HIPDMA_STATUS_WAIT_GAVE_UP, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_fetch_add(&g_status_words[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 // Two words per dmaID.  A function-local __shared__ array: every kernel that
 // constructs a warp-specialised object gets its own 128-byte copy and the
 // user never has to pass LDS for it.
@@ -112,19 +148,19 @@ __device__ __forceinline__ lds_word_t* sync_words()
 
 __device__ __forceinline__ void release_lds()
 {
-#ifdef HIPDMA_FULL_FENCE
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-#else
+#ifdef HIPDMA_LDS_ONLY_FENCE
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+#else
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
 #endif
 }
 
 __device__ __forceinline__ void acquire_lds()
 {
-#ifdef HIPDMA_FULL_FENCE
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-#else
+#ifdef HIPDMA_LDS_ONLY_FENCE
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#else
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 #endif
 }
 
@@ -162,9 +198,10 @@ __device__ __forceinline__ void wait_word(lds_word_t* word, unsigned target)
   const unsigned want = __builtin_amdgcn_readfirstlane(target);
 #if HIPDMA_SPIN_LIMIT > 0
   int polls = 0;
-  while ((int)(__builtin_amdgcn_readfirstlane(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) - want) < 0 &&
-         ++polls < HIPDMA_SPIN_LIMIT)
+  while ((int)(__builtin_amdgcn_readfirstlane(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) - want) < 0) {
+    if (++polls >= HIPDMA_SPIN_LIMIT) { record_wait_gave_up(); break; }
     __builtin_amdgcn_s_sleep(HIPDMA_SPIN_SLEEP);
+  }
 #else
   while ((int)(__builtin_amdgcn_readfirstlane(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) - want) < 0)
     __builtin_amdgcn_s_sleep(HIPDMA_SPIN_SLEEP);
@@ -189,13 +226,12 @@ __device__ __forceinline__ void wait_word_unfenced(lds_word_t* word, unsigned ta
   const unsigned addr = (unsigned)(size_t)word;
   const unsigned want = __builtin_amdgcn_readfirstlane(target);
   unsigned seen;
-#if HIPDMA_SPIN_LIMIT > 0
-  for (int polls = 0; polls < HIPDMA_SPIN_LIMIT; ++polls) {
-#else
-  for (;;) {
-#endif
+  for (int polls = 0;;) {
     asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : "v"(addr) : "memory");
     if ((int)(__builtin_amdgcn_readfirstlane(seen) - want) >= 0) break;
+#if HIPDMA_SPIN_LIMIT > 0
+    if (++polls >= HIPDMA_SPIN_LIMIT) { record_wait_gave_up(); break; }
+#endif
     __builtin_amdgcn_s_sleep(HIPDMA_SPIN_SLEEP);
   }
 }
@@ -225,6 +261,28 @@ __host__ __device__ constexpr bool store_is_direct(int q) { return q == STORE_LD
 __host__ __device__ constexpr bool store_is_swizzled(int q) { return q == STORE_LDS_SWIZZLE || q == STORE_LDS_DIRECT_SWIZZLE; }
 
 }  // namespace detail
+
+// Host side of the failure record.  The address of this translation unit's words on the current device
+// (hipGetSymbolAddress; every device holds its own copy), and a read of them: status[0] = HIPDMA_STATUS_* bits,
+// status[1] = waits that gave up since the last clear.  read_status() waits for `stream` to drain, copies
+// eight bytes and, with `clear`, writes zeros back; it allocates nothing.  Both must be compiled in the same
+// translation unit as the kernels they report on.
+static inline hipError_t status_words_address(unsigned** words)
+{
+  return hipGetSymbolAddress((void**)words, HIP_SYMBOL(detail::g_status_words));
+}
+static inline hipError_t read_status(unsigned status[2], hipStream_t stream = nullptr, bool clear = false)
+{
+  unsigned* words = nullptr;
+  hipError_t e = status_words_address(&words);
+  if (e != hipSuccess) return e;
+  e = hipStreamSynchronize(stream);
+  if (e != hipSuccess) return e;
+  e = hipMemcpy(status, words, 2 * sizeof(unsigned), hipMemcpyDeviceToHost);
+  if (e != hipSuccess || !clear) return e;
+  const unsigned zeros[2] = {0u, 0u};
+  return hipMemcpy(words, zeros, sizeof(zeros), hipMemcpyHostToDevice);
+}
 
 // The swizzled LDS layouts.  The LDS has 64 banks of 4 bytes: addresses 256 bytes apart share
 // their banks.  For rows of `chunks_per_row` chunks of `chunk_bytes` bytes each:

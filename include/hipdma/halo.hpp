@@ -11,15 +11,18 @@
 //   * RADIUS cells left and right of each of the dimy tile rows are moved
 //     (include/cudaDMA.h:3746-3749);
 //   * the source row pitch is `pitch` cells, the destination row pitch is
-//     dimx + 2*RADIUS cells (include/cudaDMA.h:3718-3719);
+//     dimx + 2*RADIUS cells (include/cudaDMA.h:3718-3719) unless the constructor is
+//     given a wider one (`dst_pitch`, an addition of this library: a consumer that
+//     reads the plane down its columns picks the pitch that keeps those reads off
+//     each other's LDS banks, as the strided classes let it with dst_stride);
 //   * the interior is not touched (src/tests/test_halo/cudaDMA_test_halo.cu:91-164).
 //
 // Work split (wave64): two slot grids laid end to end and dealt round-robin to
 // the DMA threads, thread t owning slots t, t+T, ...
 //   rows : 2*RADIUS rows of ceil(row_bytes / XR) chunks, row padded to W1 slots
 //   sides: 2*dimy strips of (RADIUS*BYTES_PER_ELMT / XS) chunks, strip padded to W2 slots
-// ALIGNMENT is what both origins, the source pitch in bytes, dimx*BYTES_PER_ELMT
-// and 2*RADIUS*BYTES_PER_ELMT (hence the destination pitch) are multiples of.
+// ALIGNMENT is what both origins, both pitches in bytes, dimx*BYTES_PER_ELMT
+// and 2*RADIUS*BYTES_PER_ELMT (hence the default destination pitch) are multiples of.
 // Rows without corners start on such a boundary and move in chunks of XR =
 // ALIGNMENT bytes; a strip, and a row with corners, starts RADIUS*BYTES_PER_ELMT
 // bytes off one and moves in pieces of XS = the largest power of two (at most
@@ -48,12 +51,14 @@ struct HaloGeom {
   static constexpr int W2 = GridPlan::slots(LPS);
   int dimx_bytes, dimy, src_pitch, dst_pitch, row_bytes, lpr, w1, s1, total;
 
-  __host__ __device__ __forceinline__ void init(const int dimx, const int dimy_, const int pitch)
+  // dst_pitch_cells <= 0 selects the reference's destination pitch, dimx + 2*RADIUS cells.
+  __host__ __device__ __forceinline__ void init(const int dimx, const int dimy_, const int pitch,
+                                                const int dst_pitch_cells = 0)
   {
     dimx_bytes = dimx * BYTES_PER_ELMT;
     dimy = dimy_;
     src_pitch = pitch * BYTES_PER_ELMT;
-    dst_pitch = (dimx + 2 * RADIUS) * BYTES_PER_ELMT;
+    dst_pitch = (dst_pitch_cells > 0 ? dst_pitch_cells : dimx + 2 * RADIUS) * BYTES_PER_ELMT;
     row_bytes = dimx_bytes + (CORNERS ? 2 * SIDE_BYTES : 0);
     lpr = ceil_div(row_bytes, XR);
     w1 = GridPlan::slots(lpr);
@@ -126,36 +131,37 @@ public:
   template<int L = LEVEL, bool S = DO_SYNC, when<(L == 1) && S> = 0>
   __device__ __forceinline__ CudaDMAHalo(const int dmaID, const int num_dma_threads, const int num_compute_threads,
                                          const int dma_threadIdx_start, const int dimx, const int dimy,
-                                         const int pitch)
+                                         const int pitch, const int dst_pitch = 0)
     : CudaDMA(dmaID, num_dma_threads, num_compute_threads, dma_threadIdx_start)
-  { init(num_dma_threads, dma_threadIdx_start, dimx, dimy, pitch); }
+  { init(num_dma_threads, dma_threadIdx_start, dimx, dimy, pitch, dst_pitch); }
   template<int L = LEVEL, bool S = DO_SYNC, when<(L == 2) && S> = 0>
   __device__ __forceinline__ CudaDMAHalo(const int dmaID, const int num_compute_threads,
                                          const int dma_threadIdx_start, const int dimx, const int dimy,
-                                         const int pitch)
+                                         const int pitch, const int dst_pitch = 0)
     : CudaDMA(dmaID, DMA_THREADS, num_compute_threads, dma_threadIdx_start)
-  { init(DMA_THREADS, dma_threadIdx_start, dimx, dimy, pitch); }
+  { init(DMA_THREADS, dma_threadIdx_start, dimx, dimy, pitch, dst_pitch); }
   template<int L = LEVEL, bool S = DO_SYNC, when<(L == 3) && S> = 0>
   __device__ __forceinline__ CudaDMAHalo(const int dmaID, const int num_compute_threads,
-                                         const int dma_threadIdx_start, const int pitch)
+                                         const int dma_threadIdx_start, const int pitch, const int dst_pitch = 0)
     : CudaDMA(dmaID, DMA_THREADS, num_compute_threads, dma_threadIdx_start)
-  { init(DMA_THREADS, dma_threadIdx_start, DIMX, DIMY, pitch); }
+  { init(DMA_THREADS, dma_threadIdx_start, DIMX, DIMY, pitch, dst_pitch); }
 
   // ---- constructors of the form that is not warp-specialised ----
   template<int L = LEVEL, bool S = DO_SYNC, when<(L == 1) && !S> = 0>
   __device__ __forceinline__ CudaDMAHalo(const int dimx, const int dimy, const int pitch,
-                                         const int num_dma_threads = 0, const int dma_threadIdx_start = 0)
+                                         const int num_dma_threads = 0, const int dma_threadIdx_start = 0,
+                                         const int dst_pitch = 0)
     : CudaDMA(hipdma::detail::no_sync_t(), threads_or_block(num_dma_threads), dma_threadIdx_start)
-  { init(threads_or_block(num_dma_threads), dma_threadIdx_start, dimx, dimy, pitch); }
+  { init(threads_or_block(num_dma_threads), dma_threadIdx_start, dimx, dimy, pitch, dst_pitch); }
   template<int L = LEVEL, bool S = DO_SYNC, when<(L == 2) && !S> = 0>
   __device__ __forceinline__ CudaDMAHalo(const int dimx, const int dimy, const int pitch,
-                                         const int dma_threadIdx_start = 0)
+                                         const int dma_threadIdx_start = 0, const int dst_pitch = 0)
     : CudaDMA(hipdma::detail::no_sync_t(), DMA_THREADS, dma_threadIdx_start)
-  { init(DMA_THREADS, dma_threadIdx_start, dimx, dimy, pitch); }
+  { init(DMA_THREADS, dma_threadIdx_start, dimx, dimy, pitch, dst_pitch); }
   template<int L = LEVEL, bool S = DO_SYNC, when<(L == 3) && !S> = 0>
-  __device__ __forceinline__ CudaDMAHalo(const int pitch, const int dma_threadIdx_start = 0)
+  __device__ __forceinline__ CudaDMAHalo(const int pitch, const int dma_threadIdx_start = 0, const int dst_pitch = 0)
     : CudaDMA(hipdma::detail::no_sync_t(), DMA_THREADS, dma_threadIdx_start)
-  { init(DMA_THREADS, dma_threadIdx_start, DIMX, DIMY, pitch); }
+  { init(DMA_THREADS, dma_threadIdx_start, DIMX, DIMY, pitch, dst_pitch); }
 
 public:
   __device__ __forceinline__ void execute_dma(const void* __restrict__ src_origin, void* __restrict__ dst_origin)
@@ -213,15 +219,16 @@ private:
   __device__ __forceinline__ static int threads_or_block(const int n) { return (n <= 0) ? int(blockDim.x) : n; }
 
   __device__ __forceinline__ void init(const int threads, const int start, const int dimx, const int dimy,
-                                       const int pitch)
+                                       const int pitch, const int dst_pitch)
   {
     using namespace hipdma::detail;
     HIPDMA_ASSERT(threads > 0 && (threads % HIPDMA_WAVE_SIZE) == 0);
     HIPDMA_ASSERT(dimx > 0 && dimy > 0 && pitch >= dimx + 2 * RADIUS);
     HIPDMA_ASSERT(((pitch * BYTES_PER_ELMT) % ALIGNMENT) == 0);
+    HIPDMA_ASSERT(dst_pitch <= 0 || (dst_pitch >= dimx + 2 * RADIUS && ((dst_pitch * BYTES_PER_ELMT) % ALIGNMENT) == 0));
     m_tid = int(threadIdx.x) - start;
     m_threads = threads;
-    m_geom.init(dimx, dimy, pitch);
+    m_geom.init(dimx, dimy, pitch, dst_pitch);
     m_steps = ceil_div(ceil_div(m_geom.total, threads), MAX_LDS);
   }
 

@@ -126,7 +126,7 @@ public:
   {
     if constexpr (DO_SYNC) CudaDMA::wait_for_dma_start();
     if (use_direct<DMA_STORE_QUAL>()) {
-      if constexpr (DMA_STORE_QUAL == STORE_LDS_DIRECT && GATHER) direct_all((char*)dst_ptr);
+      if constexpr (DMA_STORE_QUAL == STORE_LDS_DIRECT && GATHER) direct_all<DMA_LOAD_QUAL>((char*)dst_ptr);
     } else {
       hipdma::detail::GridCursor cur = m_grid.begin();
       store_step<DMA_STORE_QUAL>((char*)dst_ptr, 0, cur);
@@ -204,6 +204,7 @@ private:
     }
   }
 
+  template<int LOAD_QUAL>
   __device__ __forceinline__ void direct_all(char* dst)
   {
     using namespace hipdma::detail;
@@ -221,7 +222,7 @@ private:
         if (m_grid.live(r0 + k, cur)) {
           const int lds_off = cur.row * m_dense_stride + cur.col * ALIGNMENT;
           if constexpr (ALIGNMENT == 16 || ALIGNMENT == 4)
-            load_to_lds<ALIGNMENT>(m_src + m_idx[k] * m_grid.E + cur.col * ALIGNMENT,
+            load_to_lds<ALIGNMENT, LOAD_QUAL>(m_src + m_idx[k] * m_grid.E + cur.col * ALIGNMENT,
                                    dst + (lds_off - lane * ALIGNMENT));
         }
         m_grid.advance(cur);

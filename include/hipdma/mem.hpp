@@ -27,30 +27,58 @@ template<> struct chunk_of<16> { typedef u32x4_t type; };
 #define HIPDMA_GLOBAL_AS __attribute__((address_space(1)))
 #define HIPDMA_LDS_AS    __attribute__((address_space(3)))
 
-// One aligned vector load of sizeof(T) bytes.
-template<typename T, bool GLOBAL_LOAD, int LOAD_QUAL>
-__device__ __forceinline__ T load_vec(const void* ptr)
+// Cache-policy bits of a gfx950 vector memory instruction (the `aux` operand of the direct-to-LDS
+// loads: 1 = sc0, 2 = nt, 16 = sc1) for each load qualifier of include/cudaDMAv2.h:50-56:
+//   LOAD_CACHE_ALL       (ld.ca)  none: cached in the vector L1 and in L2
+//   LOAD_CACHE_GLOBAL    (ld.cg)  sc1: device scope, the vector L1 is bypassed and L2 serves the load
+//   LOAD_CACHE_STREAMING (ld.cs)  nt: non-temporal, the line is first in line for eviction
+//   LOAD_CACHE_LAST_USE  (ld.lu)  nt: the closest policy there is
+//   LOAD_CACHE_VOLATILE  (ld.cv)  sc0 sc1: system scope, fetched again on every access
+__host__ __device__ constexpr int load_policy_bits(const int q)
 {
-  if constexpr (GLOBAL_LOAD) {
-    const HIPDMA_GLOBAL_AS T* p = (const HIPDMA_GLOBAL_AS T*)ptr;
-    if constexpr (LOAD_QUAL == LOAD_CACHE_STREAMING || LOAD_QUAL == LOAD_CACHE_LAST_USE)
-      return __builtin_nontemporal_load(p);
-    else if constexpr (LOAD_QUAL == LOAD_CACHE_VOLATILE)
-      return *(const volatile HIPDMA_GLOBAL_AS T*)p;
-    else
-      return *p;
+  return (q == LOAD_CACHE_STREAMING || q == LOAD_CACHE_LAST_USE) ? 2
+       : (q == LOAD_CACHE_VOLATILE) ? 17
+       : (q == LOAD_CACHE_GLOBAL) ? 16 : 0;
+}
+
+// One aligned vector load of sizeof(T) bytes, P = pointer type in the address space of the source.
+// The compiler offers sc1 alone only through an agent-scope atomic load, which exists for 4 and 8
+// bytes; a 16-byte LOAD_CACHE_GLOBAL load is issued with sc0 sc1 instead (one dwordx4, the vector L1
+// bypassed all the same; for device memory the L2 treats both scopes alike).
+template<typename T, int LOAD_QUAL, typename P>
+__device__ __forceinline__ T load_vec_from(P p)
+{
+  if constexpr (LOAD_QUAL == LOAD_CACHE_STREAMING || LOAD_QUAL == LOAD_CACHE_LAST_USE) {
+    return __builtin_nontemporal_load(p);
+  } else if constexpr (LOAD_QUAL == LOAD_CACHE_VOLATILE || (LOAD_QUAL == LOAD_CACHE_GLOBAL && sizeof(T) == 16)) {
+    return *(volatile typename std::remove_pointer<P>::type*)p;     // volatile added, address space kept
+  } else if constexpr (LOAD_QUAL == LOAD_CACHE_GLOBAL && sizeof(T) == 4) {
+    return (T)__hip_atomic_load((const unsigned*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else if constexpr (LOAD_QUAL == LOAD_CACHE_GLOBAL && sizeof(T) == 8) {
+    const unsigned long long v = __hip_atomic_load((const unsigned long long*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    T out;
+    out[0] = (unsigned)v;
+    out[1] = (unsigned)(v >> 32);
+    return out;
   } else {
-    const T* p = (const T*)ptr;
-    if constexpr (LOAD_QUAL == LOAD_CACHE_STREAMING || LOAD_QUAL == LOAD_CACHE_LAST_USE)
-      return __builtin_nontemporal_load(p);
-    else if constexpr (LOAD_QUAL == LOAD_CACHE_VOLATILE)
-      return *(const volatile T*)p;
-    else
-      return *p;
+    return *p;
   }
 }
 
-// One aligned vector store of sizeof(T) bytes.
+template<typename T, bool GLOBAL_LOAD, int LOAD_QUAL>
+__device__ __forceinline__ T load_vec(const void* ptr)
+{
+  if constexpr (GLOBAL_LOAD) return load_vec_from<T, LOAD_QUAL>((const HIPDMA_GLOBAL_AS T*)ptr);
+  else return load_vec_from<T, LOAD_QUAL>((const T*)ptr);
+}
+
+// One aligned vector store of sizeof(T) bytes.  The reference's stores take generic addresses
+// (include/cudaDMAv2.h:553-679); so do these, except for the STORE_LDS* additions.
+//   STORE_WRITE_BACK          (st.wb)  plain store
+//   STORE_CACHE_GLOBAL        (st.cg)  plain store: the vector L1 is write-through and does not allocate on a
+//                                      store, so every store is already held in L2 only
+//   STORE_CACHE_STREAMING     (st.cs)  nt
+//   STORE_CACHE_WRITE_THROUGH (st.wt)  sc0 sc1: system scope, written through L2
 template<typename T, int STORE_QUAL>
 __device__ __forceinline__ void store_vec(const T& value, void* ptr)
 {
@@ -143,17 +171,17 @@ __device__ __forceinline__ void store_chunk(const typename chunk_of<CHUNK>::type
 // Direct global -> LDS move of BYTES (4 or 16) per active lane.  `lds_wave_base`
 // must be the same for every lane of the wavefront; lane L lands at
 // lds_wave_base + L*BYTES.
-template<int BYTES>
+template<int BYTES, int LOAD_QUAL = LOAD_CACHE_ALL>
 __device__ __forceinline__ void load_to_lds(const char* global_lane_ptr, char* lds_wave_base)
 {
   static_assert(BYTES == 4 || BYTES == 16, "global_load_lds moves 4 or 16 bytes per lane here");
-  // the size operand has to be a literal
+  // the size and the cache-policy operands have to be literals
   if constexpr (BYTES == 16)
     __builtin_amdgcn_global_load_lds((const HIPDMA_GLOBAL_AS void*)global_lane_ptr,
-                                     (HIPDMA_LDS_AS void*)lds_wave_base, 16, 0, 0);
+                                     (HIPDMA_LDS_AS void*)lds_wave_base, 16, 0, load_policy_bits(LOAD_QUAL));
   else
     __builtin_amdgcn_global_load_lds((const HIPDMA_GLOBAL_AS void*)global_lane_ptr,
-                                     (HIPDMA_LDS_AS void*)lds_wave_base, 4, 0, 0);
+                                     (HIPDMA_LDS_AS void*)lds_wave_base, 4, 0, load_policy_bits(LOAD_QUAL));
 }
 
 // The same move with the source address split into a part that is the same in every lane, held
@@ -172,18 +200,28 @@ __device__ __forceinline__ const char* scalar_ptr(const char* p)
 }
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"      // m0 is a reserved register: naming it keeps the compiler from merging its own writes across this one
-template<int BYTES>
+#define HIPDMA_LOAD_TO_LDS_ASM(INSN, POLICY)                                                  \
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\t" INSN " %0, %1" POLICY                          \
+               : : "v"(lane_offset), "s"(scalar_base), "s"(lds_wave_base) : "memory", "m0")
+template<int BYTES, int LOAD_QUAL = LOAD_CACHE_ALL>
 __device__ __forceinline__ void load_to_lds_scalar_base(const char* scalar_base, const unsigned lane_offset,
                                                         const unsigned lds_wave_base)
 {
   static_assert(BYTES == 4 || BYTES == 16, "global_load_lds moves 4 or 16 bytes per lane here");
-  if constexpr (BYTES == 16)
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 : : "v"(lane_offset), "s"(scalar_base), "s"(lds_wave_base) : "memory", "m0");
-  else
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1"
-                 : : "v"(lane_offset), "s"(scalar_base), "s"(lds_wave_base) : "memory", "m0");
+  constexpr int bits = load_policy_bits(LOAD_QUAL);
+  if constexpr (BYTES == 16) {
+    if constexpr (bits == 2) HIPDMA_LOAD_TO_LDS_ASM("global_load_lds_dwordx4", " nt");
+    else if constexpr (bits == 16) HIPDMA_LOAD_TO_LDS_ASM("global_load_lds_dwordx4", " sc1");
+    else if constexpr (bits == 17) HIPDMA_LOAD_TO_LDS_ASM("global_load_lds_dwordx4", " sc0 sc1");
+    else HIPDMA_LOAD_TO_LDS_ASM("global_load_lds_dwordx4", "");
+  } else {
+    if constexpr (bits == 2) HIPDMA_LOAD_TO_LDS_ASM("global_load_lds_dword", " nt");
+    else if constexpr (bits == 16) HIPDMA_LOAD_TO_LDS_ASM("global_load_lds_dword", " sc1");
+    else if constexpr (bits == 17) HIPDMA_LOAD_TO_LDS_ASM("global_load_lds_dword", " sc0 sc1");
+    else HIPDMA_LOAD_TO_LDS_ASM("global_load_lds_dword", "");
+  }
 }
+#undef HIPDMA_LOAD_TO_LDS_ASM
 #pragma clang diagnostic pop
 
 // Wait until every global -> LDS move of this wavefront has landed.

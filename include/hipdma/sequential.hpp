@@ -220,7 +220,7 @@ private:
       const int wave_off = off - lane * ALIGNMENT;
       const int rem = m_bytes - off;
       if (rem >= ALIGNMENT) {
-        load_to_lds<ALIGNMENT>(m_src + off, dst + wave_off);
+        load_to_lds<ALIGNMENT, LOAD_QUAL>(m_src + off, dst + wave_off);
       } else if (rem > 0) {
         chunk_t tail;
         load_chunk<ALIGNMENT, 4, true, LOAD_QUAL>(tail, m_src + off, rem);

@@ -162,7 +162,7 @@ public:
       if constexpr (hipdma::detail::store_is_direct(DMA_STORE_QUAL)) {
         static_assert(!hipdma::detail::store_is_direct(DMA_STORE_QUAL) || DMA_GLOBAL_LOAD,
                       "STORE_LDS_DIRECT needs a global source");
-        direct_all<hipdma::detail::store_is_swizzled(DMA_STORE_QUAL)>((char*)dst_ptr);
+        direct_all<hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), DMA_LOAD_QUAL>((char*)dst_ptr);
       }
     } else {
       hipdma::detail::GridCursor cur = m_grid.begin();
@@ -184,14 +184,14 @@ public:
   // hipdma::wait_direct_loads<YOUNGER>() waits for this transfer while the YOUNGER loads issued
   // after it (loads_per_thread() of each later transfer) stay in flight.  Needs the shape the
   // direct path needs (direct_ready()); neither call touches the handshake.
-  template<int DMA_STORE_QUAL = STORE_LDS_DIRECT>
+  template<int DMA_STORE_QUAL = STORE_LDS_DIRECT, int DMA_LOAD_QUAL = LOAD_CACHE_ALL>
   __device__ __forceinline__ void issue_direct(const void* __restrict__ src_ptr, void* __restrict__ dst_ptr)
   {
     static_assert(hipdma::detail::store_is_direct(DMA_STORE_QUAL), "issue_direct takes one of the STORE_LDS_DIRECT qualifiers");
     static_assert(ALIGNMENT == 16 || ALIGNMENT == 4, "global_load_lds moves 4 or 16 bytes per lane");
     HIPDMA_ASSERT(direct_ready());
     m_src = (const char*)src_ptr;
-    issue_direct_rounds<hipdma::detail::store_is_swizzled(DMA_STORE_QUAL)>((char*)dst_ptr);
+    issue_direct_rounds<hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), false, DMA_LOAD_QUAL>((char*)dst_ptr);
   }
   // A part of the same transfer: the loads of rounds [first_round, first_round + num_rounds) of the
   // loads_per_thread() a thread issues for it, for callers that spread the loads of a transfer between other
@@ -200,7 +200,7 @@ public:
   // With WHOLE_ROWS the caller vouches for the shape the scalar-base loads need (the DMA threads cover whole rows,
   // a non-negative source stride, a round's rows within 4 GiB): only that form is compiled, and the few scalar
   // instructions of a load fit under one matrix instruction.
-  template<int DMA_STORE_QUAL = STORE_LDS_DIRECT, bool WHOLE_ROWS = false>
+  template<int DMA_STORE_QUAL = STORE_LDS_DIRECT, bool WHOLE_ROWS = false, int DMA_LOAD_QUAL = LOAD_CACHE_ALL>
   __device__ __forceinline__ void issue_direct_part(const void* __restrict__ src_ptr, void* __restrict__ dst_ptr,
                                                     const int first_round, const int num_rounds)
   {
@@ -208,7 +208,7 @@ public:
     static_assert(ALIGNMENT == 16 || ALIGNMENT == 4, "global_load_lds moves 4 or 16 bytes per lane");
     HIPDMA_ASSERT(direct_ready());
     m_src = (const char*)src_ptr;
-    issue_direct_rounds<hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), WHOLE_ROWS>((char*)dst_ptr, first_round, first_round + num_rounds);
+    issue_direct_rounds<hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), WHOLE_ROWS, DMA_LOAD_QUAL>((char*)dst_ptr, first_round, first_round + num_rounds);
   }
   // True when this object's shape can use global_load_lds (whole chunks, whole wavefronts, rows of
   // at least a wavefront of chunks or unpadded power-of-two rows).
@@ -306,14 +306,14 @@ private:
 
   // Lane L of a wavefront always lands on LDS chunk (base + L); with SWIZZLE the lane
   // fetches the source chunk that belongs at its landing position instead.
-  template<bool SWIZZLE>
+  template<bool SWIZZLE, int LOAD_QUAL>
   __device__ __forceinline__ void direct_all(char* dst)
   {
-    issue_direct_rounds<SWIZZLE>(dst);
+    issue_direct_rounds<SWIZZLE, false, LOAD_QUAL>(dst);
     hipdma::detail::wait_lds_direct();
   }
 
-  template<bool SWIZZLE, bool WHOLE_ROWS = false>
+  template<bool SWIZZLE, bool WHOLE_ROWS = false, int LOAD_QUAL = LOAD_CACHE_ALL>
   __device__ __forceinline__ void issue_direct_rounds(char* dst, const int first = 0, const int end = 0x7fffffff)
   {
     using namespace hipdma::detail;
@@ -342,7 +342,7 @@ private:
         if (r >= first && r < end && m_grid.live(r, cur)) {
           const unsigned lane_off = lane_row + (unsigned)(lds_col<SWIZZLE>(cur) * ALIGNMENT);
           if constexpr (ALIGNMENT == 16 || ALIGNMENT == 4)
-            load_to_lds_scalar_base<ALIGNMENT>(base + r * round_src, lane_off, lds0 + r * round_lds);
+            load_to_lds_scalar_base<ALIGNMENT, LOAD_QUAL>(base + r * round_src, lane_off, lds0 + r * round_lds);
         }
         m_grid.advance(cur);
       }
@@ -353,7 +353,7 @@ private:
       if (r >= first && r < end && m_grid.live(r, cur)) {
         const int lds_off = cur.row * m_dst_stride + cur.col * ALIGNMENT;
         if constexpr (ALIGNMENT == 16 || ALIGNMENT == 4)
-          load_to_lds<ALIGNMENT>(m_src + cur.row * m_src_stride + lds_col<SWIZZLE>(cur) * ALIGNMENT,
+          load_to_lds<ALIGNMENT, LOAD_QUAL>(m_src + cur.row * m_src_stride + lds_col<SWIZZLE>(cur) * ALIGNMENT,
                                  dst + (lds_off - lane * ALIGNMENT));
       }
       m_grid.advance(cur);

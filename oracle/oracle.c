@@ -200,10 +200,18 @@ void oracle_scatter(const int32_t* index, const void* src, void* dst, int elmt_b
 void oracle_halo(const void* src_origin, void* dst_origin, int elmt_bytes, int radius, int corners,
                  int dimx, int dimy, int pitch)
 {
+  oracle_halo_pitched(src_origin, dst_origin, elmt_bytes, radius, corners, dimx, dimy, pitch, dimx + 2 * radius);
+}
+
+/* The same ring with the destination row pitch given in cells (>= dimx+2R): the layout the build's
+ * CudaDMAHalo offers next to the reference's fixed one; dst_pitch = dimx+2R is the reference's. */
+void oracle_halo_pitched(const void* src_origin, void* dst_origin, int elmt_bytes, int radius, int corners,
+                         int dimx, int dimy, int pitch, int dst_pitch)
+{
   const unsigned char* s = (const unsigned char*)src_origin;
   unsigned char* d = (unsigned char*)dst_origin;
   const ptrdiff_t sp = (ptrdiff_t)pitch * elmt_bytes;
-  const ptrdiff_t dp = (ptrdiff_t)(dimx + 2 * radius) * elmt_bytes;
+  const ptrdiff_t dp = (ptrdiff_t)dst_pitch * elmt_bytes;
   const ptrdiff_t x0 = corners ? -(ptrdiff_t)radius * elmt_bytes : 0;
   const ptrdiff_t x1 = (ptrdiff_t)dimx * elmt_bytes + (corners ? (ptrdiff_t)radius * elmt_bytes : 0);
   for (int r = 0; r < radius; ++r) {

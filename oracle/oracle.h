@@ -52,6 +52,8 @@ void oracle_gather(const int32_t* index, const void* src, void* dst, int elmt_by
 void oracle_scatter(const int32_t* index, const void* src, void* dst, int elmt_bytes, int num_elmts, int alt_stride);
 void oracle_halo(const void* src_origin, void* dst_origin, int elmt_bytes, int radius, int corners,
                  int dimx, int dimy, int pitch);
+void oracle_halo_pitched(const void* src_origin, void* dst_origin, int elmt_bytes, int radius, int corners,
+                         int dimx, int dimy, int pitch, int dst_pitch);
 /* 1 when odata holds the ring of idata; both point at the top-left of the padded tile */
 int oracle_halo_check(const void* idata, const void* odata, int elmt_bytes, int radius, int corners,
                       int dimx, int dimy, int pitch);

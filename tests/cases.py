@@ -14,14 +14,14 @@ def _round_up(v, m):
 class CaseIO:
     """Everything one run of a case needs, plus what the LDS buffer must hold afterwards."""
 
-    def __init__(self, case, flavour=0, reps=2, data="ramp", reverse=False):
+    def __init__(self, case, flavour=0, reps=2, data="ramp", reverse=False, dst_pitch=None):
         self.case = case
         self.reps = reps
         self.reverse = reverse
         a = case.alignment
         rng = np.random.default_rng(1000 * case.pattern + 17 * flavour + case.bytes_per_elmt + case.dma_threads)
         self.index = None
-        self.src_stride = self.dst_stride = self.pitch = 0
+        self.src_stride = self.dst_stride = self.pitch = self.dst_pitch = 0
         self.rep_index_elmts = 0
         self.src_offset = a * (flavour % 3)
         self.dst_offset = a * ((flavour + 1) % 2)
@@ -62,13 +62,18 @@ class CaseIO:
             r, dimx, dimy = case.radius, case.dimx, case.dimy
             unit = max(1, a // e)
             self.pitch = _round_up(dimx + 2 * r + (flavour % 3), unit)
+            # every third flavour of the v2-style classes widens the destination rows (0 = the reference's dimx + 2R)
+            if dst_pitch is None:
+                dst_pitch = _round_up(dimx + 2 * r + 1 + flavour % 5, unit) if (case.level >= 1 and flavour % 3 == 2) else 0
+            self.dst_pitch = dst_pitch
+            self.dst_cells = dst_pitch if dst_pitch > 0 else dimx + 2 * r
             src_origin = (r * self.pitch + r) * e
-            dst_origin = (r * (dimx + 2 * r) + r) * e
+            dst_origin = (r * self.dst_cells + r) * e
             self.src_offset = (-src_origin) % a
             self.dst_offset = (-dst_origin) % a
             self.rep_src_bytes = a
             footprint_src = (dimy + 2 * r) * self.pitch * e
-            footprint_dst = (dimx + 2 * r) * (dimy + 2 * r) * e
+            footprint_dst = self.dst_cells * (dimy + 2 * r) * e
         else:
             raise ValueError(pat)
         if reverse:
@@ -108,8 +113,8 @@ class CaseIO:
             O.oracle_scatter(ptr(idx), ptr(src, so), ptr(dst, do), e, n, self.src_stride)
         else:
             r = c.radius
-            O.oracle_halo(ptr(src, so + (r * self.pitch + r) * e), ptr(dst, do + (r * (c.dimx + 2 * r) + r) * e),
-                          e, r, c.corners, c.dimx, c.dimy, self.pitch)
+            O.oracle_halo_pitched(ptr(src, so + (r * self.pitch + r) * e), ptr(dst, do + (r * self.dst_cells + r) * e),
+                                  e, r, c.corners, c.dimx, c.dimy, self.pitch, self.dst_cells)
 
     def expected(self, swizzle=False):
         if self.reverse:
@@ -144,9 +149,9 @@ class CaseIO:
             O.oracle_scatter(ptr(idx), ptr(ids, so), ptr(dst, do), e, n, 4 * self.src_stride)
         else:
             r = c.radius
-            O.oracle_halo(ptr(ids, so + 4 * (r * self.pitch + r) * c.bytes_per_elmt),
-                          ptr(dst, do + 4 * (r * (c.dimx + 2 * r) + r) * c.bytes_per_elmt),
-                          e, r, c.corners, c.dimx, c.dimy, self.pitch)
+            O.oracle_halo_pitched(ptr(ids, so + 4 * (r * self.pitch + r) * c.bytes_per_elmt),
+                                  ptr(dst, do + 4 * (r * self.dst_cells + r) * c.bytes_per_elmt),
+                                  e, r, c.corners, c.dimx, c.dimy, self.pitch, self.dst_cells)
         return dst
 
     def replay_map(self, rep=0):
@@ -157,14 +162,15 @@ class CaseIO:
         dst_origin = self.dst_offset
         if c.pattern == cd.PATTERN_HALO:
             src_origin += (c.radius * self.pitch + c.radius) * e
-            dst_origin += (c.radius * (c.dimx + 2 * c.radius) + c.radius) * e
+            dst_origin += (c.radius * self.dst_cells + c.radius) * e
         idx = self.index[rep * self.rep_index_elmts:rep * self.rep_index_elmts + c.num_elmts] \
             if self.index is not None else None
         return cd.plan.plan_map(
             c.pattern, alignment=c.alignment, bytes_per_thread=c.bytes_per_thread, bytes_per_elmt=e,
             dma_threads=c.dma_threads, num_elmts=c.num_elmts, src_stride=self.src_stride,
             dst_stride=self.dst_stride, radius=c.radius, corners=c.corners,
-            dimx=(c.dimx if c.pattern == cd.PATTERN_HALO else 0), dimy=c.dimy, pitch=self.pitch, index=idx,
+            dimx=(c.dimx if c.pattern == cd.PATTERN_HALO else 0), dimy=c.dimy, pitch=self.pitch,
+            dst_pitch=self.dst_pitch, index=idx,
             src_origin=src_origin, dst_origin=dst_origin, map_len=self.lds_bytes)
 
 

@@ -26,6 +26,7 @@ _SIGS = {
     "oracle_gather": (None, [_vp, _vp, _vp, _ci, _ci, _ci]),
     "oracle_scatter": (None, [_vp, _vp, _vp, _ci, _ci, _ci]),
     "oracle_halo": (None, [_vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci]),
+    "oracle_halo_pitched": (None, [_vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci, _ci]),
     "oracle_halo_check": (_ci, [_vp, _vp, _ci, _ci, _ci, _ci, _ci, _ci]),
     "oracle_copy": (None, [_vp, _vp, _cs]),
     "oracle_transpose": (None, [_vp, _vp, _ci]),

@@ -18,8 +18,11 @@ _CASES = cd.harness.all_cases()
 
 def _styles(case):
     styles = [cd.CALL_UNQUALIFIED, cd.CALL_GLOBAL, cd.CALL_QUALIFIED]
+    # the qualifier matrix of include/cudaDMAv2.h:50-63: every load qualifier from a source known to be global
+    # and from a generic one, every store qualifier of the reference
+    styles += list(cd.CALL_MATRIX_GLOBAL) + list(cd.CALL_MATRIX_GENERIC)
     if case.pattern in (cd.PATTERN_SEQUENTIAL, cd.PATTERN_STRIDED, cd.PATTERN_GATHER) and case.alignment in (4, 16):
-        styles.append(cd.CALL_LDS_DIRECT)
+        styles += [cd.CALL_LDS_DIRECT, cd.CALL_LDS_DIRECT_SC1, cd.CALL_LDS_DIRECT_NT]
     if case.pattern == cd.PATTERN_STRIDED and case.bytes_per_elmt % case.alignment == 0:
         styles.append(cd.CALL_LDS_SWIZZLE)                    # permuted chunks, through registers
         if case.alignment in (4, 16):
@@ -45,7 +48,8 @@ def test_case_matches_oracle(case_id, device):
                                     src_offset_bytes=io.src_offset, dst_offset_bytes=io.dst_offset,
                                     src_stride=io.src_stride, dst_stride=io.dst_stride, pitch=io.pitch,
                                     call_style=style, two_phase=two_phase, reps=io.reps,
-                                    rep_src_bytes=io.rep_src_bytes, rep_index_elmts=io.rep_index_elmts)
+                                    rep_src_bytes=io.rep_src_bytes, rep_index_elmts=io.rep_index_elmts,
+                                    dst_pitch=io.dst_pitch)
                 torch.cuda.synchronize()
                 got = d_out.cpu().numpy().reshape(io.reps, io.lds_bytes)
                 if not np.array_equal(got, want):
@@ -60,7 +64,12 @@ def test_case_reverse_direction_matches_oracle(case_id, device):
     """The same objects moving LDS -> global through the generic-pointer calls: the reference's
     ld/st wrappers are direction-agnostic (include/cudaDMAv2.h:107-114,553-558), its tests never try it."""
     case = _CASES[case_id]
-    for flavour, two_phase in ((0, False), (1, True)):
+    # the unqualified calls, and two of the four qualified calls that take a generic source (the pair rotates with
+    # the case number): there the store qualifier acts on global memory
+    generic = cd.CALL_MATRIX_GENERIC
+    plan = ((0, False, cd.CALL_UNQUALIFIED), (1, True, cd.CALL_UNQUALIFIED),
+            (2, bool(case_id & 1), generic[case_id % 4]), (3, not (case_id & 1), generic[(case_id + 2) % 4]))
+    for flavour, two_phase, style in plan:
         io = CaseIO(case, flavour=flavour, reps=2, data="uniform", reverse=True)
         if io.lds_bytes > 64 * 1024 - 256:
             pytest.skip("source image does not fit the harness LDS window")
@@ -68,18 +77,18 @@ def test_case_reverse_direction_matches_oracle(case_id, device):
         d_in = torch.from_numpy(io.input).to(device)
         d_idx = torch.from_numpy(io.index).to(device) if io.index is not None else None
         d_out = torch.zeros(io.reps * io.out_bytes, dtype=torch.uint8, device=device)
-        print(f"reverse case {case_id} two_phase {two_phase} {case}", flush=True)
+        print(f"reverse case {case_id} style {style} two_phase {two_phase} {case}", flush=True)
         cd.harness.run_case(case_id, d_in, d_out, lds_bytes=io.lds_bytes, d_index=d_idx,
                             src_offset_bytes=io.src_offset, dst_offset_bytes=io.dst_offset,
                             src_stride=io.src_stride, dst_stride=io.dst_stride, pitch=io.pitch,
-                            call_style=cd.CALL_UNQUALIFIED, two_phase=two_phase, reps=io.reps,
+                            call_style=style, two_phase=two_phase, reps=io.reps,
                             rep_src_bytes=io.rep_src_bytes, rep_index_elmts=io.rep_index_elmts,
-                            reverse=True, out_bytes=io.out_bytes)
+                            reverse=True, out_bytes=io.out_bytes, dst_pitch=io.dst_pitch)
         torch.cuda.synchronize()
         got = d_out.cpu().numpy().reshape(io.reps, io.out_bytes)
         if not np.array_equal(got, want):
             bad = np.argwhere(got != want)
-            raise AssertionError(f"two_phase {two_phase}: {len(bad)} wrong bytes, first at rep {bad[0][0]} byte {bad[0][1]}")
+            raise AssertionError(f"style {style} two_phase {two_phase}: {len(bad)} wrong bytes, first at rep {bad[0][0]} byte {bad[0][1]}")
 
 
 def _runtime_draw(case, rng):
@@ -144,7 +153,8 @@ def test_runtime_parameters_swept(case_id, device):
                             src_offset_bytes=io.src_offset, dst_offset_bytes=io.dst_offset,
                             src_stride=io.src_stride, dst_stride=io.dst_stride, pitch=io.pitch,
                             call_style=style, two_phase=two_phase, reps=io.reps,
-                            rep_src_bytes=io.rep_src_bytes, rep_index_elmts=io.rep_index_elmts, **kw)
+                            rep_src_bytes=io.rep_src_bytes, rep_index_elmts=io.rep_index_elmts,
+                            dst_pitch=io.dst_pitch, **kw)
         torch.cuda.synchronize()
         got = d_out.cpu().numpy().reshape(io.reps, io.lds_bytes)
         if not np.array_equal(got, want):
@@ -186,14 +196,39 @@ def test_halo_case_passes_the_reference_checker(device):
     assert ran >= 4
 
 
-def test_unmatched_waits_end(device):
+def test_unmatched_waits_end_and_are_reported(device):
     """Unbalanced start_async_dma / finish_async_dma counts must not hang the GPU: with the poll limit
-    forced down from the host side both waits give up and the kernel finishes."""
+    forced down from the host side both waits give up, the kernel finishes, and the failure record says
+    that two wavefronts gave up (the reference would hang; its DEBUG_CUDADMA build asserts,
+    include/cudaDMAv2.h:1564-1576)."""
     import ctypes
+    assert cd.device_status(clear=True) == (0, 0)
     flags = torch.zeros(2, dtype=torch.int32, device=device)
     cd._lib.check(cd.lib().cudadma_selftest_bounded_wait(ctypes.c_void_p(flags.data_ptr()), None))
     torch.cuda.synchronize()
     assert flags.tolist() == [1, 1]
+    bits, waves = cd.device_status(clear=False)
+    assert bits == cd.STATUS_WAIT_GAVE_UP and waves == 2
+    assert cd.device_status(clear=True) == (cd.STATUS_WAIT_GAVE_UP, 2)     # the record stays until it is cleared
+    assert cd.device_status(clear=True) == (0, 0)
+
+
+def test_every_translation_unit_with_dma_objects_reports(device):
+    assert cd.lib().cudadma_device_status_sources() >= 20
+
+
+@pytest.mark.parametrize("entry", ["cudadma_selftest_global_handoff", "cudadma_selftest_global_handoff_lds_only"])
+def test_global_memory_crosses_the_handshake(device, entry):
+    """Global memory written before a signal is seen after the matching wait, in both directions: the compute
+    wavefront produces the source in global memory, the DMA wavefronts move it global -> global, the compute
+    wavefront reads the destination (bar.sync / bar.arrive order all memory, include/cudaDMAv2.h:65-75).
+    Both builds of the fences must pass on this chip: they wait the same way."""
+    import ctypes
+    scratch = torch.zeros(4096, dtype=torch.int32, device=device)
+    wrong = torch.zeros(1, dtype=torch.int32, device=device)
+    cd._lib.check(getattr(cd.lib(), entry)(ctypes.c_void_p(scratch.data_ptr()), ctypes.c_void_p(wrong.data_ptr()), 300, None))
+    torch.cuda.synchronize()
+    assert wrong.item() == 0
 
 
 def test_split_wait_sees_every_phase(device):

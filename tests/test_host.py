@@ -239,3 +239,86 @@ def test_headers_compile_standalone_for_gfx950(tmp_path, header, flags):
            "-I", os.path.join(ROOT, "include"), "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"] + flags
     res = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
     assert res.returncode == 0, res.stderr[-2000:]
+
+
+# ---- the harness refuses, on the host, a run whose transfer would leave the caller's buffers ----
+def _fake_run(case_id, case, io, **over):
+    """cudadma_run_case with pointers that are never dereferenced: every refusal tested here happens before
+    the first HIP call."""
+    import ctypes
+    from cudadma_amd._lib import RunArgs
+    kw = dict(d_in=0x10000, d_out=0x20000, d_index=0, lds_bytes=io.lds_bytes, src_offset_bytes=io.src_offset,
+              dst_offset_bytes=io.dst_offset, src_stride=io.src_stride, dst_stride=io.dst_stride, pitch=io.pitch,
+              call_style=cd.CALL_UNQUALIFIED, two_phase=0, reps=io.reps, rep_src_bytes=io.rep_src_bytes,
+              rep_index_elmts=io.rep_index_elmts, reverse=0, out_bytes=0, dst_pitch=io.dst_pitch,
+              in_bytes=io.input.size, out_capacity=io.reps * io.lds_bytes, index_elmts=0)
+    kw.update(over)
+    r = RunArgs(**kw)
+    return cd.lib().cudadma_run_case(case_id, ctypes.byref(r), None), cd.lib().cudadma_last_error().decode()
+
+
+@pytest.mark.parametrize("pattern", [cd.PATTERN_SEQUENTIAL, cd.PATTERN_STRIDED, cd.PATTERN_HALO])
+def test_run_case_refuses_transfers_that_leave_the_buffers(pattern):
+    from tests.cases import CaseIO
+    cases = cd.harness.all_cases()
+    case_id = next(i for i, c in enumerate(cases) if c.pattern == pattern and c.level >= 2 and c.bytes_per_elmt > 0
+                   and (c.num_elmts > 1 or pattern != cd.PATTERN_STRIDED))
+    case = cases[case_id]
+    io = CaseIO(case, flavour=0, reps=2)
+    ERANGE = -3
+    rc, msg = _fake_run(case_id, case, io, in_bytes=io.input.size // 2)
+    assert rc == ERANGE and "input buffer" in msg, msg
+    rc, msg = _fake_run(case_id, case, io, lds_bytes=(io.lds_bytes // 2) // 16 * 16, out_capacity=io.reps * io.lds_bytes)
+    assert rc == ERANGE and "LDS window" in msg, msg
+    rc, msg = _fake_run(case_id, case, io, out_capacity=io.reps * io.lds_bytes - 16)
+    assert rc == ERANGE and "out_capacity" in msg, msg
+    if pattern == cd.PATTERN_STRIDED:
+        rc, msg = _fake_run(case_id, case, io, src_stride=io.src_stride * 4)
+        assert rc == ERANGE and "input buffer" in msg, msg
+        rc, msg = _fake_run(case_id, case, io, dst_stride=io.dst_stride * 4)
+        assert rc == ERANGE and "LDS window" in msg, msg
+    if pattern == cd.PATTERN_HALO:
+        rc, msg = _fake_run(case_id, case, io, pitch=io.pitch * 3)
+        assert rc == ERANGE and "input buffer" in msg, msg
+        rc, msg = _fake_run(case_id, case, io, dst_pitch=(case.dimx + 2 * case.radius) * 3)
+        assert rc == ERANGE and "LDS window" in msg, msg
+        rc, msg = _fake_run(case_id, case, io, dst_pitch=case.dimx + 2 * case.radius - 1)
+        assert rc == -1 and "dst_pitch" in msg, msg
+
+
+def test_run_case_refuses_a_short_index_list():
+    from tests.cases import CaseIO
+    cases = cd.harness.all_cases()
+    case_id = next(i for i, c in enumerate(cases) if c.pattern == cd.PATTERN_GATHER and c.num_elmts > 2)
+    io = CaseIO(cases[case_id], flavour=0, reps=2)
+    rc, msg = _fake_run(case_id, cases[case_id], io, d_index=0x30000, index_elmts=cases[case_id].num_elmts)
+    assert rc == -3 and "index_elmts" in msg, msg
+
+
+def test_plan_extents_are_the_footprint_of_the_closed_form():
+    """cudadma_plan_extents (the replay the harness checks buffers with) against the footprint the oracle's
+    closed form writes, for every compiled case."""
+    from tests.cases import CaseIO
+    for case in cd.harness.all_cases():
+        io = CaseIO(case, flavour=2, reps=1)
+        want = io.expected_map()
+        touched = np.flatnonzero(want >= 0)
+        idx = io.index[:case.num_elmts] if io.index is not None else None
+        ext = cd.plan.plan_extents(case.pattern, alignment=case.alignment, bytes_per_thread=case.bytes_per_thread,
+                                   bytes_per_elmt=case.bytes_per_elmt, dma_threads=case.dma_threads,
+                                   num_elmts=case.num_elmts, src_stride=io.src_stride, dst_stride=io.dst_stride,
+                                   radius=case.radius, corners=case.corners,
+                                   dimx=(case.dimx if case.pattern == cd.PATTERN_HALO else 0), dimy=case.dimy,
+                                   pitch=io.pitch, dst_pitch=io.dst_pitch, index=idx) \
+            if not (idx is not None and case.num_elmts == 0) else (0, 0, 0, 0)
+        dst_origin = io.dst_offset
+        src_origin = io.src_offset
+        if case.pattern == cd.PATTERN_HALO:
+            dst_origin += (case.radius * io.dst_cells + case.radius) * case.bytes_per_elmt
+            src_origin += (case.radius * io.pitch + case.radius) * case.bytes_per_elmt
+        if touched.size == 0:
+            assert ext[3] == ext[2]
+            continue
+        assert (dst_origin + ext[2], dst_origin + ext[3]) == (touched[0], touched[-1] + 1), case
+        src_bytes = want[touched]
+        assert (src_origin + ext[0], src_origin + ext[1]) == (src_bytes.min(), src_bytes.max() + 1), case

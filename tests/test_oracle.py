@@ -185,6 +185,35 @@ def test_halo_matches_the_reference_checker(O, es, radius, corners, dimx, dimy, 
     assert not numpy_check_halo(idata, bad, radius, corners, dimx, dimy, pitch)
 
 
+@pytest.mark.parametrize("es", [4, 8, 16])
+@pytest.mark.parametrize("radius,corners,dimx,dimy,extra,dst_extra", [(1, 0, 8, 8, 0, 1), (3, 1, 17, 9, 5, 3), (4, 0, 32, 32, 0, 8),
+                                                                      (8, 1, 63, 20, 3, 1), (2, 1, 13, 21, 1, 0)])
+def test_halo_with_a_destination_pitch(O, es, radius, corners, dimx, dimy, extra, dst_extra):
+    """oracle_halo_pitched against numpy slicing of the two padded tiles: the ring lands in rows of dst_pitch
+    cells, nothing else is written, and dst_pitch = dimx + 2*radius is oracle_halo itself."""
+    cells = es // 4
+    pitch = dimx + 2 * radius + extra
+    dst_pitch = dimx + 2 * radius + dst_extra
+    rows = dimy + 2 * radius
+    rng = np.random.default_rng(radius * 31 + dimx + dst_extra)
+    idata = rng.integers(1, 1000, size=(rows, pitch, cells)).astype(np.float32)
+    odata = np.zeros((rows, dst_pitch, cells), dtype=np.float32)
+    O.oracle_halo_pitched(ptr(idata, (radius * pitch + radius) * es), ptr(odata, (radius * dst_pitch + radius) * es),
+                          es, radius, corners, dimx, dimy, pitch, dst_pitch)
+    want = np.zeros_like(odata)
+    c0, c1 = (0, dimx + 2 * radius) if corners else (radius, radius + dimx)
+    want[:radius, c0:c1] = idata[:radius, c0:c1]
+    want[radius + dimy:, c0:c1] = idata[radius + dimy:, c0:c1]
+    want[radius:radius + dimy, :radius] = idata[radius:radius + dimy, :radius]
+    want[radius:radius + dimy, radius + dimx:2 * radius + dimx] = idata[radius:radius + dimy, radius + dimx:2 * radius + dimx]
+    assert np.array_equal(odata, want)
+    if dst_extra == 0:
+        ref = np.zeros_like(odata)
+        O.oracle_halo(ptr(idata, (radius * pitch + radius) * es), ptr(ref, (radius * dst_pitch + radius) * es),
+                      es, radius, corners, dimx, dimy, pitch)
+        assert np.array_equal(ref, odata)
+
+
 # ------------------------------------------------------------------ workloads
 def test_copy_and_transpose(O):
     a = ol.uniform(256 * 256, 1002).reshape(256, 256)

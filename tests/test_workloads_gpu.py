@@ -184,8 +184,13 @@ def test_gather_full_size(device):
     for r in range(1, wl.RECS_PER_TILE):
         acc = acc + t[:, r, :]
     assert np.array_equal(sums.view(-1, wl.REC_FLOATS)[sample].cpu().numpy().view(np.uint32), acc.view(np.uint32))
-    # duplicates are really there
-    assert int((idx[1025:100000] == idx[1024:99999]).sum()) >= 0
+    # one draw in ten repeats one of the 1024 draws before it (the "10 % duplicates" of the configuration): count the
+    # positions of the device-generated list whose value already occurs among the 1024 before it; chance adds
+    # 1024 / 4 Mi = 0.02 % of the positions
+    sample = idx[:1 << 18].cpu().numpy()
+    windows = np.lib.stride_tricks.sliding_window_view(sample, 1025)[::37]          # [..., :1024] before, [..., 1024] the draw
+    rate = float((windows[:, :1024] == windows[:, 1024:]).any(axis=1).mean())
+    assert 0.07 <= rate <= 0.13, rate
     # empty index list is a no-op
     wl.gather_copy(table, idx[:0], out[:0], 0)
 
@@ -269,12 +274,13 @@ def test_halo_stencil_small(device, variant, shape):
     assert np.all(err <= STENCIL_RTOL * np.maximum(np.abs(want), 1.0)), float(err.max())
 
 
-def test_halo_stencil_full_size(device):
+@pytest.mark.parametrize("variant", [0, 1])     # the kernel the benchmark reports and its form with the empty/full handshake
+def test_halo_stencil_full_size(device, variant):
     n = 512
     p = 2 * wl.STENCIL_RADIUS
     d_in = wl.fill_uniform(torch.empty((n + p) ** 3, dtype=torch.float32, device=device), 1004).view(n + p, n + p, n + p)
     d_out = torch.empty((n, n, n), dtype=torch.float32, device=device)
-    wl.halo_stencil(d_in, d_out, 0)
+    wl.halo_stencil(d_in, d_out, variant)
     torch.cuda.synchronize()
     # slabs of the host statement
     g = ol.uniform((n + p) ** 3, 1004).reshape(n + p, n + p, n + p)
@@ -285,13 +291,25 @@ def test_halo_stencil_full_size(device):
         assert np.all(np.abs(got - want) <= STENCIL_RTOL * np.maximum(np.abs(want), 1.0))
     # a constant field has zero Laplacian everywhere (catches a wrong tile or plane anywhere in the grid)
     d_in.fill_(1.0)
-    wl.halo_stencil(d_in, d_out, 0)
+    wl.halo_stencil(d_in, d_out, variant)
     torch.cuda.synchronize()
     assert float(d_out.abs().max()) <= 1e-5
 
 
 # ------------------------------------------------------------------ config 5
 GEMM_RTOL = 1e-2          # benchmark config 5: within 1e-2 relative of the fp32 host GEMM
+
+
+def test_device_normal_bf16_generator_matches_the_host_statement(device):
+    """cudadma_fill_normal_bf16 (what the benchmark's GEMM inputs come from, seeds 1005 and 2005) bit for bit against
+    the oracle's generator."""
+    n = 1 << 20
+    for seed in (1005, 2005):
+        want = np.empty(n, dtype=np.uint16)
+        ol.load().oracle_fill_normal_bf16(ptr(want), n, seed)
+        got = wl.fill_normal_bf16(torch.empty(n, dtype=torch.bfloat16, device=device), seed)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16), want)
 
 
 def _bf16_inputs(m, n, k):
