@@ -28,7 +28,7 @@ struct Knob {
   const char* name;
   std::atomic<int> value;
 };
-static Knob g_knobs[] = {{"transpose_band", {0}}, {"transpose_workgroups", {0}}, {"stencil_zchunk", {0}}, {"stencil_xcd_remap", {0}}};
+static Knob g_knobs[] = {{"transpose_band", {0}}, {"transpose_workgroups", {0}}, {"transpose_split", {0}}, {"stencil_zchunk", {0}}, {"stencil_xcd_remap", {0}}};
 
 static Knob* find_knob(const char* name)
 {
@@ -45,11 +45,14 @@ int tuning(const char* name, int fallback)
 }
 
 static const VariantInfo kSequential[] = {
-  {"manual double buffer: one DMA group of 2 wavefronts, two objects, two-phase calls, registers -> ds_write_b128"},
+  {"manual double buffer: one DMA group of 2 wavefronts, two objects, two-phase calls, registers -> ds_write_b128, four "
+   "workgroups per compute unit; for more than 96 MiB (a working set beyond the Infinity Cache) variant 5 instead"},
   {"single buffer: one object, execute_dma"},
   {"double buffer: two DMA groups of 1 wavefront, one object each"},
   {"manual double buffer with STORE_LDS_DIRECT (global_load_lds_dwordx4, no VGPR staging)"},
   {"no DMA object: every wavefront copies global -> LDS -> global between workgroup barriers"},
+  {"single buffer (the next tile waits in the DMA wavefronts' registers), two workgroups per compute unit, streaming "
+   "loads and non-temporal stores: the shape for buffers beyond the Infinity Cache"},
 };
 static const VariantInfo kStrided[] = {
   {"manual double buffer: one DMA group of 2 wavefronts, two CudaDMAStrided objects, padded LDS rows (272 B)"},
@@ -67,6 +70,10 @@ static const VariantInfo kStrided[] = {
   {"one DMA wavefront and one compute wavefront per workgroup, two objects of a whole tile each on the DMA "
    "wavefront, two LDS tiles; dword stores"},
   {"as variant 8 with the quad transposition and dwordx4 stores of variant 7"},
+  {"variant 1 with the split of the workgroup as a knob (\"transpose_split\" = 100 x DMA wavefronts + 10 x compute "
+   "wavefronts + tiles requested ahead; default 311: three DMA wavefronts, one compute wavefront, one tile ahead, "
+   "the fastest of the 22 splits compiled): one LDS tile guarded by a sync-only object, one or two CudaDMAStrided "
+   "objects without a handshake of their own on the DMA wavefronts; the kernel the benchmark reports"},
 };
 static const VariantInfo kGather[] = {
   {"manual 4-stage buffering: one DMA group of 2 wavefronts, four CudaDMAIndirect objects"},

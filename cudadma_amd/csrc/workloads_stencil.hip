@@ -209,11 +209,12 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kXQ = kTX / 4;                          // 8 threads per tile row
 constexpr int kPrefetch = 3;
-constexpr int kQueue = 2 * kR + 1 + kPrefetch;        // planes held in registers: 12
+constexpr int kQueue = 2 * kR + 1 + kPrefetch;        // planes held in registers: 12 (the kernels take it as QUEUE; deeper
+                                                      // queues ran slower: 16 planes 0.248 ms against 0.200 ms at 512^3)
 // The z column is a ring of registers: plane z + p of the chunk sits in slot
 // (z + p) % kQueue, and the z loop is unrolled kQueue times so that every slot
 // number is a compile-time constant and no plane is ever moved between registers.
-#define HIPDMA_QSLOT(ROT, P) (((ROT) + (P)) % kQueue)
+#define HIPDMA_QSLOT(ROT, P) (((ROT) + (P)) % QUEUE)
 
 enum SyncMode {
   kHandshakeAndBarrier = 0,   // empty/full handshake + one s_barrier per plane (DMA wavefront joins it)
@@ -243,58 +244,102 @@ __device__ __forceinline__ int tile_row_of_thread()
   return 16 * (wave / 2) + 2 * (wave % 2) + (j / 4) + 4 * (j % 4);
 }
 
-template<int ROT>
-__device__ __forceinline__ f32x4_t stencil_cells4(const float* __restrict__ plane, const int lx, const int ly,
-                                                  const f32x4_t (&q)[kQueue], const Coeffs& k)
+// The x and y neighbours of a thread's four cells, as they come out of the LDS plane: ten ds_read_b128.
+// Named members, not arrays: the values have to live in registers across the hand-off that sits between
+// the reads and the arithmetic, and an array inside a struct ends up in scratch memory here.
+struct Neighbours {
+  f32x4_t xl, xr, up1, up2, up3, up4, dn1, dn2, dn3, dn4;
+  template<int R> __device__ __forceinline__ const f32x4_t& up() const
+  { if constexpr (R == 1) return up1; else if constexpr (R == 2) return up2; else if constexpr (R == 3) return up3; else return up4; }
+  template<int R> __device__ __forceinline__ const f32x4_t& dn() const
+  { if constexpr (R == 1) return dn1; else if constexpr (R == 2) return dn2; else if constexpr (R == 3) return dn3; else return dn4; }
+};
+static_assert(kR == 4, "Neighbours names four rows above and four below");
+__device__ __forceinline__ Neighbours stencil_fetch4(const float* __restrict__ plane, const int lx, const int ly)
+{
+  const float* c = plane + (ly + kR) * kPitch + (lx + kR);
+  Neighbours n;
+  n.xl = *(const f32x4_t*)(c - 4);
+  n.xr = *(const f32x4_t*)(c + 4);
+  n.up1 = *(const f32x4_t*)(c - 1 * kPitch);
+  n.dn1 = *(const f32x4_t*)(c + 1 * kPitch);
+  n.up2 = *(const f32x4_t*)(c - 2 * kPitch);
+  n.dn2 = *(const f32x4_t*)(c + 2 * kPitch);
+  n.up3 = *(const f32x4_t*)(c - 3 * kPitch);
+  n.dn3 = *(const f32x4_t*)(c + 3 * kPitch);
+  n.up4 = *(const f32x4_t*)(c - 4 * kPitch);
+  n.dn4 = *(const f32x4_t*)(c + 4 * kPitch);
+  return n;
+}
+
+// One radius of the sum for cell I: same operations in the same order as the host statement.
+template<int ROT, int QUEUE, int I, int R>
+__device__ __forceinline__ float stencil_term(const Neighbours& n, const float (&xs)[12], const f32x4_t (&q)[QUEUE],
+                                              const float coeff, const float acc)
 {
 #pragma clang fp contract(off)
-  const float* c = plane + (ly + kR) * kPitch + (lx + kR);
-  const float cr[5] = {0.0f, k.c1, k.c2, k.c3, k.c4};
+  const float sx = xs[4 + I - R] + xs[4 + I + R];
+  const float sy = n.template up<R>()[I] + n.template dn<R>()[I];
+  const float sz = q[HIPDMA_QSLOT(ROT, kR - R)][I] + q[HIPDMA_QSLOT(ROT, kR + R)][I];
+  return __builtin_fmaf(coeff, (sx + sy) + sz, acc);
+}
+template<int ROT, int QUEUE, int I>
+__device__ __forceinline__ float stencil_cell_i(const Neighbours& n, const float (&xs)[12], const f32x4_t (&q)[QUEUE],
+                                                const Coeffs& k)
+{
+#pragma clang fp contract(off)
+  float acc = k.c0 * xs[4 + I];
+  acc = stencil_term<ROT, QUEUE, I, 1>(n, xs, q, k.c1, acc);
+  acc = stencil_term<ROT, QUEUE, I, 2>(n, xs, q, k.c2, acc);
+  acc = stencil_term<ROT, QUEUE, I, 3>(n, xs, q, k.c3, acc);
+  acc = stencil_term<ROT, QUEUE, I, 4>(n, xs, q, k.c4, acc);
+  return acc;
+}
+
+template<int ROT, int QUEUE>
+__device__ __forceinline__ f32x4_t stencil_eval4(const Neighbours& n, const f32x4_t (&q)[QUEUE], const Coeffs& k)
+{
   // x neighbourhood: 4 cells left, the centre cells, 4 cells right
-  const f32x4_t xl = *(const f32x4_t*)(c - 4);
   const f32x4_t xc = q[HIPDMA_QSLOT(ROT, kR)];
-  const f32x4_t xr = *(const f32x4_t*)(c + 4);
-  const float xs[12] = {xl[0], xl[1], xl[2], xl[3], xc[0], xc[1], xc[2], xc[3], xr[0], xr[1], xr[2], xr[3]};
-  f32x4_t up[kR], dn[kR];
-#pragma unroll
-  for (int r = 1; r <= kR; ++r) {
-    up[r - 1] = *(const f32x4_t*)(c - r * kPitch);
-    dn[r - 1] = *(const f32x4_t*)(c + r * kPitch);
-  }
+  const float xs[12] = {n.xl[0], n.xl[1], n.xl[2], n.xl[3], xc[0], xc[1], xc[2], xc[3], n.xr[0], n.xr[1], n.xr[2], n.xr[3]};
   f32x4_t out;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    float acc = k.c0 * xc[i];
-#pragma unroll
-    for (int r = 1; r <= kR; ++r) {
-      const float sx = xs[4 + i - r] + xs[4 + i + r];
-      const float sy = up[r - 1][i] + dn[r - 1][i];
-      const float sz = q[HIPDMA_QSLOT(ROT, kR - r)][i] + q[HIPDMA_QSLOT(ROT, kR + r)][i];
-      acc = __builtin_fmaf(cr[r], (sx + sy) + sz, acc);
-    }
-    out[i] = acc;
-  }
+  out[0] = stencil_cell_i<ROT, QUEUE, 0>(n, xs, q, k);
+  out[1] = stencil_cell_i<ROT, QUEUE, 1>(n, xs, q, k);
+  out[2] = stencil_cell_i<ROT, QUEUE, 2>(n, xs, q, k);
+  out[3] = stencil_cell_i<ROT, QUEUE, 3>(n, xs, q, k);
   return out;
+}
+
+template<int ROT, int QUEUE>
+__device__ __forceinline__ f32x4_t stencil_cells4(const float* __restrict__ plane, const int lx, const int ly,
+                                                  const f32x4_t (&q)[QUEUE], const Coeffs& k)
+{
+  return stencil_eval4<ROT, QUEUE>(stencil_fetch4(plane, lx, ly), q, k);
 }
 
 // Runs the body for z = 0 .. planes-1 with ROT = z % kQueue as a constant.  Whole
 // groups of kQueue planes run without a single branch, so the compiler's
 // s_waitcnt placement can count exactly how many younger loads and stores may
 // stay in flight; only the last, partial group checks the plane count.
-#define HIPDMA_Z_STEP(J, CHECK, ...) if (!(CHECK) || z0 + (J) < planes) { constexpr int ROT = (J); const int z = z0 + (J); __VA_ARGS__ }
+#define HIPDMA_Z_STEP(J, CHECK, ...) if constexpr ((J) < QUEUE) { if (!(CHECK) || z0 + (J) < planes) { constexpr int ROT = (J); const int z = z0 + (J); __VA_ARGS__ } }
 #define HIPDMA_Z_GROUP(CHECK, ...)                                                                       \
   HIPDMA_Z_STEP(0, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(1, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(2, CHECK, __VA_ARGS__)   \
   HIPDMA_Z_STEP(3, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(4, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(5, CHECK, __VA_ARGS__)   \
   HIPDMA_Z_STEP(6, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(7, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(8, CHECK, __VA_ARGS__)   \
-  HIPDMA_Z_STEP(9, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(10, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(11, CHECK, __VA_ARGS__)
+  HIPDMA_Z_STEP(9, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(10, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(11, CHECK, __VA_ARGS__) \
+  HIPDMA_Z_STEP(12, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(13, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(14, CHECK, __VA_ARGS__) \
+  HIPDMA_Z_STEP(15, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(16, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(17, CHECK, __VA_ARGS__) \
+  HIPDMA_Z_STEP(18, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(19, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(20, CHECK, __VA_ARGS__) \
+  HIPDMA_Z_STEP(21, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(22, CHECK, __VA_ARGS__) HIPDMA_Z_STEP(23, CHECK, __VA_ARGS__)
 #define HIPDMA_FOR_Z(planes_expr, ...)                                       \
   {                                                                          \
     const int planes = (planes_expr);                                        \
     int z0 = 0;                                                              \
-    for (; z0 + kQueue <= planes; z0 += kQueue) { HIPDMA_Z_GROUP(false, __VA_ARGS__) } \
+    for (; z0 + QUEUE <= planes; z0 += QUEUE) { HIPDMA_Z_GROUP(false, __VA_ARGS__) } \
     if (z0 < planes) { HIPDMA_Z_GROUP(true, __VA_ARGS__) }                   \
   }
-static_assert(kQueue == 12 && kQueue % 4 == 0, "HIPDMA_FOR_Z unrolls twelve steps; the LDS planes rotate with period 4");
+// HIPDMA_FOR_Z unrolls QUEUE (at most 24) steps; the LDS planes rotate with period 4, so QUEUE is a multiple of 4
+template<int QUEUE> struct queue_ok { static_assert(QUEUE >= 2 * kR + 2 && QUEUE <= 24 && QUEUE % 4 == 0, "QUEUE: 12, 16, 20 or 24"); };
 
 // The DMA wavefront keeps the rings of the next kRingAhead planes in flight,
 // each in the registers of its own CudaDMAHalo object (manual buffering with
@@ -307,7 +352,11 @@ static_assert(kQueue == 12 && kQueue % 4 == 0, "HIPDMA_FOR_Z unrolls twelve step
 // the sync-only class of include/cudaDMA.h:4184-4208.
 constexpr int kBufs = 4;
 constexpr int kRingObjs = 8;
-constexpr int kRingAhead = kRingObjs - 1;
+#ifndef STENCIL_RING_AHEAD
+#define STENCIL_RING_AHEAD (kRingObjs - 1)
+#endif
+constexpr int kRingAhead = STENCIL_RING_AHEAD;
+static_assert(kRingAhead >= 2 && kRingAhead < kRingObjs, "a ring has to be requested before it lands and needs an object of its own");
 typedef CudaDMAHalo<false, 16, 32, 4, kDmaThreads, kR, false, kTX, kTY> halo_reg_t;
 
 template<typename T>
@@ -344,8 +393,10 @@ struct Four {
   }
 static_assert(kRingObjs == 8 && kRingObjs % kBufs == 0, "HIPDMA_FOR_RING unrolls eight steps");
 
-template<int SYNC>
-__global__ void __launch_bounds__(kComputeThreads + kDmaThreads)
+// One workgroup of five wavefronts per compute unit is the operating point: at most two wavefronts share a
+// SIMD, so the register allocator may use 256 registers per lane instead of spilling to stay under 128.
+template<int SYNC, int QUEUE = kQueue>
+__global__ void __launch_bounds__(kComputeThreads + kDmaThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
 stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int nx, const int ny, const int nz,
                 const int zchunk, const Coeffs k)
 {
@@ -383,8 +434,13 @@ stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int
     // wavefronts then find the `full` word of a plane set when they first look, and never poll.
     constexpr int kLand = (SYNC == kBarrierOnly) ? 1 : 2;
     // planes 0 .. kRingAhead-1 are requested up front; planes 0 .. kLand-1 land before the first barrier
-    HIPDMA_ISSUE(0, 0) HIPDMA_ISSUE(1, 1) HIPDMA_ISSUE(2, 2) HIPDMA_ISSUE(3, 3)
-    HIPDMA_ISSUE(4, 4) HIPDMA_ISSUE(5, 5) HIPDMA_ISSUE(6, 6)
+    if constexpr (kRingAhead > 0) { HIPDMA_ISSUE(0, 0) }
+    if constexpr (kRingAhead > 1) { HIPDMA_ISSUE(1, 1) }
+    if constexpr (kRingAhead > 2) { HIPDMA_ISSUE(2, 2) }
+    if constexpr (kRingAhead > 3) { HIPDMA_ISSUE(3, 3) }
+    if constexpr (kRingAhead > 4) { HIPDMA_ISSUE(4, 4) }
+    if constexpr (kRingAhead > 5) { HIPDMA_ISSUE(5, 5) }
+    if constexpr (kRingAhead > 6) { HIPDMA_ISSUE(6, 6) }
     HIPDMA_LAND(0, 0)
     if constexpr (kLand == 2) { HIPDMA_LAND(1, 1) }
     // iteration z: request plane z + kRingAhead, meet the compute wavefronts, land plane z + kLand
@@ -398,12 +454,13 @@ stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int
   } else {
     const int lx = 4 * (threadIdx.x % kXQ);
     const int ly = tile_row_of_thread();
-    f32x4_t q[kQueue];
+    (void)sizeof(queue_ok<QUEUE>);
+    f32x4_t q[QUEUE];
     const float* col = w.in_origin + (size_t)ly * px + lx;
-    // planes 0 .. kQueue-2 of the chunk; every iteration fetches one more
+    // planes 0 .. QUEUE-2 of the chunk; every iteration fetches one more
     const int avail = w.planes + 2 * kR;                  // padded planes this chunk may touch
 #pragma unroll
-    for (int p = 0; p < kQueue - 1; ++p)
+    for (int p = 0; p < QUEUE - 1; ++p)
       q[p] = (p < avail) ? *(const f32x4_t*)(col + (size_t)p * in_plane) : f32x4_t{0.f, 0.f, 0.f, 0.f};
     if constexpr (SYNC != kBarrierOnly) {
       guard.a0.start_async_dma();
@@ -421,19 +478,23 @@ stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int
       constexpr int B = ROT % kBufs;
       const cudaDMACustom& cur_halo = guard.get<B>();
       // past the end of the chunk the last plane is fetched again: unconditional loads keep the wait counts exact
-      const int zf = (z + kQueue - 1 < avail) ? (z + kQueue - 1) : (avail - 1);
-      q[HIPDMA_QSLOT(ROT, kQueue - 1)] = *(const f32x4_t*)(col + (size_t)zf * in_plane);
+      const int zf = (z + QUEUE - 1 < avail) ? (z + QUEUE - 1) : (avail - 1);
+      q[HIPDMA_QSLOT(ROT, QUEUE - 1)] = *(const f32x4_t*)(col + (size_t)zf * in_plane);
       if constexpr (SYNC != kBarrierOnly) cur_halo.wait_for_dma_finish(seen);
       if constexpr (SYNC == kHandshakeAndGroupBarrier) compute_barrier.sync();
       else __syncthreads();
-      const f32x4_t r = stencil_cells4<ROT>(plane[B], lx, ly, q, k);
-      if constexpr (SYNC != kBarrierOnly) seen = guard.get<(B + 1) % kBufs>().peek_dma_finish();
+      // With the handshake the plane is released as soon as its ten reads have returned (the release fence waits
+      // for exactly those) and the `full` word of the next plane is requested right behind the signal: both LDS
+      // round trips then run under the arithmetic of this plane instead of after it.
+      const Neighbours nb = stencil_fetch4(plane[B], lx, ly);
+      if constexpr (SYNC != kBarrierOnly) {
+        cur_halo.start_async_dma();
+        seen = guard.get<(B + 1) % kBufs>().peek_dma_finish();
+      }
       *(f32x4_t*)(&plane[(B + 1) % kBufs][kOrigin] + ly * kPitch + lx) = q[HIPDMA_QSLOT(ROT, kR + 1)];
+      const f32x4_t r = stencil_eval4<ROT, QUEUE>(nb, q, k);
       __builtin_nontemporal_store(r, (f32x4_t*)o);     // the output is not read again: 3 % faster than a plain store
       o += out_plane;
-      // The plane is released last: the store above already had to wait for every LDS read of the
-      // plane, so the release fence finds nothing left to wait for.
-      if constexpr (SYNC != kBarrierOnly) cur_halo.start_async_dma();
     })
   }
 }
@@ -454,24 +515,25 @@ stencil_all_vec4(const float* __restrict__ in, float* __restrict__ out, const in
   float* lds_origin = &plane[kR * kPitch + kR];
   const int lx = 4 * (threadIdx.x % kXQ);
   const int ly = tile_row_of_thread();
-  f32x4_t q[kQueue];
+  constexpr int QUEUE = kQueue;
+  f32x4_t q[QUEUE];
   const float* col = w.in_origin + (size_t)ly * px + lx;
   const int avail = w.planes + 2 * kR;
 #pragma unroll
-  for (int p = 0; p < kQueue - 1; ++p)
+  for (int p = 0; p < QUEUE - 1; ++p)
     q[p] = (p < avail) ? *(const f32x4_t*)(col + (size_t)p * in_plane) : f32x4_t{0.f, 0.f, 0.f, 0.f};
   const float* ring0 = w.in_origin + (size_t)kR * in_plane;
   const int last = w.planes - 1;
   float* o = w.out_origin + (size_t)ly * nx + lx;
   halo.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(ring0);
   HIPDMA_FOR_Z(w.planes, {
-    const int zf = (z + kQueue - 1 < avail) ? (z + kQueue - 1) : (avail - 1);
-    q[HIPDMA_QSLOT(ROT, kQueue - 1)] = *(const f32x4_t*)(col + (size_t)zf * in_plane);
+    const int zf = (z + QUEUE - 1 < avail) ? (z + QUEUE - 1) : (avail - 1);
+    q[HIPDMA_QSLOT(ROT, QUEUE - 1)] = *(const f32x4_t*)(col + (size_t)zf * in_plane);
     halo.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(lds_origin);
     *(f32x4_t*)(lds_origin + ly * kPitch + lx) = q[HIPDMA_QSLOT(ROT, kR)];
     __syncthreads();
     halo.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(ring0 + (size_t)(z < last ? z + 1 : last) * in_plane);
-    *(f32x4_t*)o = stencil_cells4<ROT>(plane, lx, ly, q, k);
+    *(f32x4_t*)o = stencil_cells4<ROT, QUEUE>(plane, lx, ly, q, k);
     o += out_plane;
     __syncthreads();
   })
@@ -491,12 +553,11 @@ extern "C" int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int
   CUDADMA_REQUIRE(cudadma_host::aligned_to(d_in, 16) && cudadma_host::aligned_to(d_out, 16), "pointers must be 16-byte aligned");
   const Coeffs k = {(float)(3.0 * (-205.0 / 72.0)), (float)(8.0 / 5.0), (float)(-1.0 / 5.0), (float)(8.0 / 315.0),
                     (float)(-1.0 / 560.0)};
-  // z is cut into chunks so that a 512^3 grid yields a few thousand workgroups instead of 256
   // z is cut into as few chunks as still give every compute unit work: each chunk re-reads
-  // 2*radius + prefetch planes before it produces output.  The variants that pay for the
-  // handshake want two workgroups per compute unit to hide it, the others run best with one.
+  // 2*radius + prefetch planes before it produces output.  The dwordx4 kernels run best with one workgroup
+  // per compute unit, with and without the handshake (512^3: 0.200 / 0.206 ms against 0.228 / 0.222 ms with two).
   const long long tiles_xy = (long long)(nx / kTX) * (ny / kTY);
-  const int per_cu = (variant == 0 || variant == 3) ? 1 : 2;
+  const int per_cu = (variant <= 3) ? 1 : 2;
   long long want_chunks = ((long long)per_cu * workloads::device_cus() + tiles_xy - 1) / tiles_xy;
   if (want_chunks < 1) want_chunks = 1;
   int zchunk = workloads::tuning("stencil_zchunk", (int)((nz + want_chunks - 1) / want_chunks));

@@ -353,6 +353,82 @@ transpose_single(const float* __restrict__ in, float* __restrict__ out, const in
   }
 }
 
+// The single-tile kernel with the split of the workgroup between the two roles as a parameter: DW DMA wavefronts,
+// CW compute wavefronts, and AHEAD tiles requested beyond the one in LDS (1: what execute_dma does; 2: two objects
+// that share the DMA wavefronts and the LDS tile, each holding one requested tile in registers, in the manner of
+// src/examples/stencil/warp_specialized_manual_buffer.h:54-71).  The objects carry no handshake of their own; one
+// sync-only object guards the tile (include/cudaDMA.h:4184-4208).  Streaming loads, quad transposition, non-temporal
+// dwordx4 stores as in transpose_single<true, true>.
+template<int DW, int CW, int AHEAD>
+__global__ void __launch_bounds__((DW + CW) * 64)
+transpose_split(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles, const int band)
+{
+  static_assert(CW == 1 || CW == 2 || CW == 4, "the compute wavefronts share the sixteen 16-byte columns of a tile row evenly");
+  static_assert(AHEAD == 1 || AHEAD == 2, "one or two tiles requested ahead");
+  constexpr int kLdsRow = 272;
+  constexpr int kDma = DW * 64, kCompute = CW * 64;
+  constexpr int kChunks = kTile * kRowBytes / 16;
+  constexpr int kBpt = ((kChunks + kDma - 1) / kDma) * 16;
+  __shared__ __attribute__((aligned(16))) char buf[kTile * kLdsRow];
+  cudaDMACustom guard(0, kDma, kCompute, kCompute);
+  typedef CudaDMAStrided<false, 16, kBpt, kRowBytes, kDma, kTile> obj_t;
+  const int tiles_per_side = n / kTile;
+  const int stride = gridDim.x;
+  const int last = num_tiles - 1;
+  auto src_of = [&](const int t) {
+    int ty, tx;
+    tile_coords(t < num_tiles ? t : last, tiles_per_side, band, ty, tx);     // past the end: the last tile again, loads stay unconditional
+    return (const void*)(in + (size_t)ty * kTile * n + (size_t)tx * kTile);
+  };
+  if (guard.owns_this_thread()) {
+    obj_t a(n * 4, kLdsRow, kCompute), b(n * 4, kLdsRow, kCompute);
+    auto land = [&](obj_t& o) __attribute__((always_inline)) {
+      guard.wait_for_dma_start();
+      o.template wait_xfer_finish<true, LOAD_CACHE_STREAMING, STORE_LDS>(buf);
+      guard.finish_async_dma();
+    };
+    int t = blockIdx.x;
+    if (t >= num_tiles) return;
+    a.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t));
+    if constexpr (AHEAD == 2) b.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t + stride));
+    for (; t < num_tiles; t += AHEAD * stride) {
+      land(a);
+      a.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t + AHEAD * stride));
+      if constexpr (AHEAD == 2) {
+        if (t + stride < num_tiles) land(b);
+        b.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t + 3 * stride));
+      }
+    }
+  } else {
+    // lane = tile row; wavefront w takes the 16 / CW 16-byte columns [w * 16 / CW, (w + 1) * 16 / CW) of that row
+    constexpr int kUnits = 16 / CW;
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6;
+    guard.start_async_dma();
+    for (int t = blockIdx.x; t < num_tiles; t += stride) {
+      int ty, tx;
+      tile_coords(t, tiles_per_side, band, ty, tx);
+      guard.wait_for_dma_finish();
+      vec4_t v[kUnits];
+      const vec4_t* row = (const vec4_t*)(buf + lane * kLdsRow) + w * kUnits;
+#pragma unroll
+      for (int j = 0; j < kUnits; ++j) v[j] = row[j];
+      guard.start_async_dma();
+      float* o = out + (size_t)(tx * kTile + w * 4 * kUnits + (lane & 3)) * n + (size_t)ty * kTile + (lane & ~3);
+#pragma unroll
+      for (int j = 0; j < kUnits; ++j)
+        __builtin_nontemporal_store(quad_transpose(v[j], lane), (vec4_t*)(o + (size_t)(4 * j) * n));
+    }
+  }
+}
+
+typedef void (*split_kernel_t)(const float*, float*, int, int, int);
+struct SplitEntry { int dw, cw, ahead; split_kernel_t kernel; };
+#define SPLIT(DW, CW) {DW, CW, 1, transpose_split<DW, CW, 1>}, {DW, CW, 2, transpose_split<DW, CW, 2>}
+const SplitEntry kSplits[] = {SPLIT(2, 2), SPLIT(1, 1), SPLIT(1, 2), SPLIT(2, 1), SPLIT(3, 1), SPLIT(4, 1), SPLIT(3, 2), SPLIT(4, 2),
+                              SPLIT(1, 4), SPLIT(2, 4), SPLIT(4, 4)};
+#undef SPLIT
+
 }  // namespace
 
 extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n, int variant, void* stream)
@@ -371,7 +447,7 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
   // The kernels with one LDS tile (variants 1 and 4) run best with exactly one workgroup per compute unit, i.e. one
   // 16 KB tile of loads in flight per compute unit, and with the tiles walked down the columns (the workgroups that
   // run together then write whole output rows); the others with four workgroups and bands of 16 tile rows.
-  const bool one_tile = variant == 1 || variant == 4;
+  const bool one_tile = variant == 1 || variant == 4 || variant == 10;
   int band = workloads::tuning("transpose_band", one_tile ? tiles_per_side : kDefaultBand);
   if (band > tiles_per_side) band = tiles_per_side;
   while (band > 1 && tiles_per_side % band != 0) band /= 2;      // bands must tile the matrix
@@ -391,6 +467,16 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
     case 7: hipLaunchKernelGGL((transpose_manual_double<272, true>), grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 8: hipLaunchKernelGGL(transpose_pairs<false>, grid_for(4), dim3(128), 0, s, d_in, d_out, n, tiles, band); break;
     case 9: hipLaunchKernelGGL(transpose_pairs<true>, grid_for(4), dim3(128), 0, s, d_in, d_out, n, tiles, band); break;
+    case 10: {
+      // knob "transpose_split" = 100 * DMA wavefronts + 10 * compute wavefronts + tiles ahead (default 311, the fastest)
+      const int code = workloads::tuning("transpose_split", 311);
+      const SplitEntry* e = nullptr;
+      for (const SplitEntry& c : kSplits)
+        if (100 * c.dw + 10 * c.cw + c.ahead == code) e = &c;
+      CUDADMA_REQUIRE(e != nullptr, "no transposition kernel was compiled for the split %d", code);
+      hipLaunchKernelGGL(e->kernel, grid_for(1), dim3((e->dw + e->cw) * 64), 0, s, d_in, d_out, n, tiles, band);
+      break;
+    }
     default: hipLaunchKernelGGL(transpose_not_specialized, grid_for(1), block, 0, s, d_in, d_out, n, tiles, band); break;
   }
   CUDADMA_HIP_CHECK(hipGetLastError());

@@ -3,7 +3,7 @@ compute unit, timed with HIP events.  The counterpart of the reference's
 src/perf/sequential/param_sweep.py:27-58, which rewrites params_directed.h and recompiles per
 point; here the variants are compiled in and the occupancy is a run-time knob.
 
-    python -m cudadma_amd.sweep [sequential] [strided] [strided_shape] [gather] [scatter] [halo] [gemm] [memory] [--wg 0,2,4,8] [--steps 20]
+    python -m cudadma_amd.sweep [sequential] [strided] [gather] [scatter] [halo] [gemm] [yardsticks] [--wg 0,2,4,8] [--steps 20]
     python -m cudadma_amd.sweep saxpy sgemv stencil2d        # the reference's example programs, every variant
     python -m cudadma_amd.sweep perf_sequential --wg 2,8     # read-bandwidth probe: element size x DMA wavefronts x buffering
 """
@@ -73,27 +73,6 @@ def main(argv=None):
                 for wg in wgs:
                     wl.set_workgroups_per_cu(wg)
                     _row(name, v, wg, _time(lambda: wl.strided_transpose(src, dst, v), args.steps), 2 * n * n * 4)
-        elif name == "strided_shape":
-            # the operating point of the transposition: workgroups launched x tile order, for the kernel with one LDS
-            # tile (variant 1), the one that is not warp-specialised (4) and the one with two LDS tiles (0)
-            n = 16384
-            src = wl.fill_uniform(torch.empty(n * n, device=dev), 1002).view(n, n)
-            dst = torch.empty_like(src)
-            cus = torch.cuda.get_device_properties(0).multi_processor_count
-            grids = [cus * 3 // 4, cus - 8, cus, cus + 32, 2 * cus, 3 * cus, 4 * cus, 8 * cus]
-            print("# transposition of 16384^2 floats, ms per launch; columns: workgroups launched = " + ", ".join(map(str, grids)))
-            try:
-                for v in (1, 4, 0):
-                    for band in (1, 4, 16, 64, 256):
-                        wl.set_tuning("transpose_band", band)
-                        cells = []
-                        for g in grids:
-                            wl.set_tuning("transpose_workgroups", g)
-                            cells.append(f"{_time(lambda: wl.strided_transpose(src, dst, v), args.steps, settle_ms=10.0):.4f}")
-                        print(f"variant {v}  band {band:3d}  " + "  ".join(cells), flush=True)
-            finally:
-                wl.set_tuning("transpose_band", 0)
-                wl.set_tuning("transpose_workgroups", 0)
         elif name == "gather":
             recs, n_idx = 4 << 20, 32 << 20
             table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1003)
@@ -105,16 +84,17 @@ def main(argv=None):
                     wl.set_workgroups_per_cu(wg)
                     _row(name, v, wg, _time(lambda: wl.gather_rowsum(table, idx, out, v), args.steps),
                          n_idx * 132 + out.numel() * 4)
-        elif name == "memory":
-            # what copy-shaped kernels without LDS reach on 1 GiB + 1 GiB, per launch shape
+        elif name == "yardsticks":
+            # read-only, write-only and copy streams on 2 x 1 GiB per launch shape, and the vendor's copy
             n = 16384
             src = wl.fill_uniform(torch.empty(n * n, device=dev), 1002)
             dst = torch.empty_like(src)
             cus = torch.cuda.get_device_properties(0).multi_processor_count
-            print("# memory probes on 2 x 1 GiB; GB/s of bytes read + written; columns: workgroups per CU 0.5 / 1 / 1.5 / 2 / 3 / 4 / 8 / 16")
+            shapes = (0.5, 1, 1.5, 2, 3, 4, 8, 16)
+            print("# streaming yardsticks on 2 x 1 GiB; ms and GB/s of bytes read + written; columns: workgroups per CU " + " / ".join(map(str, shapes)))
             for mode, label in enumerate(wl.PROBE_MODES):
                 cells = []
-                for wg in (0.5, 1, 1.5, 2, 3, 4, 8, 16):
+                for wg in (shapes if label != "vendor_copy" else (1,)):
                     s_, d_ = (None if label.startswith("write") else src), (None if label == "read" else dst)
                     nbytes = wl.probe_memory(mode, s_, d_, int(cus * wg))
                     ms = _time(lambda: wl.probe_memory(mode, s_, d_, int(cus * wg)), args.steps, settle_ms=10.0)

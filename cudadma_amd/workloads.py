@@ -13,6 +13,7 @@ REC_FLOATS = 32          # 128-byte records
 RECS_PER_TILE = 32
 SEQ_TILE_BYTES = 16 * 1024
 STENCIL_RADIUS = 4
+GEMM_WARP_SPECIALISED_VARIANT = 7      # the cudadma_gemm_bf16 variant in which DMA wavefronts feed compute wavefronts
 
 
 def _stream():
@@ -164,13 +165,13 @@ def perf_sequential(src, elmt_bytes, dma_wavefronts, buffering, loop_iters, work
     return int(n)
 
 
-PROBE_MODES = ("read", "write", "write_nontemporal", "copy", "copy_nontemporal", "blocks_in_place", "blocks_swapped",
-               "blocks_permuted", "write_blocks_swapped", "transpose_private")
+PROBE_MODES = ("read", "write", "write_nontemporal", "copy", "copy_nontemporal", "vendor_copy")
 
 
 def probe_memory(mode, src, dst, workgroups):
-    """One launch of a memory-system probe (mode: index into PROBE_MODES or its name).  src / dst are CUDA tensors
-    of the same size in bytes (None where the mode does not use one).  Returns bytes read + bytes written."""
+    """One launch of a streaming yardstick (mode: index into PROBE_MODES or its name; "vendor_copy" is
+    hipMemcpyDtoDAsync and ignores `workgroups`).  src / dst are CUDA tensors of the same size in bytes (None
+    where the mode does not use one).  Returns bytes read + bytes written."""
     if isinstance(mode, str):
         mode = PROBE_MODES.index(mode)
     t = src if src is not None else dst

@@ -228,6 +228,7 @@ int cudadma_set_workgroups_per_cu(int value);
  * value or CUDADMA_EINVAL for an unknown name:
  *   "transpose_band"  tile rows per band of the config 2 tile order
  *   "transpose_workgroups"  workgroups to launch for config 2, whatever the per-CU knob says
+ *   "transpose_split"  config 2, variant 10: 100 x DMA wavefronts + 10 x compute wavefronts + tiles requested ahead
  *   "stencil_zchunk"     output planes one workgroup marches through in config 4
  *   "stencil_xcd_remap"  config 4 numbers its workgroups so that each XCD gets a contiguous part of the grid; 2 turns that off */
 int cudadma_set_tuning(const char* name, int value);
@@ -322,26 +323,20 @@ enum {
 long long cudadma_perf_sequential(const void* d_src, size_t src_bytes, unsigned* d_sums, int elmt_bytes,
                                   int dma_wavefronts, int buffering, int loop_iters, int workgroups, void* stream);
 
-/* ---- memory-system probes --------------------------------------------------------------
- * Kernels without LDS and without a DMA object that show what a copy-shaped kernel reaches on the
- * device and what the placement of the blocks costs: the yardsticks for config 2.  No counterpart
- * in the reference.  `bytes` is the size of each buffer (a multiple of 16); the block modes view
- * the buffers as n x n float matrices (bytes = 4 n^2, n a power of two >= 64) cut into blocks of
- * 64 rows x 256 B, one block per wavefront and step.  Write-only modes store the float 1.0.
+/* ---- streaming yardsticks ------------------------------------------------------------------
+ * Kernels without LDS and without a DMA object (grid-stride dwordx4 accesses) that show what read-only,
+ * write-only and copy-shaped streams reach on the device at a given launch shape, and the vendor's own
+ * device-to-device copy: what the patterns' figures are read against.  No counterpart in the reference.
+ * `bytes` is the size of each buffer (a multiple of 16).  Write-only modes store the float 1.0.
  * Returns the bytes read plus the bytes written, or a negative CUDADMA_E* code. */
 enum {
   CUDADMA_PROBE_READ                 = 0,  /* d_dst may be NULL                                    */
   CUDADMA_PROBE_WRITE                = 1,  /* d_src may be NULL                                    */
   CUDADMA_PROBE_WRITE_NONTEMPORAL    = 2,
-  CUDADMA_PROBE_COPY                 = 3,  /* grid-stride dwordx4                                  */
-  CUDADMA_PROBE_COPY_NONTEMPORAL     = 4,
-  CUDADMA_PROBE_BLOCKS_IN_PLACE      = 5,  /* block (r, c) -> block (r, c)                         */
-  CUDADMA_PROBE_BLOCKS_SWAPPED       = 6,  /* block (r, c) -> block (c, r), contents not transposed */
-  CUDADMA_PROBE_BLOCKS_PERMUTED      = 7,  /* in place, blocks visited in a scattered order        */
-  CUDADMA_PROBE_WRITE_BLOCKS_SWAPPED = 8,  /* mode 6 without its loads                             */
-  CUDADMA_PROBE_TRANSPOSE_PRIVATE    = 9,  /* d_dst = transpose(d_src): every wavefront transposes its blocks
-                                              through an LDS tile of its own, no DMA object, no handshake    */
-  CUDADMA_PROBE_MODES                = 10
+  CUDADMA_PROBE_COPY                 = 3,
+  CUDADMA_PROBE_COPY_NONTEMPORAL     = 4,  /* non-temporal loads and stores                        */
+  CUDADMA_PROBE_VENDOR_COPY          = 5,  /* hipMemcpyDtoDAsync; `workgroups` is ignored          */
+  CUDADMA_PROBE_MODES                = 6
 };
 long long cudadma_probe_memory(int mode, const void* d_src, void* d_dst, size_t bytes, int workgroups, void* stream);
 

@@ -79,7 +79,6 @@ def test_run_case_validates_before_launching():
     assert L.cudadma_scatter_copy(4096, 4096, 8192, 16, 33, 0, None) == -1
     assert L.cudadma_probe_memory(3, 4096, 8192, 100, 8, None) == -1           # bytes not a multiple of 16
     assert L.cudadma_probe_memory(99, 4096, 8192, 1024, 8, None) == -3
-    assert L.cudadma_probe_memory(6, 4096, 8192, 3 * 16384, 8, None) == -1     # not 4 n^2
     assert L.cudadma_fill_permutation(4096, 0, 1, None) == -1
     # workloads: sizes and variants are checked first
     assert L.cudadma_sequential_copy(4096, 8192, 1000, 0, None) == -1

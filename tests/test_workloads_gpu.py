@@ -100,7 +100,7 @@ def test_strided_transpose_small(device, variant, n):
     assert np.array_equal(dst.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("variant", [1, 4, 0])
+@pytest.mark.parametrize("variant", [10, 1, 4, 0])
 @pytest.mark.parametrize("band,workgroups", [(0, 0), (1, 0), (3, 7), (5, 300), (256, 255), (1000, 100000)])
 def test_strided_transpose_under_every_tuning(device, variant, band, workgroups):
     """The tile order and the number of workgroups are tuning knobs: the result does not depend on them."""
@@ -119,7 +119,36 @@ def test_strided_transpose_under_every_tuning(device, variant, band, workgroups)
     assert np.array_equal(dst.cpu().numpy().view(np.uint32), np.ascontiguousarray(host.T).view(np.uint32))
 
 
-@pytest.mark.parametrize("variant", [1, 0])                       # the reported kernel and the one with two LDS tiles
+_SPLITS = [221, 222, 111, 112, 121, 122, 211, 212, 311, 312, 411, 412, 321, 322, 421, 422, 141, 142, 241, 242, 441, 442]
+
+
+@pytest.mark.parametrize("split", _SPLITS)
+@pytest.mark.parametrize("n,workgroups", [(64, 0), (1344, 0), (1344, 5), (2112, 700)])
+def test_strided_transpose_under_every_split(device, split, n, workgroups):
+    """Variant 10 with every compiled split of the workgroup (DMA wavefronts, compute wavefronts, tiles requested ahead):
+    the result does not depend on it, whether a workgroup gets one tile, several, or an odd number of them."""
+    host = ol.uniform(n * n, 78).reshape(n, n)
+    src = torch.from_numpy(host).to(device)
+    dst = torch.full_like(src, float("nan"))
+    try:
+        wl.set_tuning("transpose_split", split)
+        wl.set_tuning("transpose_workgroups", workgroups)
+        print(f"transpose split {split} n {n} workgroups {workgroups}", flush=True)
+        wl.strided_transpose(src, dst, 10)
+        torch.cuda.synchronize()
+    finally:
+        wl.set_tuning("transpose_split", 0)
+        wl.set_tuning("transpose_workgroups", 0)
+    assert np.array_equal(dst.cpu().numpy().view(np.uint32), np.ascontiguousarray(host.T).view(np.uint32))
+    with pytest.raises(cd.CudaDMAError, match="split"):
+        try:
+            wl.set_tuning("transpose_split", 999)
+            wl.strided_transpose(src, dst, 10)
+        finally:
+            wl.set_tuning("transpose_split", 0)
+
+
+@pytest.mark.parametrize("variant", [10, 1, 0])                   # the reported kernel, its even split and the one with two LDS tiles
 def test_strided_transpose_full_size(device, variant):
     n = 16384
     src = wl.fill_uniform(torch.empty(n * n, dtype=torch.float32, device=device), 1002).view(n, n)
@@ -379,16 +408,14 @@ def test_gemm_rejects_ragged_shapes(device):
         wl.gemm_bf16(a, b, c)
 
 
-# ------------------------------------------------------------------ memory-system probes
+# ------------------------------------------------------------------ streaming yardsticks
 @pytest.mark.parametrize("workgroups", [1, 7, 512])
-def test_memory_probes_move_what_they_say(device, workgroups):
-    n = 256                                                     # 256 x 256 floats: 4 x 4 blocks of 64 rows x 256 B
-    src = wl.fill_uniform(torch.empty(n * n, dtype=torch.float32, device=device), 77)
+def test_yardsticks_move_what_they_say(device, workgroups):
+    src = wl.fill_uniform(torch.empty(256 * 256, dtype=torch.float32, device=device), 77)
     nbytes = src.numel() * 4
-    want_blocks = src.view(n // 64, 64, n // 64, 64)            # [block row][row][block column][column]
     for mode, label in enumerate(wl.PROBE_MODES):
         dst = torch.full_like(src, -3.0)
-        print(f"probe {label} workgroups {workgroups}", flush=True)
+        print(f"yardstick {label} workgroups {workgroups}", flush=True)
         moved = wl.probe_memory(mode, None if label.startswith("write") else src, None if label == "read" else dst, workgroups)
         torch.cuda.synchronize()
         assert moved == nbytes * ((0 if label.startswith("write") else 1) + (0 if label == "read" else 1))
@@ -396,23 +423,16 @@ def test_memory_probes_move_what_they_say(device, workgroups):
             continue
         if label.startswith("write"):
             assert bool((dst == 1.0).all())
-        elif label == "transpose_private":
-            assert torch.equal(dst.view(n, n).view(torch.int32), src.view(n, n).t().contiguous().view(torch.int32))
-        elif label == "blocks_swapped":
-            got = dst.view(n // 64, 64, n // 64, 64)
-            assert torch.equal(got.view(torch.int32), want_blocks.permute(2, 1, 0, 3).contiguous().view(torch.int32))
         else:
             assert torch.equal(dst.view(torch.int32), src.view(torch.int32))
 
 
-def test_memory_probe_argument_checks(device):
+def test_yardstick_argument_checks(device):
     t = torch.zeros(64 * 64, dtype=torch.float32, device=device)
     with pytest.raises(cd.CudaDMAError):
         wl.probe_memory(len(wl.PROBE_MODES), t, t.clone(), 4)
     with pytest.raises(cd.CudaDMAError):
         wl.probe_memory("copy", t, t.clone(), 0)
-    with pytest.raises(cd.CudaDMAError, match="power of two"):
-        wl.probe_memory("blocks_swapped", t[:3 * 64 * 64 // 4], t.clone()[:3 * 64 * 64 // 4], 4)
     with pytest.raises(cd.CudaDMAError, match="NULL"):
         wl.probe_memory("copy", t, None, 4)
 
