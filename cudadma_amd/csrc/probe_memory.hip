@@ -9,18 +9,23 @@ using workloads::vec4_t;
 
 constexpr int kThreads = 256;
 
+template<bool NONTEMPORAL>
 __global__ void __launch_bounds__(kThreads)
 probe_read(const vec4_t* __restrict__ in, vec4_t* __restrict__ sink, const size_t n_vec)
 {
+  auto ld = [](const vec4_t* p) __attribute__((always_inline)) {
+    if constexpr (NONTEMPORAL) return __builtin_nontemporal_load(p);
+    else return *p;
+  };
   vec4_t acc = {0u, 0u, 0u, 0u};
   const size_t stride = (size_t)gridDim.x * kThreads;
   size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x;
   // four loads in flight per lane
   for (; i + 3 * stride < n_vec; i += 4 * stride) {
-    const vec4_t a = in[i], b = in[i + stride], c = in[i + 2 * stride], d = in[i + 3 * stride];
+    const vec4_t a = ld(in + i), b = ld(in + i + stride), c = ld(in + i + 2 * stride), d = ld(in + i + 3 * stride);
     acc ^= a ^ b ^ c ^ d;
   }
-  for (; i < n_vec; i += stride) acc ^= in[i];
+  for (; i < n_vec; i += stride) acc ^= ld(in + i);
   // never true for the benchmark data (finite floats); keeps the loads alive
   if ((acc.x & acc.y & acc.z & acc.w) == 0xffffffffu && sink != nullptr) sink[threadIdx.x] = acc;
 }
@@ -59,7 +64,7 @@ extern "C" long long cudadma_probe_memory(int mode, const void* d_src, void* d_d
   }
   CUDADMA_REQUIRE(bytes > 0 && (bytes % 16) == 0, "bytes must be a positive multiple of 16");
   const bool reads = mode != CUDADMA_PROBE_WRITE && mode != CUDADMA_PROBE_WRITE_NONTEMPORAL;
-  const bool writes = mode != CUDADMA_PROBE_READ;
+  const bool writes = mode != CUDADMA_PROBE_READ && mode != CUDADMA_PROBE_READ_NONTEMPORAL;
   CUDADMA_REQUIRE((!reads || d_src != nullptr) && (!writes || d_dst != nullptr), "NULL pointer");
   CUDADMA_REQUIRE((!reads || cudadma_host::aligned_to(d_src, 16)) && (!writes || cudadma_host::aligned_to(d_dst, 16)),
                   "pointers must be 16-byte aligned");
@@ -73,7 +78,8 @@ extern "C" long long cudadma_probe_memory(int mode, const void* d_src, void* d_d
   const dim3 grid((unsigned)workgroups), block(kThreads);
   const size_t n_vec = bytes / 16;
   switch (mode) {
-    case CUDADMA_PROBE_READ: hipLaunchKernelGGL(probe_read, grid, block, 0, s, (const vec4_t*)d_src, (vec4_t*)d_dst, n_vec); break;
+    case CUDADMA_PROBE_READ: hipLaunchKernelGGL(probe_read<false>, grid, block, 0, s, (const vec4_t*)d_src, (vec4_t*)d_dst, n_vec); break;
+    case CUDADMA_PROBE_READ_NONTEMPORAL: hipLaunchKernelGGL(probe_read<true>, grid, block, 0, s, (const vec4_t*)d_src, (vec4_t*)d_dst, n_vec); break;
     case CUDADMA_PROBE_WRITE: hipLaunchKernelGGL(probe_write<false>, grid, block, 0, s, (vec4_t*)d_dst, n_vec); break;
     case CUDADMA_PROBE_WRITE_NONTEMPORAL: hipLaunchKernelGGL(probe_write<true>, grid, block, 0, s, (vec4_t*)d_dst, n_vec); break;
     case CUDADMA_PROBE_COPY: hipLaunchKernelGGL(probe_copy<false>, grid, block, 0, s, (const vec4_t*)d_src, (vec4_t*)d_dst, n_vec); break;

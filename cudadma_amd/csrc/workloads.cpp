@@ -53,6 +53,7 @@ static const VariantInfo kSequential[] = {
   {"no DMA object: every wavefront copies global -> LDS -> global between workgroup barriers"},
   {"single buffer (the next tile waits in the DMA wavefronts' registers), two workgroups per compute unit, streaming "
    "loads and non-temporal stores: the shape for buffers beyond the Infinity Cache"},
+  {"variant 5 with a contiguous run of tiles per workgroup instead of every n-th tile"},
 };
 static const VariantInfo kStrided[] = {
   {"manual double buffer: one DMA group of 2 wavefronts, two CudaDMAStrided objects, padded LDS rows (272 B)"},

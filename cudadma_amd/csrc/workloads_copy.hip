@@ -88,19 +88,28 @@ copy_manual_double(const char* __restrict__ in, char* __restrict__ out, const in
 // variant 1: one object, one buffer.  execute_dma requests a tile into the DMA wavefronts' registers before it
 // waits for the buffer, so the double buffer is the LDS tile plus those registers.  STREAM (used for working sets
 // beyond the Infinity Cache): streaming loads and non-temporal stores, neither side is read again.
-template<bool STREAM>
+// CHUNKED: a workgroup takes a contiguous run of tiles instead of every gridDim.x-th one.  The tiles in flight at one
+// time are then spread over the whole buffer instead of forming one window that moves through it, and the speed
+// no longer depends on how source and destination lie relative to each other (with the moving window, a 1 GiB
+// copy ran between 0.350 and 0.440 ms depending on the distance between the two buffers modulo 64 MiB: reads and
+// writes of the same window meet in the same memory channels and banks).
+template<bool STREAM, bool CHUNKED = false>
 __global__ void __launch_bounds__(kDmaThreads + kComputeThreads)
 copy_single(const char* __restrict__ in, char* __restrict__ out, const int num_tiles)
 {
   __shared__ __attribute__((aligned(16))) vec4_t buf[kTileVecs];
   CudaDMASequential<true, 16, kTileBytes / kDmaThreads, kTileBytes, kDmaThreads> dma(0, kComputeThreads, kComputeThreads);
   constexpr int kLoad = STREAM ? LOAD_CACHE_STREAMING : LOAD_CACHE_ALL;
+  const int per = (num_tiles + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int first = CHUNKED ? (int)blockIdx.x * per : (int)blockIdx.x;
+  const int step = CHUNKED ? 1 : (int)gridDim.x;
+  const int end = CHUNKED ? ((first + per < num_tiles) ? first + per : num_tiles) : num_tiles;
   if (dma.owns_this_thread()) {
-    for (int t = blockIdx.x; t < num_tiles; t += gridDim.x)
+    for (int t = first; t < end; t += step)
       dma.template execute_dma<true, kLoad, STORE_LDS>(in + (size_t)t * kTileBytes, buf);
   } else {
     dma.start_async_dma();
-    for (int t = blockIdx.x; t < num_tiles; t += gridDim.x) {
+    for (int t = first; t < end; t += step) {
       dma.wait_for_dma_finish();
       drain_tile<STREAM>(buf, (vec4_t*)(out + (size_t)t * kTileBytes), dma);
     }
@@ -318,6 +327,7 @@ extern "C" int cudadma_sequential_copy(const float* d_in, float* d_out, size_t b
       break;
     case 1: hipLaunchKernelGGL(copy_single<false>, dim3(workloads::persistent_grid(tiles, 8)), block, 0, s, in, out, tiles); break;
     case 5: hipLaunchKernelGGL(copy_single<true>, dim3(workloads::persistent_grid(tiles, 2)), block, 0, s, in, out, tiles); break;
+    case 6: hipLaunchKernelGGL((copy_single<true, true>), dim3(workloads::persistent_grid(tiles, 2)), block, 0, s, in, out, tiles); break;
     case 2: hipLaunchKernelGGL(copy_double, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, in, out, tiles); break;
     case 3: hipLaunchKernelGGL(copy_manual_double<STORE_LDS_DIRECT>, dim3(workloads::persistent_grid(tiles, 4)), block, 0, s, in, out, tiles); break;
     default: hipLaunchKernelGGL(copy_not_specialized, dim3(workloads::persistent_grid(tiles, 8)), block, 0, s, in, out, tiles); break;

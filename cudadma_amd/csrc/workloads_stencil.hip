@@ -351,6 +351,13 @@ template<int QUEUE> struct queue_ok { static_assert(QUEUE >= 2 * kR + 2 && QUEUE
 // carry no handshake; the four LDS planes are guarded by cudaDMACustom objects,
 // the sync-only class of include/cudaDMA.h:4184-4208.
 constexpr int kBufs = 4;
+#ifndef STENCIL_RING_LOAD
+#define STENCIL_RING_LOAD LOAD_CACHE_ALL
+#endif
+#ifndef STENCIL_INTERIOR_NT
+#define STENCIL_INTERIOR_NT 0
+#endif
+constexpr int kRingLoad = STENCIL_RING_LOAD;
 constexpr int kRingObjs = 8;
 #ifndef STENCIL_RING_AHEAD
 #define STENCIL_RING_AHEAD (kRingObjs - 1)
@@ -423,11 +430,11 @@ stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int
     // a request past the last plane re-reads the last one: the loads stay unconditional, nothing lands from them
     const int last = w.planes - 1;
 #define HIPDMA_ISSUE(I, ZP) \
-    ring.get<(I)>().template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(ring0 + (size_t)((ZP) < last ? (ZP) : last) * in_plane);
+    ring.get<(I)>().template start_xfer_async<true, kRingLoad, STORE_LDS>(ring0 + (size_t)((ZP) < last ? (ZP) : last) * in_plane);
 #define HIPDMA_LAND(I, ZP)                                                                                   \
     if ((ZP) < w.planes) {                                                                                   \
       if constexpr (SYNC != kBarrierOnly) guard.get<(I) % kBufs>().wait_for_dma_start();                     \
-      ring.get<(I)>().template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(&plane[(I) % kBufs][kOrigin]); \
+      ring.get<(I)>().template wait_xfer_finish<true, kRingLoad, STORE_LDS>(&plane[(I) % kBufs][kOrigin]); \
       if constexpr (SYNC != kBarrierOnly) guard.get<(I) % kBufs>().finish_async_dma();                       \
     }
     // With the handshake the ring lands two planes ahead of its use instead of one: the compute
@@ -479,7 +486,8 @@ stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int
       const cudaDMACustom& cur_halo = guard.get<B>();
       // past the end of the chunk the last plane is fetched again: unconditional loads keep the wait counts exact
       const int zf = (z + QUEUE - 1 < avail) ? (z + QUEUE - 1) : (avail - 1);
-      q[HIPDMA_QSLOT(ROT, QUEUE - 1)] = *(const f32x4_t*)(col + (size_t)zf * in_plane);
+      if constexpr (STENCIL_INTERIOR_NT) q[HIPDMA_QSLOT(ROT, QUEUE - 1)] = __builtin_nontemporal_load((const f32x4_t*)(col + (size_t)zf * in_plane));
+      else q[HIPDMA_QSLOT(ROT, QUEUE - 1)] = *(const f32x4_t*)(col + (size_t)zf * in_plane);
       if constexpr (SYNC != kBarrierOnly) cur_halo.wait_for_dma_finish(seen);
       if constexpr (SYNC == kHandshakeAndGroupBarrier) compute_barrier.sync();
       else __syncthreads();

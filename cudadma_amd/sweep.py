@@ -95,7 +95,7 @@ def main(argv=None):
             for mode, label in enumerate(wl.PROBE_MODES):
                 cells = []
                 for wg in (shapes if label != "vendor_copy" else (1,)):
-                    s_, d_ = (None if label.startswith("write") else src), (None if label == "read" else dst)
+                    s_, d_ = (None if label.startswith("write") else src), (None if label.startswith("read") else dst)
                     nbytes = wl.probe_memory(mode, s_, d_, int(cus * wg))
                     ms = _time(lambda: wl.probe_memory(mode, s_, d_, int(cus * wg)), args.steps, settle_ms=10.0)
                     cells.append(f"{ms:7.4f} ms {nbytes / ms / 1e6:6.0f}")

@@ -165,7 +165,7 @@ def perf_sequential(src, elmt_bytes, dma_wavefronts, buffering, loop_iters, work
     return int(n)
 
 
-PROBE_MODES = ("read", "write", "write_nontemporal", "copy", "copy_nontemporal", "vendor_copy")
+PROBE_MODES = ("read", "write", "write_nontemporal", "copy", "copy_nontemporal", "vendor_copy", "read_nontemporal")
 
 
 def probe_memory(mode, src, dst, workgroups):

@@ -336,7 +336,8 @@ enum {
   CUDADMA_PROBE_COPY                 = 3,
   CUDADMA_PROBE_COPY_NONTEMPORAL     = 4,  /* non-temporal loads and stores                        */
   CUDADMA_PROBE_VENDOR_COPY          = 5,  /* hipMemcpyDtoDAsync; `workgroups` is ignored          */
-  CUDADMA_PROBE_MODES                = 6
+  CUDADMA_PROBE_READ_NONTEMPORAL     = 6,  /* d_dst may be NULL                                    */
+  CUDADMA_PROBE_MODES                = 7
 };
 long long cudadma_probe_memory(int mode, const void* d_src, void* d_dst, size_t bytes, int workgroups, void* stream);
 

@@ -43,15 +43,27 @@ __host__ __device__ constexpr int load_policy_bits(const int q)
 
 // One aligned vector load of sizeof(T) bytes, P = pointer type in the address space of the source.
 // The compiler offers sc1 alone only through an agent-scope atomic load, which exists for 4 and 8
-// bytes; a 16-byte LOAD_CACHE_GLOBAL load is issued with sc0 sc1 instead (one dwordx4, the vector L1
-// bypassed all the same; for device memory the L2 treats both scopes alike).
+// bytes: a 16-byte LOAD_CACHE_GLOBAL load is issued as two dwordx2 loads with sc1.  (One dwordx4 with
+// sc0 sc1 would bypass the vector L1 as well, but system-scope loads have a much longer latency: a
+// read-only stream of 1 GiB ran at 2.4 TB/s with them at one workgroup per compute unit, at 6.0 TB/s
+// with the two sc1 halves, 6.3 TB/s plain and 6.4 TB/s non-temporal.)
 template<typename T, int LOAD_QUAL, typename P>
 __device__ __forceinline__ T load_vec_from(P p)
 {
   if constexpr (LOAD_QUAL == LOAD_CACHE_STREAMING || LOAD_QUAL == LOAD_CACHE_LAST_USE) {
     return __builtin_nontemporal_load(p);
-  } else if constexpr (LOAD_QUAL == LOAD_CACHE_VOLATILE || (LOAD_QUAL == LOAD_CACHE_GLOBAL && sizeof(T) == 16)) {
+  } else if constexpr (LOAD_QUAL == LOAD_CACHE_VOLATILE) {
     return *(volatile typename std::remove_pointer<P>::type*)p;     // volatile added, address space kept
+  } else if constexpr (LOAD_QUAL == LOAD_CACHE_GLOBAL && sizeof(T) == 16) {
+    const unsigned long long* q = (const unsigned long long*)p;
+    const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    T out;
+    out[0] = (unsigned)lo;
+    out[1] = (unsigned)(lo >> 32);
+    out[2] = (unsigned)hi;
+    out[3] = (unsigned)(hi >> 32);
+    return out;
   } else if constexpr (LOAD_QUAL == LOAD_CACHE_GLOBAL && sizeof(T) == 4) {
     return (T)__hip_atomic_load((const unsigned*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   } else if constexpr (LOAD_QUAL == LOAD_CACHE_GLOBAL && sizeof(T) == 8) {

@@ -416,10 +416,10 @@ def test_yardsticks_move_what_they_say(device, workgroups):
     for mode, label in enumerate(wl.PROBE_MODES):
         dst = torch.full_like(src, -3.0)
         print(f"yardstick {label} workgroups {workgroups}", flush=True)
-        moved = wl.probe_memory(mode, None if label.startswith("write") else src, None if label == "read" else dst, workgroups)
+        moved = wl.probe_memory(mode, None if label.startswith("write") else src, None if label.startswith("read") else dst, workgroups)
         torch.cuda.synchronize()
-        assert moved == nbytes * ((0 if label.startswith("write") else 1) + (0 if label == "read" else 1))
-        if label == "read":
+        assert moved == nbytes * ((0 if label.startswith("write") else 1) + (0 if label.startswith("read") else 1))
+        if label.startswith("read"):
             continue
         if label.startswith("write"):
             assert bool((dst == 1.0).all())
