@@ -28,7 +28,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0           # MI355X published HBM3E bandwidth
 MFMA_PEAK_TFLOPS = 2500.0       # MI355X published dense bf16 rate
 SETTLE_MS = 30.0                # wall time of untimed warm-up for the secondary patterns
-STRIDED_VARIANT = 10            # cudadma_strided_transpose variant timed as the headline (three DMA + one compute wavefront)
+STRIDED_VARIANT = 0             # cudadma_strided_transpose variant timed as the headline: the library's choice (three DMA + one compute wavefront)
 COUNTERS_JSON = os.path.join(ROOT, "profiles", "counters.json")
 
 # name -> (kernel the pattern launches, as rocprofv3 names it; used by cudadma_amd.profile_summary)
@@ -37,7 +37,7 @@ PATTERN_KERNELS = {
     "strided_even_split": "transpose_single<true, true>",
     "strided_two_lds_tiles": "transpose_manual_double<272, false>",
     "sequential": "copy_manual_double<4>",
-    "sequential_hbm": "copy_single<true>",
+    "sequential_hbm": "copy_single<true, false>",
     "gather": "gather_manual<(anonymous namespace)::RowsumConsumer, 4>",
     "gather_hbm": "gather_manual<(anonymous namespace)::RowsumConsumer, 4>",
     "scatter": "scatter_manual<4>",
@@ -221,7 +221,7 @@ def main():
         ms, _ = time_launches(lambda: wl.strided_transpose(src, dst, 1), steps, warmup, SETTLE_MS)
         report(patterns, "strided_even_split", ms, strided_bytes, "the same kernel shape with two DMA and two compute wavefronts (128 + 128 threads)")
     if want("strided_two_lds_tiles"):
-        ms, _ = time_launches(lambda: wl.strided_transpose(src, dst, 0), steps, warmup, SETTLE_MS)
+        ms, _ = time_launches(lambda: wl.strided_transpose(src, dst, wl.TRANSPOSE_TWO_LDS_TILES_VARIANT), steps, warmup, SETTLE_MS)
         report(patterns, "strided_two_lds_tiles", ms, strided_bytes,
                "the same transposition with two LDS tiles and two CudaDMAStrided objects (manual double buffering in LDS)")
     # ---- yardsticks on the same two 1 GiB buffers: the plain copy used to calibrate the counters, the vendor's

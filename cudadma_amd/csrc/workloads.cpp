@@ -56,7 +56,8 @@ static const VariantInfo kSequential[] = {
   {"variant 5 with a contiguous run of tiles per workgroup instead of every n-th tile"},
 };
 static const VariantInfo kStrided[] = {
-  {"manual double buffer: one DMA group of 2 wavefronts, two CudaDMAStrided objects, padded LDS rows (272 B)"},
+  {"the library's choice: variant 10 at its default split (three DMA wavefronts, one compute wavefront, one LDS tile, "
+   "the next tile in the DMA wavefronts' registers)"},
   {"single buffer: one object and one LDS tile, execute_dma (the next tile waits in the DMA wavefronts' registers); one "
    "workgroup per compute unit, tiles walked down the columns, streaming loads (LOAD_CACHE_STREAMING), the consumer "
    "transposes 4 x 4 words inside each quad and writes non-temporal dwordx4: the fastest shape"},
@@ -66,7 +67,7 @@ static const VariantInfo kStrided[] = {
   {"two DMA groups, unpadded 256 B LDS rows filled by global_load_lds_dwordx4 with XOR-swizzled chunks "
    "(STORE_LDS_DIRECT_SWIZZLE): no VGPR staging, no padding, no bank conflicts"},
   {"two DMA groups, unpadded 256 B LDS rows with XOR-swizzled chunks written from registers (STORE_LDS_SWIZZLE)"},
-  {"as variant 0, but the compute lanes transpose 4 x 4 words inside each quad (quad-permute moves) and write "
+  {"as variant 11, but the compute lanes transpose 4 x 4 words inside each quad (quad-permute moves) and write "
    "dwordx4: one store covers four output rows of 256 contiguous bytes instead of one"},
   {"one DMA wavefront and one compute wavefront per workgroup, two objects of a whole tile each on the DMA "
    "wavefront, two LDS tiles; dword stores"},
@@ -75,6 +76,8 @@ static const VariantInfo kStrided[] = {
    "wavefronts + tiles requested ahead; default 311: three DMA wavefronts, one compute wavefront, one tile ahead, "
    "the fastest of the 22 splits compiled): one LDS tile guarded by a sync-only object, one or two CudaDMAStrided "
    "objects without a handshake of their own on the DMA wavefronts; the kernel the benchmark reports"},
+  {"manual double buffer in LDS: one DMA group of 2 wavefronts, two CudaDMAStrided objects and two LDS tiles with padded "
+   "rows (272 B), four workgroups per compute unit"},
 };
 static const VariantInfo kGather[] = {
   {"manual 4-stage buffering: one DMA group of 2 wavefronts, four CudaDMAIndirect objects"},

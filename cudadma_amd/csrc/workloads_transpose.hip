@@ -447,7 +447,7 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
   // The kernels with one LDS tile (variants 1 and 4) run best with exactly one workgroup per compute unit, i.e. one
   // 16 KB tile of loads in flight per compute unit, and with the tiles walked down the columns (the workgroups that
   // run together then write whole output rows); the others with four workgroups and bands of 16 tile rows.
-  const bool one_tile = variant == 1 || variant == 4 || variant == 10;
+  const bool one_tile = variant == 0 || variant == 1 || variant == 4 || variant == 10;
   int band = workloads::tuning("transpose_band", one_tile ? tiles_per_side : kDefaultBand);
   if (band > tiles_per_side) band = tiles_per_side;
   while (band > 1 && tiles_per_side % band != 0) band /= 2;      // bands must tile the matrix
@@ -458,7 +458,7 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
   hipStream_t s = (hipStream_t)stream;
   const dim3 block(kDmaThreads + kComputeThreads);
   switch (variant) {
-    case 0: hipLaunchKernelGGL(transpose_manual_double<272>, grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
+    case 11: hipLaunchKernelGGL(transpose_manual_double<272>, grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 1: hipLaunchKernelGGL((transpose_single<true, true>), grid_for(1), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 2: hipLaunchKernelGGL(transpose_manual_double<256>, grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 3: hipLaunchKernelGGL(transpose_double_groups<272>, grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
@@ -467,9 +467,12 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
     case 7: hipLaunchKernelGGL((transpose_manual_double<272, true>), grid_for(4), block, 0, s, d_in, d_out, n, tiles, band); break;
     case 8: hipLaunchKernelGGL(transpose_pairs<false>, grid_for(4), dim3(128), 0, s, d_in, d_out, n, tiles, band); break;
     case 9: hipLaunchKernelGGL(transpose_pairs<true>, grid_for(4), dim3(128), 0, s, d_in, d_out, n, tiles, band); break;
+    case 0:
     case 10: {
-      // knob "transpose_split" = 100 * DMA wavefronts + 10 * compute wavefronts + tiles ahead (default 311, the fastest)
-      const int code = workloads::tuning("transpose_split", 311);
+      // variant 0 is the library's choice: the fastest split (three DMA wavefronts, one compute wavefront, one tile
+      // ahead).  Variant 10 takes the split from the knob "transpose_split" = 100 * DMA wavefronts + 10 * compute
+      // wavefronts + tiles ahead (the same default).
+      const int code = variant == 0 ? 311 : workloads::tuning("transpose_split", 311);
       const SplitEntry* e = nullptr;
       for (const SplitEntry& c : kSplits)
         if (100 * c.dw + 10 * c.cw + c.ahead == code) e = &c;

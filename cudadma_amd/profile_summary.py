@@ -3,7 +3,7 @@ fields from) and a table for the text summaries under profiles/.
 
 Expected layout, one directory per pattern of bench.py (`--only <pattern>`), one sub-directory per collection:
 
-    <root>/<pattern>/trace/   rocprofv3 --kernel-trace --output-format csv -d <root>/<pattern>/trace -o b -- python3 bench.py --only <pattern> --steps 20 --no-cpu-baseline > <root>/<pattern>/trace.json
+    <root>/<pattern>/trace/   rocprofv3 --kernel-trace --stats --output-format csv -d <root>/<pattern>/trace -o b -- python3 bench.py --only <pattern> --steps 20 --no-cpu-baseline > <root>/<pattern>/trace.json
     <root>/<pattern>/fetch/   rocprofv3 --pmc FETCH_SIZE --output-format csv -d ... -o b -- python3 bench.py --only <pattern>,plain_copy --steps 3 --warmup 1 --no-cpu-baseline
     <root>/<pattern>/write/   rocprofv3 --pmc WRITE_SIZE ...                                   (same command)
     <root>/<pattern>/lds/     rocprofv3 --pmc SQ_LDS_BANK_CONFLICT SQ_LDS_IDX_ACTIVE ...       (optional)
@@ -51,6 +51,14 @@ def durations_us(directory, kernel, last=20):
     return {"dispatches": len(d), "avg_us": sum(tail) / len(tail), "min_us": min(tail), "max_us": max(tail)}
 
 
+def stats_row(directory, kernel):
+    """rocprofv3's own --stats line for `kernel`: calls and average duration over every dispatch of the run."""
+    for r in _rows(directory, "_kernel_stats.csv"):
+        if _matches(r["Name"], kernel):
+            return {"stats_calls": int(r["Calls"]), "stats_avg_us": round(float(r["AverageNs"]) / 1e3, 2)}
+    return {}
+
+
 def counter_means(directory, kernel):
     """Mean value per dispatch of every counter collected for `kernel`."""
     acc = {}
@@ -94,6 +102,7 @@ def summarise(root):
         t = durations_us(os.path.join(pdir, "trace"), kernel) if os.path.isdir(os.path.join(pdir, "trace")) else None
         if t:
             row.update({k: round(v, 2) if isinstance(v, float) else v for k, v in t.items()})
+            row.update(stats_row(os.path.join(pdir, "trace"), kernel))
             if algorithmic:
                 row["GB/s_at_avg"] = round(algorithmic / t["avg_us"] / 1e3, 1)
             if row.get("flop"):
@@ -141,7 +150,7 @@ def summarise(root):
 
 
 def markdown(summary):
-    cols = ["kernel", "dispatches", "avg_us", "min_us", "max_us", "GB/s_at_avg", "TFLOP/s_at_avg", "FETCH_SIZE_KiB", "WRITE_SIZE_KiB",
+    cols = ["kernel", "dispatches", "avg_us", "min_us", "max_us", "stats_avg_us", "hip_event_ms", "GB/s_at_avg", "TFLOP/s_at_avg", "FETCH_SIZE_KiB", "WRITE_SIZE_KiB",
             "traffic_bytes", "traffic_over_algorithmic", "lds_bank_conflict_ratio", "mfma_busy"]
     lines = ["| pattern | " + " | ".join(cols) + " |", "|---|" + "---|" * len(cols)]
     for name, row in summary["patterns"].items():

@@ -6,6 +6,8 @@ point; here the variants are compiled in and the occupancy is a run-time knob.
     python -m cudadma_amd.sweep [sequential] [strided] [gather] [scatter] [halo] [gemm] [yardsticks] [--wg 0,2,4,8] [--steps 20]
     python -m cudadma_amd.sweep saxpy sgemv stencil2d        # the reference's example programs, every variant
     python -m cudadma_amd.sweep perf_sequential --wg 2,8     # read-bandwidth probe: element size x DMA wavefronts x buffering
+    python -m cudadma_amd.sweep transpose_split              # DMA : compute wavefronts x tiles ahead x workgroups per CU
+    python -m cudadma_amd.sweep placement                    # 1 GiB copies against the distance between source and destination
 """
 import argparse
 import sys
@@ -100,6 +102,50 @@ def main(argv=None):
                     ms = _time(lambda: wl.probe_memory(mode, s_, d_, int(cus * wg)), args.steps, settle_ms=10.0)
                     cells.append(f"{ms:7.4f} ms {nbytes / ms / 1e6:6.0f}")
                 print(f"{label:22s} " + "   ".join(cells), flush=True)
+        elif name == "transpose_split":
+            # the transposition of config 2 with every compiled (DMA wavefronts, compute wavefronts, tiles ahead)
+            # split, at one, two and three workgroups per compute unit; each split is checked against torch first
+            n = 16384
+            src = wl.fill_uniform(torch.empty(n * n, device=dev), 1002).view(n, n)
+            dst = torch.empty_like(src)
+            ref = src.t().contiguous()
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            print("# DMA + compute wavefronts, tiles ahead: ms (% of 8 TB/s) at 1 / 2 / 3 workgroups per compute unit")
+            for code in wl.TRANSPOSE_SPLITS:
+                wl.set_tuning("transpose_split", code)
+                dst.zero_()
+                wl.strided_transpose(src, dst, wl.TRANSPOSE_SPLIT_VARIANT)
+                exact = torch.equal(dst, ref)
+                cells = []
+                for wg in (1, 2, 3):
+                    wl.set_tuning("transpose_workgroups", cus * wg)
+                    ms = _time(lambda: wl.strided_transpose(src, dst, wl.TRANSPOSE_SPLIT_VARIANT), args.steps, settle_ms=15.0)
+                    cells.append(f"{ms:.4f} ({2 * n * n * 4 / ms / 1e6 / PEAK_GBS * 100:4.1f}%)")
+                wl.set_tuning("transpose_workgroups", 0)
+                print(f"{code // 100} + {code // 10 % 10}, {code % 10} ahead:  " + "   ".join(cells) + ("" if exact else "   WRONG RESULT"),
+                      flush=True)
+            wl.set_tuning("transpose_split", 0)
+            del ref
+        elif name == "placement":
+            # linear copies of 1 GiB inside one allocation, against the distance from source to destination;
+            # the transposition of the same bytes beside them
+            m = (1 << 30) // 4
+            pool = torch.empty(2 * m + (64 << 20) // 4, device=dev)
+            src = wl.fill_uniform(pool[:m], 1001)
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            print("# destination - source = 1 GiB + offset: ms (% of 8 TB/s) of sequential variant 5 (tile-interleaved) / variant 6 "
+                  "(contiguous runs) / copy_nontemporal yardstick at 4 workgroups per CU / transposition (headline variant)")
+            for off in (0, 4096, 16384, 65536, 1 << 20, 2 << 20, 4 << 20, 8 << 20, 16 << 20, (16 << 20) + 4096, 24 << 20,
+                        32 << 20, 48 << 20, 64 << 20):
+                dst = pool[m + off // 4: 2 * m + off // 4]
+                cells = []
+                for fn in (lambda: wl.sequential_copy(src, dst, 5), lambda: wl.sequential_copy(src, dst, 6),
+                           lambda: wl.probe_memory("copy_nontemporal", src, dst, cus * 4),
+                           lambda: wl.strided_transpose(src.view(16384, 16384), dst.view(16384, 16384), 0)):
+                    ms = _time(fn, args.steps, settle_ms=15.0)
+                    cells.append(f"{ms:.4f} ({2 * m * 4 / ms / 1e6 / PEAK_GBS * 100:4.1f}%)")
+                print(f"+{off:>9d} B:  " + "   ".join(cells), flush=True)
+            del pool
         elif name == "scatter":
             recs = 4 << 20
             records = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1006)

@@ -13,6 +13,10 @@ REC_FLOATS = 32          # 128-byte records
 RECS_PER_TILE = 32
 SEQ_TILE_BYTES = 16 * 1024
 STENCIL_RADIUS = 4
+TRANSPOSE_SPLIT_VARIANT = 10           # cudadma_strided_transpose variant whose wavefront split follows the knob "transpose_split"
+# knob values = 100 x DMA wavefronts + 10 x compute wavefronts + tiles ahead, every compiled combination
+TRANSPOSE_SPLITS = (111, 112, 121, 122, 141, 142, 211, 212, 221, 222, 241, 242, 311, 312, 321, 322, 411, 412, 421, 422, 441, 442)
+TRANSPOSE_TWO_LDS_TILES_VARIANT = 11    # two LDS tiles and two CudaDMAStrided objects (manual double buffering in LDS)
 GEMM_WARP_SPECIALISED_VARIANT = 7      # the cudadma_gemm_bf16 variant in which DMA wavefronts feed compute wavefronts
 
 

@@ -100,7 +100,7 @@ def test_strided_transpose_small(device, variant, n):
     assert np.array_equal(dst.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("variant", [10, 1, 4, 0])
+@pytest.mark.parametrize("variant", [0, 10, 1, 4, 11])
 @pytest.mark.parametrize("band,workgroups", [(0, 0), (1, 0), (3, 7), (5, 300), (256, 255), (1000, 100000)])
 def test_strided_transpose_under_every_tuning(device, variant, band, workgroups):
     """The tile order and the number of workgroups are tuning knobs: the result does not depend on them."""
@@ -119,7 +119,7 @@ def test_strided_transpose_under_every_tuning(device, variant, band, workgroups)
     assert np.array_equal(dst.cpu().numpy().view(np.uint32), np.ascontiguousarray(host.T).view(np.uint32))
 
 
-_SPLITS = [221, 222, 111, 112, 121, 122, 211, 212, 311, 312, 411, 412, 321, 322, 421, 422, 141, 142, 241, 242, 441, 442]
+_SPLITS = list(wl.TRANSPOSE_SPLITS)
 
 
 @pytest.mark.parametrize("split", _SPLITS)
@@ -148,7 +148,7 @@ def test_strided_transpose_under_every_split(device, split, n, workgroups):
             wl.set_tuning("transpose_split", 0)
 
 
-@pytest.mark.parametrize("variant", [10, 1, 0])                   # the reported kernel, its even split and the one with two LDS tiles
+@pytest.mark.parametrize("variant", [0, 1, 11])                   # the reported kernel, its even split and the one with two LDS tiles
 def test_strided_transpose_full_size(device, variant):
     n = 16384
     src = wl.fill_uniform(torch.empty(n * n, dtype=torch.float32, device=device), 1002).view(n, n)
