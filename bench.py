@@ -38,8 +38,8 @@ PATTERN_KERNELS = {
     "strided_two_lds_tiles": "transpose_manual_double<272, false>",
     "sequential": "copy_manual_double<4>",
     "sequential_hbm": "copy_single<true, false>",
-    "gather": "gather_manual<(anonymous namespace)::RowsumConsumer, 4>",
-    "gather_hbm": "gather_manual<(anonymous namespace)::RowsumConsumer, 4>",
+    "gather": "gather_manual<(anonymous namespace)::RowsumConsumer, 2, true>",
+    "gather_hbm": "gather_manual<(anonymous namespace)::RowsumConsumer, 2, true>",
     "scatter": "scatter_manual<4>",
     "halo": "stencil_ws_vec4<2, 12>",
     "halo_handshake": "stencil_ws_vec4<0, 12>",
@@ -340,6 +340,12 @@ def main():
                         "this level are the form of the same objects that is not warp-specialised")
         gemm["warp_specialised"] = gemm_row(wl.GEMM_WARP_SPECIALISED_VARIANT, "gemm_warp_specialised",
                                             "the same problem with DMA wavefronts feeding compute wavefronts through the handshake")
+        if want("yardsticks") or want("vendor_gemm"):
+            # the vendor library's GEMM (torch.matmul = hipBLASLt) on the same operands: the practical yardstick beside the peak
+            ms, _ = time_launches(lambda: torch.matmul(ga, gb), max(steps, 50), warmup, SETTLE_MS)
+            log(f"{'vendor_gemm':24s} {ms:9.4f} ms  {flops / ms / 1e9:8.1f} TFLOP/s  (torch.matmul, bf16 result)")
+            gemm["vendor_library"] = {"TFLOP/s": round(flops / ms / 1e9, 1), "ms": round(ms, 4),
+                                      "what": "torch.matmul (hipBLASLt) on the same bf16 operands, bf16 result"}
         del ga, gb, gc
 
     value = patterns["strided"]["GB/s"]

@@ -8,6 +8,7 @@ not been built: there is no CPU fallback.
 """
 from ._lib import (  # noqa: F401
     CALL_GLOBAL,
+    CALL_INDEX_AHEAD,
     CALL_LDS_DIRECT_NT,
     CALL_LDS_DIRECT_SC1,
     CALL_MATRIX_GENERIC,

@@ -8,7 +8,7 @@ PATTERN_SEQUENTIAL, PATTERN_STRIDED, PATTERN_GATHER, PATTERN_SCATTER, PATTERN_HA
 (CALL_UNQUALIFIED, CALL_GLOBAL, CALL_QUALIFIED, CALL_LDS_DIRECT, CALL_LDS_SWIZZLE, CALL_LDS_DIRECT_SWIZZLE,
  CALL_Q_GLOBAL_CG, CALL_Q_LASTUSE_CS, CALL_Q_VOLATILE_WT, CALL_Q_STREAMING_WB,
  CALL_QG_GLOBAL_CS, CALL_QG_STREAMING_WT, CALL_QG_LASTUSE_CG, CALL_QG_VOLATILE_WB,
- CALL_LDS_DIRECT_SC1, CALL_LDS_DIRECT_NT) = range(16)
+ CALL_LDS_DIRECT_SC1, CALL_LDS_DIRECT_NT, CALL_INDEX_AHEAD) = range(17)
 # the qualifier matrix: source known to be global / generic source (the latter also run LDS -> global)
 STATUS_WAIT_GAVE_UP = 1
 CALL_MATRIX_GLOBAL = (CALL_Q_GLOBAL_CG, CALL_Q_LASTUSE_CS, CALL_Q_VOLATILE_WT, CALL_Q_STREAMING_WB)

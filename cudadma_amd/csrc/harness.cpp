@@ -100,7 +100,10 @@ extern "C" int cudadma_run_case(int case_id, const cudadma_run_t* run, void* str
   const bool swizzled = run->call_style == CUDADMA_CALL_LDS_SWIZZLE || run->call_style == CUDADMA_CALL_LDS_DIRECT_SWIZZLE;
   const bool direct = run->call_style == CUDADMA_CALL_LDS_DIRECT || run->call_style == CUDADMA_CALL_LDS_DIRECT_SWIZZLE ||
                       run->call_style == CUDADMA_CALL_LDS_DIRECT_SC1 || run->call_style == CUDADMA_CALL_LDS_DIRECT_NT;
-  const bool generic_source = run->call_style == CUDADMA_CALL_UNQUALIFIED ||
+  if (run->call_style == CUDADMA_CALL_INDEX_AHEAD)
+    CUDADMA_REQUIRE(d.pattern == CUDADMA_PATTERN_GATHER || d.pattern == CUDADMA_PATTERN_SCATTER,
+                    "the index-ahead call style belongs to the gather and scatter cases");
+  const bool generic_source = run->call_style == CUDADMA_CALL_UNQUALIFIED || run->call_style == CUDADMA_CALL_INDEX_AHEAD ||
                               (run->call_style >= CUDADMA_CALL_QG_GLOBAL_CS && run->call_style <= CUDADMA_CALL_QG_VOLATILE_WB);
   if (swizzled) {
     CUDADMA_REQUIRE(d.pattern == CUDADMA_PATTERN_STRIDED, "swizzled LDS rows are a CudaDMAStrided layout");

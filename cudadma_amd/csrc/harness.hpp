@@ -223,7 +223,7 @@ __device__ __forceinline__ void run_body(Obj& dma, const Args& a, unsigned* lds,
   }
 }
 
-inline bool is_matrix_style(const int call_style) { return call_style >= CUDADMA_CALL_Q_GLOBAL_CG; }
+inline bool is_matrix_style(const int call_style) { return call_style >= CUDADMA_CALL_Q_GLOBAL_CG && call_style <= CUDADMA_CALL_LDS_DIRECT_NT; }
 
 // `kernel` runs the first six call styles, `matrix_kernel` the qualifier matrix.
 template<typename Kernel>

@@ -69,6 +69,18 @@ __global__ void __launch_bounds__(1024) indirect_kernel(const Args a)
           dma.template execute_dma<true, LOAD_CACHE_ALL, STORE_LDS_DIRECT>(index, src, dst);
         }
       }
+    } else if (a.call_style == CUDADMA_CALL_INDEX_AHEAD) {
+      if (a.two_phase) {
+        // as a multi-buffered kernel does it: the next repetition's index words are requested between the phases
+        if (rep == 0) dma.template prefetch_index<true>(index);
+        const int next = rep + 1 < a.reps ? rep + 1 : rep;
+        dma.template start_xfer_async_prefetched<false, LOAD_CACHE_ALL, STORE_WRITE_BACK>(index, src);
+        dma.template prefetch_index<true>(a.index + (size_t)next * a.rep_index_elmts);
+        dma.template wait_xfer_finish<false, LOAD_CACHE_ALL, STORE_WRITE_BACK>(dst);
+      } else {
+        dma.template prefetch_index<true>(index);
+        dma.template execute_dma_prefetched<false, LOAD_CACHE_ALL, STORE_WRITE_BACK>(index, src, dst);
+      }
     } else {
       harness::do_transfer_indexed(dma, a.call_style, a.two_phase, index, src, dst);
     }

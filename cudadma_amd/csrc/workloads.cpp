@@ -80,9 +80,13 @@ static const VariantInfo kStrided[] = {
    "rows (272 B), four workgroups per compute unit"},
 };
 static const VariantInfo kGather[] = {
-  {"manual 4-stage buffering: one DMA group of 2 wavefronts, four CudaDMAIndirect objects"},
+  {"the library's choice: variant 6 (two objects, index words requested one transfer ahead)"},
   {"single buffer: one object, execute_dma"},
-  {"manual double buffer: two objects"},
+  {"manual double buffer: one DMA group of 2 wavefronts, two CudaDMAIndirect objects, each transfer fetches its own index words"},
+  {"manual 4-stage buffering: four objects, each transfer fetches its own index words"},
+  {"four objects, the index words of each object's next tile requested one turn of the ring ahead (prefetch_index)"},
+  {"three objects, index words requested ahead"},
+  {"two objects, index words requested ahead; three workgroups per compute unit (four for tables beyond 1 GiB)"},
 };
 static const VariantInfo kHalo[] = {
   {"warp-specialised, 4 cells per thread as one dwordx4: 1 DMA wavefront keeps the rings of 7 planes in flight in 8 "
@@ -124,6 +128,8 @@ static const VariantInfo kScatter[] = {
   {"single buffer: one LDS tile, one guard"},
   {"manual double buffer: two LDS tiles, two guards"},
   {"not warp-specialised: all four wavefronts fill the tile, meet, and all four scatter it"},
+  {"variant 0 with the index words of the next tile requested before the current tile's stores (prefetch_index)"},
+  {"variant 2 with the index words requested ahead"},
 };
 
 static const VariantInfo* table(int workload, int* count)

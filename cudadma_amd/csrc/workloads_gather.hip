@@ -52,8 +52,12 @@ struct RowsumConsumer {
   }
 };
 
-// STAGES objects share the DMA threads; each has its own 4 KiB buffer.
-template<typename Consumer, int STAGES>
+// STAGES objects share the DMA threads; each has its own 4 KiB buffer.  With PREFETCH the index words of an
+// object's next tile are requested right after its current tile (prefetch_index), one turn of the ring before
+// they are used: the transfer that uses them then waits only for loads older than they are, and the elements of
+// the other STAGES - 1 objects stay in flight across it.  Without it every start_xfer_async fetches its own index
+// words and, a wavefront's loads returning in order, waits until nothing of the thread is in flight any more.
+template<typename Consumer, int STAGES, bool PREFETCH = false>
 __global__ void __launch_bounds__(kDmaThreads + kComputeThreads)
 gather_manual(const float* __restrict__ table, const int* __restrict__ idx, float* __restrict__ out,
               const long long num_tiles)
@@ -75,16 +79,35 @@ gather_manual(const float* __restrict__ table, const int* __restrict__ idx, floa
     if (t + (2 * STAGES - 1) * stride < num_tiles) {
       // Steady state with no branch around any load, entered from a prologue that has none either:
       // waiting for one stage then leaves the loads of the other stages in flight.
-      HIPDMA_FOR_STAGES({
-        d.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(idx + (t + s * stride) * kRecsPerTile, table);
-      })
-      do {
+      if constexpr (PREFETCH) {
+        // a prefetch beyond the last tile reads the last tile's words instead (never used): no branch
+        const long long last = num_tiles - 1;
+        HIPDMA_FOR_STAGES({ d.template prefetch_index<true>(idx + (t + s * stride) * kRecsPerTile); })
         HIPDMA_FOR_STAGES({
-          d.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf[s]);
-          d.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(idx + (t + (s + STAGES) * stride) * kRecsPerTile, table);
+          d.template start_xfer_async_prefetched<true, LOAD_CACHE_ALL, STORE_LDS>(idx + (t + s * stride) * kRecsPerTile, table);
+          d.template prefetch_index<true>(idx + (t + (s + STAGES) * stride) * kRecsPerTile);
         })
-        t += STAGES * stride;
-      } while (t + (2 * STAGES - 1) * stride < num_tiles);
+        do {
+          HIPDMA_FOR_STAGES({
+            d.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf[s]);
+            d.template start_xfer_async_prefetched<true, LOAD_CACHE_ALL, STORE_LDS>(idx + (t + (s + STAGES) * stride) * kRecsPerTile, table);
+            const long long ahead = t + (s + 2 * STAGES) * stride;
+            d.template prefetch_index<true>(idx + (ahead < last ? ahead : last) * kRecsPerTile);
+          })
+          t += STAGES * stride;
+        } while (t + (2 * STAGES - 1) * stride < num_tiles);
+      } else {
+        HIPDMA_FOR_STAGES({
+          d.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(idx + (t + s * stride) * kRecsPerTile, table);
+        })
+        do {
+          HIPDMA_FOR_STAGES({
+            d.template wait_xfer_finish<true, LOAD_CACHE_ALL, STORE_LDS>(buf[s]);
+            d.template start_xfer_async<true, LOAD_CACHE_ALL, STORE_LDS>(idx + (t + (s + STAGES) * stride) * kRecsPerTile, table);
+          })
+          t += STAGES * stride;
+        } while (t + (2 * STAGES - 1) * stride < num_tiles);
+      }
     } else {
       HIPDMA_FOR_STAGES({
         const long long tt = t + s * stride;
@@ -153,12 +176,21 @@ int launch_gather(const float* d_table, const int32_t* d_idx, float* d_out, size
   const long long tiles = (long long)(n_idx / kRecsPerTile);
   hipStream_t s = (hipStream_t)stream;
   const dim3 block(kDmaThreads + kComputeThreads);
+  // Workgroups per compute unit.  Objects that fetch their own index words drain the DMA wavefronts at every
+  // transfer and need many workgroups to cover that (six with several objects, eight with one).  With the index
+  // words requested ahead two objects and three workgroups are enough (0.634 ms on the configuration's 512 MiB
+  // table, which the caches help to serve); a table several times the Infinity Cache wants four (0.724 ms against
+  // 0.775 ms without the prefetch on 1.875 GiB).
+  const int ahead_wgs = n_records * (size_t)kRecBytes <= (1ull << 30) ? 3 : 4;
+  auto grid = [&](const int per_cu) { return dim3((unsigned)workloads::persistent_grid(tiles, per_cu)); };
   switch (variant) {
-    // workgroups per compute unit: six where several tiles are buffered (0.635 ms against 0.645 ms with eight and
-    // 0.683 ms with five on the full-size table), eight where one is
-    case 0: hipLaunchKernelGGL((gather_manual<Consumer, 4>), dim3(workloads::persistent_grid(tiles, 6)), block, 0, s, d_table, d_idx, d_out, tiles); break;
-    case 1: hipLaunchKernelGGL(gather_single<Consumer>, dim3(workloads::persistent_grid(tiles, 8)), block, 0, s, d_table, d_idx, d_out, tiles); break;
-    default: hipLaunchKernelGGL((gather_manual<Consumer, 2>), dim3(workloads::persistent_grid(tiles, 6)), block, 0, s, d_table, d_idx, d_out, tiles); break;
+    case 0:
+    case 6: hipLaunchKernelGGL((gather_manual<Consumer, 2, true>), grid(ahead_wgs), block, 0, s, d_table, d_idx, d_out, tiles); break;
+    case 1: hipLaunchKernelGGL(gather_single<Consumer>, grid(8), block, 0, s, d_table, d_idx, d_out, tiles); break;
+    case 2: hipLaunchKernelGGL((gather_manual<Consumer, 2>), grid(6), block, 0, s, d_table, d_idx, d_out, tiles); break;
+    case 3: hipLaunchKernelGGL((gather_manual<Consumer, 4>), grid(6), block, 0, s, d_table, d_idx, d_out, tiles); break;
+    case 4: hipLaunchKernelGGL((gather_manual<Consumer, 4, true>), grid(ahead_wgs), block, 0, s, d_table, d_idx, d_out, tiles); break;
+    default: hipLaunchKernelGGL((gather_manual<Consumer, 3, true>), grid(ahead_wgs), block, 0, s, d_table, d_idx, d_out, tiles); break;
   }
   CUDADMA_HIP_CHECK(hipGetLastError());
   return CUDADMA_OK;

@@ -69,7 +69,11 @@ enum {
   /* the direct-to-LDS path with the load qualifier in the instruction's cache-policy bits */
   CUDADMA_CALL_LDS_DIRECT_SC1   = 14,  /* <true,  LOAD_CACHE_GLOBAL,    STORE_LDS_DIRECT>          */
   CUDADMA_CALL_LDS_DIRECT_NT    = 15,  /* <true,  LOAD_CACHE_STREAMING, STORE_LDS_DIRECT>          */
-  CUDADMA_CALL_STYLES           = 16
+  /* gather and scatter cases only: prefetch_index() + start_xfer_async_prefetched() / execute_dma_prefetched()
+   * (an addition of this library to CudaDMAIndirect); with two_phase the index words of the next repetition are
+   * requested between the two phases of the current one.  Generic source, so also accepted with reverse = 1. */
+  CUDADMA_CALL_INDEX_AHEAD      = 16,
+  CUDADMA_CALL_STYLES           = 17
 };
 
 typedef struct cudadma_case {

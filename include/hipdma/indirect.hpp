@@ -11,6 +11,15 @@
 // The work split is the slot grid of grid.hpp; every lane fetches the index of
 // the row it works on (lanes of one row read the same word, which the memory
 // pipeline serves as one access), all indices of a step before its data loads.
+//
+// An addition without a counterpart in the reference: prefetch_index() asks for
+// the index words of the first step of a later transfer and leaves them in
+// flight; start_xfer_async_prefetched() / execute_dma_prefetched() then start
+// that transfer from them.  A wavefront's loads return in issue order, so a
+// transfer that fetches its index words itself has to wait for every load the
+// thread still has in flight (the elements of other objects that share the DMA
+// threads) before it can form its first address; with the words requested one
+// transfer ahead, the wait covers only loads that are older than they are.
 #pragma once
 
 #include "grid.hpp"
@@ -110,15 +119,37 @@ public:
 
   template<bool DMA_GLOBAL_LOAD, int DMA_LOAD_QUAL, int DMA_STORE_QUAL>
   __device__ __forceinline__ void start_xfer_async(const int* __restrict__ index_ptr, const void* __restrict__ src_ptr)
+  { start_with<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL, DMA_STORE_QUAL, false>(index_ptr, src_ptr); }
+
+  // Requests the index words of the first step of the transfer that will be started with the same index_ptr
+  // by start_xfer_async_prefetched() or execute_dma_prefetched(); returns with the loads in flight.
+  // DMA_GLOBAL_LOAD says whether index_ptr points to global memory.
+  template<bool DMA_GLOBAL_LOAD = false>
+  __device__ __forceinline__ void prefetch_index(const int* __restrict__ index_ptr)
   {
-    static_assert(DMA_STORE_QUAL != STORE_LDS_DIRECT || (GATHER && DMA_GLOBAL_LOAD),
-                  "STORE_LDS_DIRECT needs a gather from a global source");
-    static_assert(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), "swizzled LDS rows are a CudaDMAStrided layout");
-    HIPDMA_ASSERT(index_ptr != nullptr && (reinterpret_cast<uintptr_t>(src_ptr) % ALIGNMENT) == 0);
-    m_index = index_ptr;
-    m_src = (const char*)src_ptr;
-    if (use_direct<DMA_STORE_QUAL>()) return;
-    load_step<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL>(0, m_grid.begin());
+    HIPDMA_ASSERT(index_ptr != nullptr);
+    hipdma::detail::GridCursor c = m_grid.begin();
+#pragma unroll
+    for (int k = 0; k < MAX_LDS; ++k) {
+      m_idx_next[k] = m_grid.live(k, c)
+          ? (int)hipdma::detail::load_vec<unsigned, DMA_GLOBAL_LOAD, LOAD_CACHE_ALL>(index_ptr + c.row) : 0;
+      m_grid.advance(c);
+    }
+  }
+
+  // start_xfer_async() / execute_dma() for a transfer whose index_ptr went through prefetch_index() after the
+  // previous transfer of this object was started (the words of later steps are still fetched here).
+  template<bool DMA_GLOBAL_LOAD = false, int DMA_LOAD_QUAL = LOAD_CACHE_ALL, int DMA_STORE_QUAL = STORE_WRITE_BACK>
+  __device__ __forceinline__ void start_xfer_async_prefetched(const int* __restrict__ index_ptr,
+                                                              const void* __restrict__ src_ptr)
+  { start_with<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL, DMA_STORE_QUAL, true>(index_ptr, src_ptr); }
+
+  template<bool DMA_GLOBAL_LOAD = false, int DMA_LOAD_QUAL = LOAD_CACHE_ALL, int DMA_STORE_QUAL = STORE_WRITE_BACK>
+  __device__ __forceinline__ void execute_dma_prefetched(const int* __restrict__ index_ptr,
+                                                         const void* __restrict__ src_ptr, void* __restrict__ dst_ptr)
+  {
+    start_with<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL, DMA_STORE_QUAL, true>(index_ptr, src_ptr);
+    wait_xfer_finish<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL, DMA_STORE_QUAL>(dst_ptr);
   }
 
   template<bool DMA_GLOBAL_LOAD, int DMA_LOAD_QUAL, int DMA_STORE_QUAL>
@@ -140,6 +171,19 @@ public:
 
 private:
   __device__ __forceinline__ static int threads_or_block(const int n) { return (n <= 0) ? int(blockDim.x) : n; }
+
+  template<bool DMA_GLOBAL_LOAD, int DMA_LOAD_QUAL, int DMA_STORE_QUAL, bool PREFETCHED>
+  __device__ __forceinline__ void start_with(const int* __restrict__ index_ptr, const void* __restrict__ src_ptr)
+  {
+    static_assert(DMA_STORE_QUAL != STORE_LDS_DIRECT || (GATHER && DMA_GLOBAL_LOAD),
+                  "STORE_LDS_DIRECT needs a gather from a global source");
+    static_assert(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), "swizzled LDS rows are a CudaDMAStrided layout");
+    HIPDMA_ASSERT(index_ptr != nullptr && (reinterpret_cast<uintptr_t>(src_ptr) % ALIGNMENT) == 0);
+    m_index = index_ptr;
+    m_src = (const char*)src_ptr;
+    if (use_direct<DMA_STORE_QUAL>()) return;          // the direct form reads its index words when it issues its loads
+    load_step<DMA_GLOBAL_LOAD, DMA_LOAD_QUAL, PREFETCHED>(0, m_grid.begin());
+  }
 
   __device__ __forceinline__ void init(const int e, const int n, const int t, const int start, const int alt)
   {
@@ -166,14 +210,16 @@ private:
   __device__ __forceinline__ int load_index(const int row) const
   { return (int)hipdma::detail::load_vec<unsigned, GLOBAL_LOAD, LOAD_CACHE_ALL>(m_index + row); }
 
-  template<bool GLOBAL_LOAD, int LOAD_QUAL>
+  // PREFETCHED (step 0 only): the index words are the ones prefetch_index() asked for.
+  template<bool GLOBAL_LOAD, int LOAD_QUAL, bool PREFETCHED = false>
   __device__ __forceinline__ void load_step(const int step, hipdma::detail::GridCursor cur)
   {
     using namespace hipdma::detail;
     GridCursor c = cur;
 #pragma unroll
     for (int k = 0; k < MAX_LDS; ++k) {
-      m_idx[k] = m_grid.live(step * MAX_LDS + k, c) ? load_index<GLOBAL_LOAD>(c.row) : 0;
+      if constexpr (PREFETCHED) m_idx[k] = m_idx_next[k];
+      else m_idx[k] = m_grid.live(step * MAX_LDS + k, c) ? load_index<GLOBAL_LOAD>(c.row) : 0;
       m_grid.advance(c);
     }
     c = cur;
@@ -237,6 +283,7 @@ private:
   const int* m_index;
   const char* m_src;
   int m_idx[MAX_LDS];
+  int m_idx_next[MAX_LDS];      // prefetch_index(): index words of the first step of the next transfer
   chunk_t m_buf[MAX_LDS];
 };
 

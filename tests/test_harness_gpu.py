@@ -23,6 +23,8 @@ def _styles(case):
     styles += list(cd.CALL_MATRIX_GLOBAL) + list(cd.CALL_MATRIX_GENERIC)
     if case.pattern in (cd.PATTERN_SEQUENTIAL, cd.PATTERN_STRIDED, cd.PATTERN_GATHER) and case.alignment in (4, 16):
         styles += [cd.CALL_LDS_DIRECT, cd.CALL_LDS_DIRECT_SC1, cd.CALL_LDS_DIRECT_NT]
+    if case.pattern in (cd.PATTERN_GATHER, cd.PATTERN_SCATTER):
+        styles.append(cd.CALL_INDEX_AHEAD)                    # prefetch_index + the _prefetched calls
     if case.pattern == cd.PATTERN_STRIDED and case.bytes_per_elmt % case.alignment == 0:
         styles.append(cd.CALL_LDS_SWIZZLE)                    # permuted chunks, through registers
         if case.alignment in (4, 16):
@@ -69,6 +71,8 @@ def test_case_reverse_direction_matches_oracle(case_id, device):
     generic = cd.CALL_MATRIX_GENERIC
     plan = ((0, False, cd.CALL_UNQUALIFIED), (1, True, cd.CALL_UNQUALIFIED),
             (2, bool(case_id & 1), generic[case_id % 4]), (3, not (case_id & 1), generic[(case_id + 2) % 4]))
+    if case.pattern in (cd.PATTERN_GATHER, cd.PATTERN_SCATTER):
+        plan += ((4, True, cd.CALL_INDEX_AHEAD), (5, False, cd.CALL_INDEX_AHEAD))      # index words requested ahead
     for flavour, two_phase, style in plan:
         io = CaseIO(case, flavour=flavour, reps=2, data="uniform", reverse=True)
         if io.lds_bytes > 64 * 1024 - 256:

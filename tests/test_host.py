@@ -294,6 +294,15 @@ def test_run_case_refuses_a_short_index_list():
     assert rc == -3 and "index_elmts" in msg, msg
 
 
+def test_run_case_keeps_the_index_ahead_style_to_the_indexed_cases():
+    from tests.cases import CaseIO
+    cases = cd.harness.all_cases()
+    case_id = next(i for i, c in enumerate(cases) if c.pattern == cd.PATTERN_STRIDED and c.level >= 2)
+    io = CaseIO(cases[case_id], flavour=0, reps=1)
+    rc, msg = _fake_run(case_id, cases[case_id], io, call_style=cd.CALL_INDEX_AHEAD)
+    assert rc == -1 and "index-ahead" in msg, msg
+
+
 def test_plan_extents_are_the_footprint_of_the_closed_form():
     """cudadma_plan_extents (the replay the harness checks buffers with) against the footprint the oracle's
     closed form writes, for every compiled case."""
