@@ -42,7 +42,7 @@ PATTERN_KERNELS = {
     "gather_hbm": "gather_manual<(anonymous namespace)::RowsumConsumer, 2, true>",
     "scatter": "scatter_manual<4>",
     "halo": "stencil_ws_vec4<2, 12>",
-    "halo_handshake": "stencil_ws_vec4<0, 12>",
+    "halo_handshake": "stencil_ws_vec4<0, 8>",
     "gemm": "gemm_bf16_all_direct_a64",
     "gemm_warp_specialised": "gemm_bf16_ws_direct4_a64",
 }
@@ -275,11 +275,12 @@ def main():
     n_idx = 32 * 1024 * 1024
     for name, recs, note, bound in (
             ("gather", 4 * 1024 * 1024, "CudaDMAIndirect 32 x 128 B records per tile from the configuration's 512 MiB table (4 Mi records, "
-             "each read 8 times over per launch: most reads are served by L2 and the 256 MB Infinity Cache), row-sum consumer",
+             "each read 8 times over per launch: most reads are served by L2 and the 256 MB Infinity Cache), two objects per DMA "
+             "group with the index words requested one transfer ahead, three workgroups per compute unit, row-sum consumer",
              "infinity cache + hbm"),
             ("gather_hbm", 15 * 1024 * 1024, "the same kernel and index count on a 1.875 GiB table (15 Mi records, each read twice "
              "on average; 7.5 times the Infinity Cache; the objects address the table with int offsets as the reference's do, "
-             "which keeps a table below 2 GiB), row-sum consumer", "hbm")):
+             "which keeps a table below 2 GiB), four workgroups per compute unit, row-sum consumer", "hbm")):
         if not want(name):
             continue
         table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev), 1003)

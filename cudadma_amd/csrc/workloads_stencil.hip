@@ -59,8 +59,14 @@ struct TileWork {
 // `zchunk` carries the chunk length in its low 24 bits; bit 24 asks for the
 // XCD-aware numbering: workgroup b runs on XCD b % 8 (8 XCDs, round-robin
 // dispatch), so giving XCD k the k-th eighth of the tile list keeps tiles that
-// share ghost cells behind the same L2.
+// share ghost cells behind the same L2.  Bit 25 (one z-chunk, tile grid divisible
+// by 2 x 4) makes that eighth a compact block of the tile grid, half of the tiles
+// in x by a quarter in y, instead of a slab over the whole width: the ghost cells
+// on a block's rim are the only ones two XCDs both read from memory, and the rim
+// of a 256 x 128 block is shorter than that of a 512 x 64 slab (read overhead
+// 9.6 % against 14.3 % on the 512^3 grid).
 constexpr int kXcdFlag = 1 << 24;
+constexpr int kXcdBlockFlag = 1 << 25;
 constexpr int kXcds = 8;
 
 __device__ __forceinline__ TileWork tile_work(const float* in, float* out, const int nx, const int ny, const int nz,
@@ -69,10 +75,20 @@ __device__ __forceinline__ TileWork tile_work(const float* in, float* out, const
   const int zchunk = zchunk_and_flags & (kXcdFlag - 1);
   const int tiles_x = nx / kTX, tiles_y = ny / kTY;
   int b = blockIdx.x;
-  if ((zchunk_and_flags & kXcdFlag) && (gridDim.x % kXcds) == 0)
-    b = (b % kXcds) * (gridDim.x / kXcds) + b / kXcds;
-  const int tx = b % tiles_x; b /= tiles_x;
-  const int ty = b % tiles_y; b /= tiles_y;
+  int tx, ty;
+  if (zchunk_and_flags & kXcdBlockFlag) {
+    // XCD k = (kx, ky) of a 2 x 4 arrangement owns the block of tiles_x/2 x tiles_y/4 tiles at (kx, ky)
+    const int xcd = b % kXcds, slot = b / kXcds;
+    const int bw = tiles_x / 2, bh = tiles_y / 4;
+    tx = (xcd % 2) * bw + slot % bw;
+    ty = (xcd / 2) * bh + slot / bw;
+    b = 0;
+  } else {
+    if ((zchunk_and_flags & kXcdFlag) && (gridDim.x % kXcds) == 0)
+      b = (b % kXcds) * (gridDim.x / kXcds) + b / kXcds;
+    tx = b % tiles_x; b /= tiles_x;
+    ty = b % tiles_y; b /= tiles_y;
+  }
   const int z0 = b * zchunk;
   const size_t px = (size_t)nx + 2 * kR, py = (size_t)ny + 2 * kR;
   TileWork w;
@@ -209,8 +225,8 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kXQ = kTX / 4;                          // 8 threads per tile row
 constexpr int kPrefetch = 3;
-constexpr int kQueue = 2 * kR + 1 + kPrefetch;        // planes held in registers: 12 (the kernels take it as QUEUE; deeper
-                                                      // queues ran slower: 16 planes 0.248 ms against 0.200 ms at 512^3)
+constexpr int kQueue = 2 * kR + 1 + kPrefetch;        // planes held in registers: 12 (the warp-specialised kernels take
+                                                      // theirs, QUEUE, from the depth of the DMA wavefront's ring)
 // The z column is a ring of registers: plane z + p of the chunk sits in slot
 // (z + p) % kQueue, and the z loop is unrolled kQueue times so that every slot
 // number is a compile-time constant and no plane is ever moved between registers.
@@ -341,11 +357,11 @@ __device__ __forceinline__ f32x4_t stencil_cells4(const float* __restrict__ plan
 // HIPDMA_FOR_Z unrolls QUEUE (at most 24) steps; the LDS planes rotate with period 4, so QUEUE is a multiple of 4
 template<int QUEUE> struct queue_ok { static_assert(QUEUE >= 2 * kR + 2 && QUEUE <= 24 && QUEUE % 4 == 0, "QUEUE: 12, 16, 20 or 24"); };
 
-// The DMA wavefront keeps the rings of the next kRingAhead planes in flight,
+// The DMA wavefront keeps the rings of the next RING - 1 planes in flight,
 // each in the registers of its own CudaDMAHalo object (manual buffering with
 // two-phase calls, as src/examples/stencil/warp_specialized_manual_buffer.h:54-71,
-// eight objects deep), and lands them one per plane in one of four LDS planes.
-// kRingAhead matches the distance at which the compute threads fetch the
+// eight or twelve objects deep), and lands them one per plane in one of four LDS planes.
+// That distance matches the one at which the compute threads fetch the
 // interior, so a ring is requested while the neighbouring tiles are pulling the
 // same cache lines as their interior.  The objects that hold the registers
 // carry no handshake; the four LDS planes are guarded by cudaDMACustom objects,
@@ -358,22 +374,22 @@ constexpr int kBufs = 4;
 #define STENCIL_INTERIOR_NT 0
 #endif
 constexpr int kRingLoad = STENCIL_RING_LOAD;
-constexpr int kRingObjs = 8;
 #ifndef STENCIL_RING_AHEAD
-#define STENCIL_RING_AHEAD (kRingObjs - 1)
+#define STENCIL_RING_AHEAD (RING - 1)
 #endif
-constexpr int kRingAhead = STENCIL_RING_AHEAD;
-static_assert(kRingAhead >= 2 && kRingAhead < kRingObjs, "a ring has to be requested before it lands and needs an object of its own");
 typedef CudaDMAHalo<false, 16, 32, 4, kDmaThreads, kR, false, kTX, kTY> halo_reg_t;
 
 template<typename T>
-struct Eight {
-  T a0, a1, a2, a3, a4, a5, a6, a7;
+struct Sixteen {
+  T a0, a1, a2, a3, a4, a5, a6, a7, a8, a9, a10, a11, a12, a13, a14, a15;
   template<int I> __device__ __forceinline__ T& get()
   {
     if constexpr (I == 0) return a0; else if constexpr (I == 1) return a1; else if constexpr (I == 2) return a2;
     else if constexpr (I == 3) return a3; else if constexpr (I == 4) return a4; else if constexpr (I == 5) return a5;
-    else if constexpr (I == 6) return a6; else return a7;
+    else if constexpr (I == 6) return a6; else if constexpr (I == 7) return a7; else if constexpr (I == 8) return a8;
+    else if constexpr (I == 9) return a9; else if constexpr (I == 10) return a10; else if constexpr (I == 11) return a11;
+    else if constexpr (I == 12) return a12; else if constexpr (I == 13) return a13; else if constexpr (I == 14) return a14;
+    else return a15;
   }
 };
 template<typename T>
@@ -386,23 +402,30 @@ struct Four {
   }
 };
 
-#define HIPDMA_RING_STEP(J, CHECK, ...) if (!(CHECK) || z0 + (J) < planes) { constexpr int S = (J); const int z = z0 + (J); __VA_ARGS__ }
+#define HIPDMA_RING_STEP(J, CHECK, ...) \
+  if constexpr ((J) < RING) { if (!(CHECK) || z0 + (J) < planes) { constexpr int S = (J); const int z = z0 + (J); __VA_ARGS__ } }
 #define HIPDMA_RING_GROUP(CHECK, ...)                                                                            \
   HIPDMA_RING_STEP(0, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(1, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(2, CHECK, __VA_ARGS__) \
   HIPDMA_RING_STEP(3, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(4, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(5, CHECK, __VA_ARGS__) \
-  HIPDMA_RING_STEP(6, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(7, CHECK, __VA_ARGS__)
+  HIPDMA_RING_STEP(6, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(7, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(8, CHECK, __VA_ARGS__) \
+  HIPDMA_RING_STEP(9, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(10, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(11, CHECK, __VA_ARGS__) \
+  HIPDMA_RING_STEP(12, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(13, CHECK, __VA_ARGS__) HIPDMA_RING_STEP(14, CHECK, __VA_ARGS__) \
+  HIPDMA_RING_STEP(15, CHECK, __VA_ARGS__)
 #define HIPDMA_FOR_RING(planes_expr, ...)                                        \
   {                                                                              \
     const int planes = (planes_expr);                                            \
     int z0 = 0;                                                                  \
-    for (; z0 + kRingObjs <= planes; z0 += kRingObjs) { HIPDMA_RING_GROUP(false, __VA_ARGS__) } \
+    for (; z0 + RING <= planes; z0 += RING) { HIPDMA_RING_GROUP(false, __VA_ARGS__) } \
     if (z0 < planes) { HIPDMA_RING_GROUP(true, __VA_ARGS__) }                    \
   }
-static_assert(kRingObjs == 8 && kRingObjs % kBufs == 0, "HIPDMA_FOR_RING unrolls eight steps");
 
 // One workgroup of five wavefronts per compute unit is the operating point: at most two wavefronts share a
 // SIMD, so the register allocator may use 256 registers per lane instead of spilling to stay under 128.
-template<int SYNC, int QUEUE = kQueue>
+// RING: halo objects of the DMA wavefront; the rings of RING - 1 planes are in flight, and the compute threads
+// fetch the interior at the same distance (QUEUE = RING + 4 planes in registers).  Eight objects (0.7 us of
+// look-ahead per plane step at 512^3) are enough where the handshake paces the DMA wavefront; the kernel with the
+// barrier alone runs 2-3 % faster with twelve.
+template<int SYNC, int RING = 8>
 __global__ void __launch_bounds__(kComputeThreads + kDmaThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
 stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int nx, const int ny, const int nz,
                 const int zchunk, const Coeffs k)
@@ -419,12 +442,14 @@ stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int
   hipdma::GroupBarrier compute_barrier(4, kComputeThreads);
   const TileWork w = tile_work(in, out, nx, ny, nz, zchunk);
   constexpr int kOrigin = kR * kPitch + kR;
+  constexpr int QUEUE = RING + kR;
+  constexpr int kRingAhead = STENCIL_RING_AHEAD;
+  static_assert(RING >= 8 && RING <= 16 && RING % kBufs == 0, "HIPDMA_FOR_RING unrolls 8, 12 or 16 steps");
+  static_assert(kRingAhead >= 2 && kRingAhead < RING, "a ring has to be requested before it lands and needs an object of its own");
 
   if (guard.a0.owns_this_thread()) {
-    Eight<halo_reg_t> ring{halo_reg_t(px, kComputeThreads), halo_reg_t(px, kComputeThreads),
-                           halo_reg_t(px, kComputeThreads), halo_reg_t(px, kComputeThreads),
-                           halo_reg_t(px, kComputeThreads), halo_reg_t(px, kComputeThreads),
-                           halo_reg_t(px, kComputeThreads), halo_reg_t(px, kComputeThreads)};
+    const halo_reg_t one(px, kComputeThreads);          // objects beyond RING are never used and cost nothing
+    Sixteen<halo_reg_t> ring{one, one, one, one, one, one, one, one, one, one, one, one, one, one, one, one};
     // ring of the centre plane of output plane z: padded plane z + kR
     const float* ring0 = w.in_origin + (size_t)kR * in_plane;
     // a request past the last plane re-reads the last one: the loads stay unconditional, nothing lands from them
@@ -448,13 +473,21 @@ stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int
     if constexpr (kRingAhead > 4) { HIPDMA_ISSUE(4, 4) }
     if constexpr (kRingAhead > 5) { HIPDMA_ISSUE(5, 5) }
     if constexpr (kRingAhead > 6) { HIPDMA_ISSUE(6, 6) }
+    if constexpr (kRingAhead > 7) { HIPDMA_ISSUE(7, 7) }
+    if constexpr (kRingAhead > 8) { HIPDMA_ISSUE(8, 8) }
+    if constexpr (kRingAhead > 9) { HIPDMA_ISSUE(9, 9) }
+    if constexpr (kRingAhead > 10) { HIPDMA_ISSUE(10, 10) }
+    if constexpr (kRingAhead > 11) { HIPDMA_ISSUE(11, 11) }
+    if constexpr (kRingAhead > 12) { HIPDMA_ISSUE(12, 12) }
+    if constexpr (kRingAhead > 13) { HIPDMA_ISSUE(13, 13) }
+    if constexpr (kRingAhead > 14) { HIPDMA_ISSUE(14, 14) }
     HIPDMA_LAND(0, 0)
     if constexpr (kLand == 2) { HIPDMA_LAND(1, 1) }
     // iteration z: request plane z + kRingAhead, meet the compute wavefronts, land plane z + kLand
     HIPDMA_FOR_RING(w.planes, {
-      HIPDMA_ISSUE((S + kRingAhead) % kRingObjs, z + kRingAhead)
+      HIPDMA_ISSUE((S + kRingAhead) % RING, z + kRingAhead)
       if constexpr (SYNC != kHandshakeAndGroupBarrier) __syncthreads();
-      HIPDMA_LAND((S + kLand) % kRingObjs, z + kLand)
+      HIPDMA_LAND((S + kLand) % RING, z + kLand)
     })
 #undef HIPDMA_ISSUE
 #undef HIPDMA_LAND
@@ -572,15 +605,28 @@ extern "C" int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int
   if (zchunk < 16) zchunk = 16;
   if (zchunk > nz) zchunk = nz;
   const int chunks = (nz + zchunk - 1) / zchunk;
-  if (workloads::tuning("stencil_xcd_remap", 1) != 2) zchunk |= kXcdFlag;    // knob: 2 turns the XCD-aware numbering off
+  // knob "stencil_xcd_remap": 2 turns the XCD-aware numbering off, 3 keeps the slabs over the whole width
+  const int remap = workloads::tuning("stencil_xcd_remap", 1);
   const long long grid = (long long)(nx / kTX) * (ny / kTY) * chunks;
+  if (remap != 2) zchunk |= kXcdFlag;
+  if (remap == 1 && chunks == 1 && ((nx / kTX) % 2) == 0 && ((ny / kTY) % 4) == 0) zchunk |= kXcdBlockFlag;
   CUDADMA_REQUIRE(grid <= 0x7fffffffLL, "grid too large");
   hipStream_t s = (hipStream_t)stream;
   const dim3 g((unsigned)grid), ws(kComputeThreads + kDmaThreads), all(kComputeThreads);
   switch (variant) {
-    case 0: hipLaunchKernelGGL(stencil_ws_vec4<kBarrierOnly>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
-    case 1: hipLaunchKernelGGL(stencil_ws_vec4<kHandshakeAndBarrier>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
-    case 2: hipLaunchKernelGGL(stencil_ws_vec4<kHandshakeAndGroupBarrier>, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+    // knob "stencil_ring": 8 or 12 halo objects on the DMA wavefront (default: 12 without the handshake, 8 with it)
+    case 0:
+      if (workloads::tuning("stencil_ring", 12) == 8) hipLaunchKernelGGL((stencil_ws_vec4<kBarrierOnly, 8>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);
+      else hipLaunchKernelGGL((stencil_ws_vec4<kBarrierOnly, 12>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);
+      break;
+    case 1:
+      if (workloads::tuning("stencil_ring", 8) == 12) hipLaunchKernelGGL((stencil_ws_vec4<kHandshakeAndBarrier, 12>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);
+      else hipLaunchKernelGGL((stencil_ws_vec4<kHandshakeAndBarrier, 8>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);
+      break;
+    case 2:
+      if (workloads::tuning("stencil_ring", 8) == 12) hipLaunchKernelGGL((stencil_ws_vec4<kHandshakeAndGroupBarrier, 12>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);
+      else hipLaunchKernelGGL((stencil_ws_vec4<kHandshakeAndGroupBarrier, 8>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);
+      break;
     case 3: hipLaunchKernelGGL(stencil_all_vec4, g, all, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
     case 4: hipLaunchKernelGGL(stencil_warp_specialized, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
     default: hipLaunchKernelGGL(stencil_not_specialized, g, all, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;

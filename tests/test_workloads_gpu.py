@@ -303,6 +303,35 @@ def test_halo_stencil_small(device, variant, shape):
     assert np.all(err <= STENCIL_RTOL * np.maximum(np.abs(want), 1.0)), float(err.max())
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("ring", [8, 12])
+@pytest.mark.parametrize("remap", [1, 2, 3])
+@pytest.mark.parametrize("shape", [(64, 128, 21), (192, 256, 9), (96, 64, 40)])
+def test_halo_stencil_under_every_tuning(device, variant, ring, remap, shape):
+    """The depth of the DMA wavefront's ring of halo objects and the numbering of the workgroups (compact blocks
+    per XCD where the tile grid divides by 2 x 4: the first two shapes; slabs; none) are tuning knobs: the result
+    does not depend on them."""
+    nx, ny, nz = shape
+    p = 2 * wl.STENCIL_RADIUS
+    g = ol.uniform((nx + p) * (ny + p) * (nz + p), 4004).reshape(nz + p, ny + p, nx + p)
+    want = np.empty((nz, ny, nx), dtype=np.float32)
+    ol.load().oracle_stencil25(ptr(g), ptr(want), nx, ny, nz, wl.STENCIL_RADIUS)
+    d_in = torch.from_numpy(g).to(device)
+    d_out = torch.full((nz, ny, nx), float("nan"), dtype=torch.float32, device=device)
+    print(f"stencil variant {variant} ring {ring} remap {remap} shape {shape}", flush=True)
+    try:
+        wl.set_tuning("stencil_ring", ring)
+        wl.set_tuning("stencil_xcd_remap", remap)
+        wl.halo_stencil(d_in, d_out, variant)
+        torch.cuda.synchronize()
+    finally:
+        wl.set_tuning("stencil_ring", 0)
+        wl.set_tuning("stencil_xcd_remap", 0)
+    got = d_out.cpu().numpy()
+    err = np.abs(got - want)
+    assert np.all(err <= STENCIL_RTOL * np.maximum(np.abs(want), 1.0)), float(err.max())
+
+
 @pytest.mark.parametrize("variant", [0, 1])     # the kernel the benchmark reports and its form with the empty/full handshake
 def test_halo_stencil_full_size(device, variant):
     n = 512
