@@ -41,7 +41,7 @@ PATTERN_KERNELS = {
     "gather": "gather_manual<(anonymous namespace)::RowsumConsumer, 2, true>",
     "gather_hbm": "gather_manual<(anonymous namespace)::RowsumConsumer, 2, true>",
     "scatter": "scatter_manual<4>",
-    "halo": "stencil_ws_vec4<2, 12>",
+    "halo": "stencil_ws_vec4<2, 8>",
     "halo_handshake": "stencil_ws_vec4<0, 8>",
     "gemm": "gemm_bf16_all_direct_a64",
     "gemm_warp_specialised": "gemm_bf16_ws_direct4_a64",

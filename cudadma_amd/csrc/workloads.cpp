@@ -89,11 +89,10 @@ static const VariantInfo kGather[] = {
   {"two objects, index words requested ahead; three workgroups per compute unit (four for tables beyond 1 GiB)"},
 };
 static const VariantInfo kHalo[] = {
-  {"warp-specialised, 4 cells per thread as one dwordx4: 1 DMA wavefront keeps the rings of 11 planes in flight in 12 "
+  {"warp-specialised, 4 cells per thread as one dwordx4: 1 DMA wavefront keeps the rings of 7 planes in flight in 8 "
    "CudaDMAHalo objects and lands one per plane (execute_dma_no_sync style); one s_barrier per plane orders the ring, "
    "the interior exchange and the reuse of the 4 LDS planes"},
-  {"as variant 0 plus the empty/full handshake (cudaDMACustom guards on the 4 LDS planes) next to the s_barrier; "
-   "8 objects, rings of 7 planes in flight"},
+  {"as variant 0 plus the empty/full handshake (cudaDMACustom guards on the 4 LDS planes) next to the s_barrier"},
   {"as variant 1 but the compute wavefronts meet in an LDS-counter GroupBarrier and the DMA wavefront runs free"},
   {"not warp-specialised, dwordx4 cells: every thread computes, half of them also carry a ring chunk requested one "
    "plane ahead; one LDS plane, two s_barriers per plane"},
@@ -129,8 +128,6 @@ static const VariantInfo kScatter[] = {
   {"single buffer: one LDS tile, one guard"},
   {"manual double buffer: two LDS tiles, two guards"},
   {"not warp-specialised: all four wavefronts fill the tile, meet, and all four scatter it"},
-  {"variant 0 with the index words of the next tile requested before the current tile's stores (prefetch_index)"},
-  {"variant 2 with the index words requested ahead"},
 };
 
 static const VariantInfo* table(int workload, int* count)

@@ -59,12 +59,15 @@ struct TileWork {
 // `zchunk` carries the chunk length in its low 24 bits; bit 24 asks for the
 // XCD-aware numbering: workgroup b runs on XCD b % 8 (8 XCDs, round-robin
 // dispatch), so giving XCD k the k-th eighth of the tile list keeps tiles that
-// share ghost cells behind the same L2.  Bit 25 (one z-chunk, tile grid divisible
-// by 2 x 4) makes that eighth a compact block of the tile grid, half of the tiles
-// in x by a quarter in y, instead of a slab over the whole width: the ghost cells
-// on a block's rim are the only ones two XCDs both read from memory, and the rim
-// of a 256 x 128 block is shorter than that of a 512 x 64 slab (read overhead
-// 9.6 % against 14.3 % on the 512^3 grid).
+// share ghost cells behind the same L2.  That eighth is a slab over the whole
+// width of the grid (two tile rows at 512^3): the only ghost cells two XCDs both
+// read from memory are the rows above and below a slab, 8 rows on 64 (reads
+// 1.16 x the grid, reads + writes 1.08 x).  Bit 25 (one z-chunk, tile grid divisible
+// by 2 x 4) makes it a compact block instead, half of the tiles in x by a quarter
+// in y.  Its rim is shorter in cells, but not in cache lines: the 16 bytes of ghost
+// cells on the inner side of a 1 KiB row piece cost a whole 128-byte line per row,
+// and the measured traffic is higher (reads 1.21 x, total 1.11 x) at the same or a
+// slightly shorter time; the slabs stay the default.
 constexpr int kXcdFlag = 1 << 24;
 constexpr int kXcdBlockFlag = 1 << 25;
 constexpr int kXcds = 8;
@@ -422,9 +425,9 @@ struct Four {
 // One workgroup of five wavefronts per compute unit is the operating point: at most two wavefronts share a
 // SIMD, so the register allocator may use 256 registers per lane instead of spilling to stay under 128.
 // RING: halo objects of the DMA wavefront; the rings of RING - 1 planes are in flight, and the compute threads
-// fetch the interior at the same distance (QUEUE = RING + 4 planes in registers).  Eight objects (0.7 us of
-// look-ahead per plane step at 512^3) are enough where the handshake paces the DMA wavefront; the kernel with the
-// barrier alone runs 2-3 % faster with twelve.
+// fetch the interior at the same distance (QUEUE = RING + 4 planes in registers).  Eight objects (seven planes,
+// 2.8 us of look-ahead at 512^3) are the default; twelve (knob "stencil_ring") measured within +-2.5 % of eight
+// from run to run, in both directions.
 template<int SYNC, int RING = 8>
 __global__ void __launch_bounds__(kComputeThreads + kDmaThreads) __attribute__((amdgpu_waves_per_eu(1, 2)))
 stencil_ws_vec4(const float* __restrict__ in, float* __restrict__ out, const int nx, const int ny, const int nz,
@@ -605,19 +608,19 @@ extern "C" int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int
   if (zchunk < 16) zchunk = 16;
   if (zchunk > nz) zchunk = nz;
   const int chunks = (nz + zchunk - 1) / zchunk;
-  // knob "stencil_xcd_remap": 2 turns the XCD-aware numbering off, 3 keeps the slabs over the whole width
+  // knob "stencil_xcd_remap": 2 turns the XCD-aware numbering off, 4 asks for compact blocks instead of slabs
   const int remap = workloads::tuning("stencil_xcd_remap", 1);
   const long long grid = (long long)(nx / kTX) * (ny / kTY) * chunks;
   if (remap != 2) zchunk |= kXcdFlag;
-  if (remap == 1 && chunks == 1 && ((nx / kTX) % 2) == 0 && ((ny / kTY) % 4) == 0) zchunk |= kXcdBlockFlag;
+  if (remap == 4 && chunks == 1 && ((nx / kTX) % 2) == 0 && ((ny / kTY) % 4) == 0) zchunk |= kXcdBlockFlag;
   CUDADMA_REQUIRE(grid <= 0x7fffffffLL, "grid too large");
   hipStream_t s = (hipStream_t)stream;
   const dim3 g((unsigned)grid), ws(kComputeThreads + kDmaThreads), all(kComputeThreads);
   switch (variant) {
-    // knob "stencil_ring": 8 or 12 halo objects on the DMA wavefront (default: 12 without the handshake, 8 with it)
+    // knob "stencil_ring": 8 (default) or 12 halo objects on the DMA wavefront
     case 0:
-      if (workloads::tuning("stencil_ring", 12) == 8) hipLaunchKernelGGL((stencil_ws_vec4<kBarrierOnly, 8>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);
-      else hipLaunchKernelGGL((stencil_ws_vec4<kBarrierOnly, 12>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);
+      if (workloads::tuning("stencil_ring", 8) == 12) hipLaunchKernelGGL((stencil_ws_vec4<kBarrierOnly, 12>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);
+      else hipLaunchKernelGGL((stencil_ws_vec4<kBarrierOnly, 8>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);
       break;
     case 1:
       if (workloads::tuning("stencil_ring", 8) == 12) hipLaunchKernelGGL((stencil_ws_vec4<kHandshakeAndBarrier, 12>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);

@@ -234,8 +234,8 @@ int cudadma_set_workgroups_per_cu(int value);
  *   "transpose_workgroups"  workgroups to launch for config 2, whatever the per-CU knob says
  *   "transpose_split"  config 2, variant 10: 100 x DMA wavefronts + 10 x compute wavefronts + tiles requested ahead
  *   "stencil_zchunk"     output planes one workgroup marches through in config 4
- *   "stencil_xcd_remap"  config 4 numbers its workgroups so that each XCD gets a compact block of the tile grid (slabs over
- *                        the whole width where the grid does not divide by 2 x 4); 3 asks for the slabs, 2 turns the numbering off
+ *   "stencil_xcd_remap"  config 4 numbers its workgroups so that each XCD gets a slab of the grid over its whole width;
+ *                        4 asks for compact blocks of the tile grid instead (2 x 4 blocks), 2 turns the numbering off
  *   "stencil_ring"       halo objects on the DMA wavefront of config 4's warp-specialised kernels: 8 or 12 */
 int cudadma_set_tuning(const char* name, int value);
 
