@@ -3,7 +3,7 @@ compute unit, timed with HIP events.  The counterpart of the reference's
 src/perf/sequential/param_sweep.py:27-58, which rewrites params_directed.h and recompiles per
 point; here the variants are compiled in and the occupancy is a run-time knob.
 
-    python -m cudadma_amd.sweep [sequential] [strided] [gather] [scatter] [halo] [gemm] [yardsticks] [--wg 0,2,4,8] [--steps 20]
+    python -m cudadma_amd.sweep [sequential] [strided] [gather] [gather_hbm] [scatter] [halo] [gemm] [yardsticks] [--wg 0,2,4,8] [--steps 20]
     python -m cudadma_amd.sweep saxpy sgemv stencil2d        # the reference's example programs, every variant
     python -m cudadma_amd.sweep perf_sequential --wg 2,8     # read-bandwidth probe: element size x DMA wavefronts x buffering
     python -m cudadma_amd.sweep transpose_split              # DMA : compute wavefronts x tiles ahead x workgroups per CU
@@ -75,8 +75,9 @@ def main(argv=None):
                 for wg in wgs:
                     wl.set_workgroups_per_cu(wg)
                     _row(name, v, wg, _time(lambda: wl.strided_transpose(src, dst, v), args.steps), 2 * n * n * 4)
-        elif name == "gather":
-            recs, n_idx = 4 << 20, 32 << 20
+        elif name in ("gather", "gather_hbm"):
+            # the configuration's 512 MiB table, or one of 1.875 GiB (7.5 times the Infinity Cache)
+            recs, n_idx = (4 << 20) if name == "gather" else (15 << 20), 32 << 20
             table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1003)
             idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=dev), recs, 1003)
             out = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, device=dev)
