@@ -25,7 +25,7 @@
 //     direct-to-LDS transfers in flight or spread the loads of one between other instructions
 //     (strided.hpp, base.hpp);
 //   * hipdma::GroupBarrier, a barrier among some of the workgroup's wavefronts (base.hpp);
-//   * HIPDMA_SPIN_LIMIT, HIPDMA_FULL_FENCE, DEBUG_CUDADMA build switches (base.hpp).
+//   * HIPDMA_SPIN_LIMIT, HIPDMA_LDS_ONLY_FENCE, DEBUG_CUDADMA build switches (base.hpp).
 #pragma once
 
 #include "hipdma/base.hpp"

@@ -222,7 +222,7 @@ static_assert(WARP_SIZE == 64, "thread groups are sized in wavefronts");
 
 
 @pytest.mark.parametrize("header,flags", [("cudaDMAv2.h", []), ("hipDMA.h", ["-DWARP_SIZE=64"]), ("cudaDMA.h", []),
-                                          ("cudaDMAv2.h", ["-DDEBUG_CUDADMA"]), ("cudaDMAv2.h", ["-DHIPDMA_FULL_FENCE"]),
+                                          ("cudaDMAv2.h", ["-DDEBUG_CUDADMA"]), ("cudaDMAv2.h", ["-DHIPDMA_LDS_ONLY_FENCE"]),
                                           ("cudaDMAv2.h", ["-DHIPDMA_SPIN_LIMIT=0"])])
 def test_headers_compile_standalone_for_gfx950(tmp_path, header, flags):
     """The drop-in boundary is the include line: a kernel that names only the reference's header must build
