@@ -25,6 +25,11 @@
 //     direct-to-LDS transfers in flight or spread the loads of one between other instructions
 //     (strided.hpp, base.hpp);
 //   * hipdma::GroupBarrier, a barrier among some of the workgroup's wavefronts (base.hpp);
+//   * CudaDMAIndirect::prefetch_index() + start_xfer_async_prefetched() / execute_dma_prefetched(): the index
+//     words of a transfer requested ahead of it, for several objects on the same DMA threads (indirect.hpp);
+//   * a destination pitch as the last constructor argument of CudaDMAHalo (halo.hpp);
+//   * a failure record: a handshake wait that gives up sets HIPDMA_STATUS_WAIT_GAVE_UP in a device word that
+//     hipdma::read_status() returns to the host (base.hpp);
 //   * HIPDMA_SPIN_LIMIT, HIPDMA_LDS_ONLY_FENCE, DEBUG_CUDADMA build switches (base.hpp).
 #pragma once
 
