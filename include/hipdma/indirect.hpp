@@ -128,6 +128,9 @@ public:
   __device__ __forceinline__ void prefetch_index(const int* __restrict__ index_ptr)
   {
     HIPDMA_ASSERT(index_ptr != nullptr);
+#ifdef DEBUG_CUDADMA
+    m_idx_next_from = index_ptr;
+#endif
     hipdma::detail::GridCursor c = m_grid.begin();
 #pragma unroll
     for (int k = 0; k < MAX_LDS; ++k) {
@@ -179,6 +182,9 @@ private:
                   "STORE_LDS_DIRECT needs a gather from a global source");
     static_assert(!hipdma::detail::store_is_swizzled(DMA_STORE_QUAL), "swizzled LDS rows are a CudaDMAStrided layout");
     HIPDMA_ASSERT(index_ptr != nullptr && (reinterpret_cast<uintptr_t>(src_ptr) % ALIGNMENT) == 0);
+#ifdef DEBUG_CUDADMA
+    if constexpr (PREFETCHED) HIPDMA_ASSERT(m_idx_next_from == index_ptr);   // the words on hand belong to this transfer
+#endif
     m_index = index_ptr;
     m_src = (const char*)src_ptr;
     if (use_direct<DMA_STORE_QUAL>()) return;          // the direct form reads its index words when it issues its loads
@@ -284,6 +290,9 @@ private:
   const char* m_src;
   int m_idx[MAX_LDS];
   int m_idx_next[MAX_LDS];      // prefetch_index(): index words of the first step of the next transfer
+#ifdef DEBUG_CUDADMA
+  const int* m_idx_next_from = nullptr;
+#endif
   chunk_t m_buf[MAX_LDS];
 };
 

@@ -206,11 +206,14 @@ __global__ void k(const float* in, const int* idx, float* out)
     a.execute_dma(in, buf);
     b.execute_dma<true>(in, buf);
     c.execute_dma<true, LOAD_CACHE_STREAMING, STORE_WRITE_BACK>(idx, in, buf);
+    c.prefetch_index<true>(idx + 8);
+    c.execute_dma_prefetched<true, LOAD_CACHE_ALL, STORE_WRITE_BACK>(idx + 8, in, buf);
     h.execute_dma(in + 1024, buf + 512);
     d.wait_for_dma_start(); d.finish_async_dma();
   } else {
     a.start_async_dma(); a.wait_for_dma_finish();
     b.start_async_dma(); b.wait_for_dma_finish();
+    c.start_async_dma(); c.wait_for_dma_finish();
     c.start_async_dma(); c.wait_for_dma_finish();
     h.start_async_dma(); h.wait_for_dma_finish();
     d.start_async_dma(); d.wait_for_dma_finish();
