@@ -69,6 +69,21 @@ def test_sequential_copy(device, variant, tiles):
         assert np.array_equal(dst.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("variant", [0, 5, 6])          # what the library picks beyond the Infinity Cache, and its two walks
+def test_sequential_copy_of_a_gibibyte(device, variant):
+    """The size of the benchmark's sequential_hbm row: 65 536 tiles, source and destination cut from one allocation."""
+    m = (1 << 30) // 4
+    pool = torch.empty(2 * m, dtype=torch.float32, device=device)
+    src = wl.fill_uniform(pool[:m], 1001)
+    dst = pool[m:]
+    dst.fill_(float("nan"))
+    wl.sequential_copy(src, dst, variant)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(torch.int32), src.view(torch.int32))
+    head = ol.uniform(1 << 16, 1001)                       # and the source is what the oracle's generator says
+    assert np.array_equal(dst[:1 << 16].cpu().numpy().view(np.uint32), head.view(np.uint32))
+
+
 def test_sequential_copy_rejects_ragged_sizes(device):
     src = torch.zeros(5000, dtype=torch.float32, device=device)
     with pytest.raises(cd.CudaDMAError, match="multiple"):
@@ -189,8 +204,9 @@ def test_gather_small(device, variant, n_tiles):
     assert np.array_equal(got_sum.cpu().numpy().view(np.uint32), want_sum.view(np.uint32))
 
 
-def test_gather_full_size(device):
-    recs, n_idx = 4 * 1024 * 1024, 32 * 1024 * 1024
+@pytest.mark.parametrize("recs", [4 * 1024 * 1024, 15 * 1024 * 1024])     # the configuration's table, and the benchmark's gather_hbm row
+def test_gather_full_size(device, recs):
+    n_idx = 32 * 1024 * 1024
     table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=device), 1003)
     idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=device), recs, 1003)
     out = torch.empty(n_idx * wl.REC_FLOATS, dtype=torch.float32, device=device)
@@ -215,7 +231,7 @@ def test_gather_full_size(device):
     assert np.array_equal(sums.view(-1, wl.REC_FLOATS)[sample].cpu().numpy().view(np.uint32), acc.view(np.uint32))
     # one draw in ten repeats one of the 1024 draws before it (the "10 % duplicates" of the configuration): count the
     # positions of the device-generated list whose value already occurs among the 1024 before it; chance adds
-    # 1024 / 4 Mi = 0.02 % of the positions
+    # 1024 / 4 Mi = 0.02 % of the positions at most
     sample = idx[:1 << 18].cpu().numpy()
     windows = np.lib.stride_tricks.sliding_window_view(sample, 1025)[::37]          # [..., :1024] before, [..., 1024] the draw
     rate = float((windows[:, :1024] == windows[:, 1024:]).any(axis=1).mean())
