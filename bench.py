@@ -43,6 +43,7 @@ PATTERN_KERNELS = {
     "scatter": "scatter_manual<4>",
     "halo": "stencil_ws_vec4<2, 8>",
     "halo_handshake": "stencil_ws_vec4<0, 8>",
+    "halo_wide_tiles": "stencil_ws_vec4<2, 8>",          # the same template in the translation unit compiled for 64 x 16 tiles
     "gemm": "gemm_bf16_all_direct_a64",
     "gemm_warp_specialised": "gemm_bf16_ws_direct4_a64",
 }
@@ -302,7 +303,7 @@ def main():
         del records, perm, table
 
     # ---- config 4: halo stencil ----
-    if want("halo") or want("halo_handshake"):
+    if want("halo") or want("halo_handshake") or want("halo_wide_tiles"):
         g = 512
         p = 2 * wl.STENCIL_RADIUS
         grid_in = wl.fill_uniform(torch.empty((g + p) ** 3, dtype=torch.float32, device=dev), 1004).view(g + p, g + p, g + p)
@@ -314,6 +315,10 @@ def main():
         if want("halo_handshake"):
             ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 1), steps, warmup, SETTLE_MS)
             report(patterns, "halo_handshake", ms, 2 * g ** 3 * 4, "same kernel with the empty/full handshake on the LDS planes next to the s_barrier")
+        if want("halo_wide_tiles"):
+            ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, wl.HALO_WIDE_TILES_VARIANT), steps, warmup, SETTLE_MS)
+            report(patterns, "halo_wide_tiles", ms, 2 * g ** 3 * 4, "the kernel of the halo row with tiles of 64x16 cells (rows of 256 B in memory) "
+                   "instead of the 32x32 tiles the configuration names")
         del grid_in, grid_out
 
     # ---- config 5: bf16 GEMM fed by CudaDMAStrided (MFMA-bound, reported in TFLOP/s); inputs normal(0,1) from seeds 1005 / 2005 ----

@@ -98,6 +98,9 @@ static const VariantInfo kHalo[] = {
    "plane ahead; one LDS plane, two s_barriers per plane"},
   {"warp-specialised, one cell per dword load (first version kept for comparison)"},
   {"not warp-specialised, one cell per dword load"},
+  {"variant 0 with tiles of 64 x 16 cells (rows of 256 B; nx a multiple of 64, ny of 16): 2 to 8 % faster at 512^3, not "
+   "the tile the benchmark configuration names"},
+  {"variant 1 with tiles of 64 x 16 cells"},
 };
 
 static const VariantInfo kGemm[] = {

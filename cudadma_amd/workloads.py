@@ -17,6 +17,7 @@ TRANSPOSE_SPLIT_VARIANT = 10           # cudadma_strided_transpose variant whose
 # knob values = 100 x DMA wavefronts + 10 x compute wavefronts + tiles ahead, every compiled combination
 TRANSPOSE_SPLITS = (111, 112, 121, 122, 141, 142, 211, 212, 221, 222, 241, 242, 311, 312, 321, 322, 411, 412, 421, 422, 441, 442)
 TRANSPOSE_TWO_LDS_TILES_VARIANT = 11    # two LDS tiles and two CudaDMAStrided objects (manual double buffering in LDS)
+HALO_WIDE_TILES_VARIANT = 6            # cudadma_halo_stencil variant 0 with tiles of 64 x 16 cells
 GEMM_WARP_SPECIALISED_VARIANT = 7      # the cudadma_gemm_bf16 variant in which DMA wavefronts feed compute wavefronts
 
 
