@@ -291,7 +291,8 @@ int cudadma_scatter_copy(const float* d_records, const int32_t* d_idx, float* d_
 /* Config 4 (src/examples/stencil/cudaDMA_stencil2D.cu:100-240): 8th-order
  * 25-point star stencil.  d_in is (nx+8) x (ny+8) x (nz+8) floats, x fastest;
  * d_out is nx x ny x nz.  nx, ny multiples of 32.  CudaDMAHalo brings the ring
- * of each 32x32 tile, plane by plane along z. */
+ * of each 32x32 tile, plane by plane along z.  Variants 6 and 7 are variants 0 and 1
+ * with tiles of 64 x 16 cells and need nx a multiple of 64 and ny a multiple of 16. */
 int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int ny, int nz, int variant, void* stream);
 
 /* Config 5 (no GEMM in the reference; nearest: src/examples/sgemv/sgemv_dma.cu:329-388):
