@@ -9,7 +9,7 @@ the timed region.  The other HBM-bound patterns (sequential copy, indirect gathe
 in the opposite direction and the GEMM are timed the same way (HIP events on the launch stream) and reported
 under "patterns" / "gemm".  The sequential copy and the gather are each reported twice: at the size the
 configuration names (64 MiB buffer, 512 MiB table: both working sets are helped by the 256 MB Infinity Cache)
-and at a size that is not (1 GiB buffer, 1.875 GiB table).  "yardsticks" holds what read-only, write-only and
+and at a size that is not (1 GiB buffer, 4 GiB table).  "yardsticks" holds what read-only, write-only and
 copy-shaped streams and the vendor's own device-to-device copy reach on the same 1 GiB buffers in the same
 run; roofline.ceiling is the best read + write yardstick of the run.  Counter-derived fields (HBM traffic per
 launch, matrix-core occupancy) come from profiles/counters.json, which `python -m cudadma_amd.profile_summary`
@@ -279,9 +279,8 @@ def main():
              "each read 8 times over per launch: most reads are served by L2 and the 256 MB Infinity Cache), two objects per DMA "
              "group with the index words requested one transfer ahead, three workgroups per compute unit, row-sum consumer",
              "infinity cache + hbm"),
-            ("gather_hbm", 15 * 1024 * 1024, "the same kernel and index count on a 1.875 GiB table (15 Mi records, each read twice "
-             "on average; 7.5 times the Infinity Cache; the objects address the table with int offsets as the reference's do, "
-             "which keeps a table below 2 GiB), four workgroups per compute unit, row-sum consumer", "hbm")):
+            ("gather_hbm", 32 * 1024 * 1024, "the same kernel and index count on a 4 GiB table (32 Mi records, each read once on "
+             "average; sixteen times the Infinity Cache), four workgroups per compute unit, row-sum consumer", "hbm")):
         if not want(name):
             continue
         table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev), 1003)

@@ -118,8 +118,7 @@ extern "C" int cudadma_scatter_copy(const float* d_records, const int32_t* d_idx
                                     size_t n_idx, int variant, void* stream)
 {
   CUDADMA_REQUIRE((n_idx % kRecsPerTile) == 0, "n_idx (%zu) must be a multiple of %d", n_idx, kRecsPerTile);
-  CUDADMA_REQUIRE(n_records > 0 && n_records * (size_t)kRecBytes <= 0x7fffffffull,
-                  "the table (%zu records) must stay below 2 GiB: the objects address it with int offsets", n_records);
+  CUDADMA_REQUIRE(n_records > 0 && n_records <= 0x7fffffffull, "the table (%zu records) is indexed with int record numbers", n_records);
   if (variant < 0 || variant >= cudadma_num_variants(CUDADMA_WORKLOAD_SCATTER)) {
     cudadma_host::set_error("scatter has no variant %d", variant);
     return CUDADMA_ERANGE;

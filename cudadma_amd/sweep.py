@@ -76,8 +76,8 @@ def main(argv=None):
                     wl.set_workgroups_per_cu(wg)
                     _row(name, v, wg, _time(lambda: wl.strided_transpose(src, dst, v), args.steps), 2 * n * n * 4)
         elif name in ("gather", "gather_hbm"):
-            # the configuration's 512 MiB table, or one of 1.875 GiB (7.5 times the Infinity Cache)
-            recs, n_idx = (4 << 20) if name == "gather" else (15 << 20), 32 << 20
+            # the configuration's 512 MiB table, or one of 4 GiB (sixteen times the Infinity Cache)
+            recs, n_idx = (4 << 20) if name == "gather" else (32 << 20), 32 << 20
             table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1003)
             idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=dev), recs, 1003)
             out = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, device=dev)

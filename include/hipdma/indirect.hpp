@@ -2,7 +2,8 @@
 //   GATHER :  dst[i*S + j] = src[index[i]*BYTES_PER_ELMT + j]
 //   SCATTER:  dst[index[i]*BYTES_PER_ELMT + j] = src[i*S + j]
 // with S = max(alternate_stride, BYTES_PER_ELMT); index[] holds element
-// numbers, not byte offsets.
+// numbers, not byte offsets.  The byte offset on the indexed side is formed in 64 bits, so the indexed buffer
+// may be larger than 2 GiB (the reference forms it in int, include/cudaDMAv2.h:9940-9957).
 //
 // API contract: include/cudaDMAv2.h:9370-14728 (template parameters :9381-9382,
 // dense-side stride :9406, call form :9700-9814, addressing :9940-9957 and
@@ -232,8 +233,9 @@ private:
 #pragma unroll
     for (int k = 0; k < MAX_LDS; ++k) {
       if (m_grid.live(step * MAX_LDS + k, c)) {
-        const int off = GATHER ? (m_idx[k] * m_grid.E + c.col * ALIGNMENT)
-                               : (c.row * m_dense_stride + c.col * ALIGNMENT);
+        // the indexed side takes a 64-bit offset: a table may exceed 2 GiB (the reference multiplies in int)
+        const long long off = GATHER ? ((long long)m_idx[k] * m_grid.E + c.col * ALIGNMENT)
+                                     : (long long)(c.row * m_dense_stride + c.col * ALIGNMENT);
         load_chunk<ALIGNMENT, ALIGNMENT, GLOBAL_LOAD, LOAD_QUAL>(m_buf[k], m_src + off,
                                                                  m_grid.chunk_bytes(ALIGNMENT, c));
       }
@@ -248,8 +250,8 @@ private:
 #pragma unroll
     for (int k = 0; k < MAX_LDS; ++k) {
       if (m_grid.live(step * MAX_LDS + k, cur)) {
-        const int off = GATHER ? (cur.row * m_dense_stride + cur.col * ALIGNMENT)
-                               : (m_idx[k] * m_grid.E + cur.col * ALIGNMENT);
+        const long long off = GATHER ? (long long)(cur.row * m_dense_stride + cur.col * ALIGNMENT)
+                                     : ((long long)m_idx[k] * m_grid.E + cur.col * ALIGNMENT);
         store_chunk<ALIGNMENT, ALIGNMENT, STORE_QUAL>(m_buf[k], dst + off, m_grid.chunk_bytes(ALIGNMENT, cur));
       }
       m_grid.advance(cur);
@@ -274,7 +276,7 @@ private:
         if (m_grid.live(r0 + k, cur)) {
           const int lds_off = cur.row * m_dense_stride + cur.col * ALIGNMENT;
           if constexpr (ALIGNMENT == 16 || ALIGNMENT == 4)
-            load_to_lds<ALIGNMENT, LOAD_QUAL>(m_src + m_idx[k] * m_grid.E + cur.col * ALIGNMENT,
+            load_to_lds<ALIGNMENT, LOAD_QUAL>(m_src + ((long long)m_idx[k] * m_grid.E + cur.col * ALIGNMENT),
                                    dst + (lds_off - lane * ALIGNMENT));
         }
         m_grid.advance(cur);
