@@ -4,6 +4,8 @@ buffer (so stray writes outside the footprint fail too).  The variant matrix is 
 reference's: warp-specialised or not x one-phase or two-phase x unqualified / global /
 fully qualified calls x every template level (cudaDMA_test_strided_v2.cu:693-812), plus
 the direct-to-LDS path that only exists here."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -139,7 +141,7 @@ def test_runtime_parameters_swept(case_id, device):
     which refuses a step outside the buffers) and only then launched."""
     case = _CASES[case_id]
     rng = np.random.default_rng(7000 + case_id)
-    for draw in range(6):
+    for draw in range(int(os.environ.get("CUDADMA_SWEEP_DRAWS", "6"))):     # more draws for an occasional longer hunt
         kw, c = _runtime_draw(case, rng)
         style = _styles(c)[draw % len(_styles(c))]
         two_phase = bool(draw & 1)
