@@ -1,0 +1,220 @@
+"""Builds oracle/_ref/libref_kernels.so: the device kernels of the reference's own v2 test programs, compiled from the
+reference tree where it lies (never copied into this repository) against this repository's cudaDMAv2.h, each behind
+a small launcher that does what the reference's run_experiment() does (one workgroup; for the warp-specialised kernels
+one compute wavefront of 64 threads plus DMA_THREADS DMA threads; dynamic LDS of the buffer size):
+
+    src/tests/test_sequential/cudaDMA_test_sequential_v2.cu   kernels :52-391, launch :432-480
+    src/tests/test_strided/cudaDMA_test_strided_v2.cu         kernels :52-535, launch :586-650
+    src/tests/test_indirect/cudaDMA_test_indirect_v2.cu       kernels :55-536, launch :590-652
+    src/tests/test_halo/cudaDMA_test_halo.cu                  kernel :180-232 with its element helpers :52-90
+                                                              (first-generation cudaDMAHalo, "cudaDMA.h"), launch :261-268
+
+The kernels take their parameters as template arguments named like the macros the reference's Makefiles pass
+(-DALIGNMENT=... and so on); here the template heads are left out and the macros of one parameter set are defined in
+front of the text, one translation unit per (program, parameter set).  Test infrastructure only: the GPU tests run
+these kernels and compare their output with the oracle's closed forms.
+
+    python oracle/build_ref_kernels.py          # needs /root/reference and hipcc; writes only into oracle/_ref/
+"""
+import concurrent.futures
+import os
+import re
+import shutil
+import subprocess
+import sys
+import tempfile
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+REFERENCE_TESTS = "/root/reference/src/tests"
+OUT_DIR = os.path.join(HERE, "_ref")
+OUT = os.path.join(OUT_DIR, "libref_kernels.so")
+
+PROGRAMS = {
+    "sequential": "test_sequential/cudaDMA_test_sequential_v2.cu",
+    "strided": "test_strided/cudaDMA_test_strided_v2.cu",
+    "indirect": "test_indirect/cudaDMA_test_indirect_v2.cu",
+}
+# Parameter sets (the macros of the reference's param_sweep_v2.py); thread counts in multiples of 64.  ALIGN_OFFSET is
+# in floats and keeps the ALIGNMENT; sizes are chosen to hit whole chunks, 4/8/12-byte tails and several steps.
+PARAMETER_SETS = {
+    "a16_e1024_t128_n8": dict(ALIGNMENT=16, ALIGN_OFFSET=0, BYTES_PER_THREAD=64, BYTES_PER_ELMT=1024, DMA_THREADS=128, NUM_ELMTS=8),
+    "a4_e132_t64_n5": dict(ALIGNMENT=4, ALIGN_OFFSET=1, BYTES_PER_THREAD=16, BYTES_PER_ELMT=132, DMA_THREADS=64, NUM_ELMTS=5),
+    "a8_e40_t192_n33": dict(ALIGNMENT=8, ALIGN_OFFSET=2, BYTES_PER_THREAD=24, BYTES_PER_ELMT=40, DMA_THREADS=192, NUM_ELMTS=33),
+    "a16_e1004_t256_n3": dict(ALIGNMENT=16, ALIGN_OFFSET=4, BYTES_PER_THREAD=32, BYTES_PER_ELMT=1004, DMA_THREADS=256, NUM_ELMTS=3),
+    "a16_e6000_t64_n2": dict(ALIGNMENT=16, ALIGN_OFFSET=0, BYTES_PER_THREAD=16, BYTES_PER_ELMT=6000, DMA_THREADS=64, NUM_ELMTS=2),
+}
+COMPUTE_THREADS = 64          # one compute wavefront, where the reference launches one warp
+
+# kernel numbers of a launcher: 0-3 warp-specialised with four / three / two / one compile-time parameters (the
+# sequential program has no "four"), 4-7 the same not warp-specialised
+_LAUNCHERS = {
+    "sequential": r'''
+extern "C" int refk_sequential_@SET@(int which, float* d_in, float* d_out, int* /*unused*/, int single, int qualified, void* stream)
+{
+  const int buffer_size = BYTES_PER_ELMT / 4 + ALIGN_OFFSET;
+  const size_t lds = (size_t)buffer_size * 4;
+  hipStream_t s = (hipStream_t)stream;
+  const bool one = single != 0, q = qualified != 0;
+  switch (which) {
+    case 1: hipLaunchKernelGGL(special_xfer_three, dim3(1), dim3(@C@ + DMA_THREADS), lds, s, d_in, d_out, buffer_size, @C@, one, q); break;
+    case 2: hipLaunchKernelGGL(special_xfer_two, dim3(1), dim3(@C@ + DMA_THREADS), lds, s, d_in, d_out, buffer_size, @C@, DMA_THREADS, one, q); break;
+    case 3: hipLaunchKernelGGL(special_xfer_one, dim3(1), dim3(@C@ + DMA_THREADS), lds, s, d_in, d_out, buffer_size, @C@, DMA_THREADS, BYTES_PER_ELMT, one, q); break;
+    case 5: hipLaunchKernelGGL(nonspec_xfer_three, dim3(1), dim3(DMA_THREADS), lds, s, d_in, d_out, buffer_size, one, q); break;
+    case 6: hipLaunchKernelGGL(nonspec_xfer_two, dim3(1), dim3(DMA_THREADS), lds, s, d_in, d_out, buffer_size, one, q); break;
+    case 7: hipLaunchKernelGGL(nonspec_xfer_one, dim3(1), dim3(DMA_THREADS), lds, s, d_in, d_out, buffer_size, BYTES_PER_ELMT, one, q); break;
+    default: return -1;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+''',
+    "strided": r'''
+extern "C" int refk_strided_@SET@(int which, float* d_in, float* d_out, int* /*unused*/, int single, int qualified, void* stream)
+{
+  // the strides of the reference's run_experiment: the element rounded up to the alignment, both sides
+  const int element = BYTES_PER_ELMT / 4, per = ALIGNMENT / 4;
+  const int stride_floats = element + ((element % per) ? per - element % per : 0);
+  const int stride = stride_floats * 4;
+  const int buffer_size = NUM_ELMTS * stride_floats + ALIGN_OFFSET;
+  const size_t lds = (size_t)buffer_size * 4;
+  hipStream_t s = (hipStream_t)stream;
+  const bool one = single != 0, q = qualified != 0;
+  switch (which) {
+    case 0: hipLaunchKernelGGL(special_xfer_four, dim3(1), dim3(@C@ + DMA_THREADS), lds, s, d_in, d_out, stride, stride, @C@, buffer_size, one, q); break;
+    case 1: hipLaunchKernelGGL(special_xfer_three, dim3(1), dim3(@C@ + DMA_THREADS), lds, s, d_in, d_out, stride, stride, @C@, NUM_ELMTS, buffer_size, one, q); break;
+    case 2: hipLaunchKernelGGL(special_xfer_two, dim3(1), dim3(@C@ + DMA_THREADS), lds, s, d_in, d_out, stride, stride, @C@, DMA_THREADS, NUM_ELMTS, buffer_size, one, q); break;
+    case 3: hipLaunchKernelGGL(special_xfer_one, dim3(1), dim3(@C@ + DMA_THREADS), lds, s, d_in, d_out, stride, stride, @C@, DMA_THREADS, BYTES_PER_ELMT, NUM_ELMTS, buffer_size, one, q); break;
+    case 4: hipLaunchKernelGGL(nonspec_xfer_four, dim3(1), dim3(DMA_THREADS), lds, s, d_in, d_out, stride, stride, buffer_size, one, q); break;
+    case 5: hipLaunchKernelGGL(nonspec_xfer_three, dim3(1), dim3(DMA_THREADS), lds, s, d_in, d_out, stride, stride, NUM_ELMTS, buffer_size, one, q); break;
+    case 6: hipLaunchKernelGGL(nonspec_xfer_two, dim3(1), dim3(DMA_THREADS), lds, s, d_in, d_out, stride, stride, NUM_ELMTS, buffer_size, one, q); break;
+    case 7: hipLaunchKernelGGL(nonspec_xfer_one, dim3(1), dim3(DMA_THREADS), lds, s, d_in, d_out, stride, stride, BYTES_PER_ELMT, NUM_ELMTS, buffer_size, one, q); break;
+    default: return -1;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+''',
+    "indirect": r'''
+extern "C" int refk_indirect_@SET@(int which, float* d_in, float* d_out, int* d_offsets, int single, int qualified, void* stream)
+{
+  const int buffer_size = NUM_ELMTS * BYTES_PER_ELMT / 4 + ALIGN_OFFSET;
+  const size_t lds = (size_t)buffer_size * 4;
+  hipStream_t s = (hipStream_t)stream;
+  const bool one = single != 0, q = qualified != 0;
+  switch (which) {
+    case 0: hipLaunchKernelGGL(special_xfer_four, dim3(1), dim3(@C@ + DMA_THREADS), lds, s, d_in, d_out, d_offsets, @C@, buffer_size, one, q); break;
+    case 1: hipLaunchKernelGGL(special_xfer_three, dim3(1), dim3(@C@ + DMA_THREADS), lds, s, d_in, d_out, d_offsets, @C@, NUM_ELMTS, buffer_size, one, q); break;
+    case 2: hipLaunchKernelGGL(special_xfer_two, dim3(1), dim3(@C@ + DMA_THREADS), lds, s, d_in, d_out, d_offsets, @C@, DMA_THREADS, NUM_ELMTS, buffer_size, one, q); break;
+    case 3: hipLaunchKernelGGL(special_xfer_one, dim3(1), dim3(@C@ + DMA_THREADS), lds, s, d_in, d_out, d_offsets, @C@, DMA_THREADS, BYTES_PER_ELMT, NUM_ELMTS, buffer_size, one, q); break;
+    case 4: hipLaunchKernelGGL(nonspec_xfer_four, dim3(1), dim3(DMA_THREADS), lds, s, d_in, d_out, d_offsets, buffer_size, one, q); break;
+    case 5: hipLaunchKernelGGL(nonspec_xfer_three, dim3(1), dim3(DMA_THREADS), lds, s, d_in, d_out, d_offsets, NUM_ELMTS, buffer_size, one, q); break;
+    case 6: hipLaunchKernelGGL(nonspec_xfer_two, dim3(1), dim3(DMA_THREADS), lds, s, d_in, d_out, d_offsets, NUM_ELMTS, buffer_size, one, q); break;
+    case 7: hipLaunchKernelGGL(nonspec_xfer_one, dim3(1), dim3(DMA_THREADS), lds, s, d_in, d_out, d_offsets, BYTES_PER_ELMT, NUM_ELMTS, buffer_size, one, q); break;
+    default: return -1;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+''',
+}
+# Instantiations of the halo test kernel dma_ld_test<ALIGNMENT, ALIGN_OFFSET, ELMT_TYPE, RADIUS, CORNERS>, taken from the
+# combinations run_all_experiments() of the reference allows (RADIUS * sizeof(ELMT_TYPE) keeps the ALIGNMENT)
+HALO_INSTANCES = [
+    dict(ALIGNMENT=4, ELMT="float", ELMT_BYTES=4, RADIUS=1, CORNERS=False),
+    dict(ALIGNMENT=4, ELMT="float", ELMT_BYTES=4, RADIUS=3, CORNERS=True),
+    dict(ALIGNMENT=8, ELMT="float", ELMT_BYTES=4, RADIUS=2, CORNERS=True),
+    dict(ALIGNMENT=8, ELMT="float2", ELMT_BYTES=8, RADIUS=1, CORNERS=False),
+    dict(ALIGNMENT=16, ELMT="float", ELMT_BYTES=4, RADIUS=4, CORNERS=False),
+    dict(ALIGNMENT=16, ELMT="float", ELMT_BYTES=4, RADIUS=4, CORNERS=True),
+    dict(ALIGNMENT=16, ELMT="float2", ELMT_BYTES=8, RADIUS=2, CORNERS=True),
+    dict(ALIGNMENT=16, ELMT="float4", ELMT_BYTES=16, RADIUS=1, CORNERS=False),
+]
+
+
+def _halo_launcher():
+    cases = "".join(
+        f"    case {i}: hipLaunchKernelGGL((dma_ld_test<{h['ALIGNMENT']}, 0, {h['ELMT']}, {h['RADIUS']}, {'true' if h['CORNERS'] else 'false'}>), "
+        f"dim3(1), dim3(@C@ + dma_threads), (size_t)((dimx + 2 * {h['RADIUS']}) * (dimy + 2 * {h['RADIUS']})) * {h['ELMT_BYTES']}, s, "
+        f"({h['ELMT']}*)d_in, ({h['ELMT']}*)d_out, dimx, dimy, pitch, (dimx + 2 * {h['RADIUS']}) * (dimy + 2 * {h['RADIUS']}), @C@, dma_threads); break;\n"
+        for i, h in enumerate(HALO_INSTANCES))
+    return ('''
+extern "C" int refk_halo(int instance, void* d_in, void* d_out, int dimx, int dimy, int pitch, int dma_threads, void* stream)
+{
+  hipStream_t s = (hipStream_t)stream;
+  switch (instance) {
+''' + cases + '''    default: return -1;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+''').replace("@C@", str(COMPUTE_THREADS))
+
+
+def _compile_halo_unit(hipcc, scratch):
+    text = open(os.path.join(REFERENCE_TESTS, "test_halo/cudaDMA_test_halo.cu")).read()
+    start = text.index("template<typename TYPE>")                    # initialize<> / get_val<> come before the kernel
+    end = _END_OF_FUNCTION.search(text, text.index("dma_ld_test")).end()
+    source = ('#include <hip/hip_runtime.h>\n#include <stdio.h>\n#include <stdlib.h>\n#include <assert.h>\n#include <math.h>\n'
+              '#include "cudaDMA.h"\nnamespace {\n' + text[start:end] + "\n}\n" + _halo_launcher())
+    src, obj = os.path.join(scratch, "halo.hip"), os.path.join(scratch, "halo.o")
+    with open(src, "w") as f:
+        f.write(source)
+    cmd = [hipcc, "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unused-function", "-I", os.path.join(ROOT, "include"),
+           "-c", src, "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("halo:\n" + "\n".join(l for l in res.stderr.splitlines() if "error" in l)[:3000])
+    return obj
+
+
+_END_OF_FUNCTION = re.compile(r"^\}[ \t]*$", re.M)
+
+
+def reference_kernels(program):
+    """The text of every __global__ function of the program, template heads left out."""
+    text = open(os.path.join(REFERENCE_TESTS, PROGRAMS[program])).read()
+    return [text[m.start():_END_OF_FUNCTION.search(text, m.start()).end()] for m in re.finditer(r"^__global__", text, re.M)]
+
+
+def _compile_unit(hipcc, scratch, program, set_name, macros):
+    # each unit in a namespace of its own would hide the extern "C" launcher; static kernels would not launch: the
+    # kernels of different units carry the same names, so every unit becomes a code object of its own (-fgpu-rdc off)
+    # and the kernels are given internal linkage through an unnamed namespace around the reference's text
+    source = ('#include <hip/hip_runtime.h>\n#include "cudaDMAv2.h"\n' +
+              "".join(f"#define {k} {v}\n" for k, v in macros.items()) +
+              "namespace {\n" + "\n".join(reference_kernels(program)) + "\n}\n" +
+              _LAUNCHERS[program].replace("@SET@", set_name).replace("@C@", str(COMPUTE_THREADS)))
+    src = os.path.join(scratch, f"{program}_{set_name}.hip")
+    obj = os.path.join(scratch, f"{program}_{set_name}.o")
+    with open(src, "w") as f:
+        f.write(source)
+    cmd = [hipcc, "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-I", os.path.join(ROOT, "include"), "-c", src, "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"{program} {set_name}:\n" + "\n".join(l for l in res.stderr.splitlines() if "error" in l)[:3000])
+    return obj
+
+
+def has_unit(program, macros):
+    """An indexed transfer puts element i at i * BYTES_PER_ELMT: its element size has to keep the ALIGNMENT."""
+    return program != "indirect" or macros["BYTES_PER_ELMT"] % macros["ALIGNMENT"] == 0
+
+
+def build(jobs=None):
+    if not os.path.isdir(REFERENCE_TESTS):
+        print(f"{REFERENCE_TESTS} is not present: nothing to build")
+        return None
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    os.makedirs(OUT_DIR, exist_ok=True)
+    units = [(p, s, m) for p in PROGRAMS for s, m in PARAMETER_SETS.items() if has_unit(p, m)]
+    with tempfile.TemporaryDirectory() as scratch:        # the reference's text exists only here, and only for the build
+        with concurrent.futures.ThreadPoolExecutor(max_workers=jobs or min(16, os.cpu_count() or 8)) as pool:
+            halo = pool.submit(_compile_halo_unit, hipcc, scratch)
+            objs = list(pool.map(lambda u: _compile_unit(hipcc, scratch, *u), units)) + [halo.result()]
+        subprocess.check_call([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950"] + objs + ["-o", OUT])
+    print(f"built {OUT}: {len(units)} units ({len(PROGRAMS)} programs, {len(PARAMETER_SETS)} parameter sets) + the halo "
+          f"test kernel in {len(HALO_INSTANCES)} instantiations")
+    return OUT
+
+
+if __name__ == "__main__":
+    sys.exit(0 if build() or not os.path.isdir(REFERENCE_TESTS) else 1)
