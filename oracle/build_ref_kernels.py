@@ -8,6 +8,13 @@ one compute wavefront of 64 threads plus DMA_THREADS DMA threads; dynamic LDS of
     src/tests/test_indirect/cudaDMA_test_indirect_v2.cu       kernels :55-536, launch :590-652
     src/tests/test_halo/cudaDMA_test_halo.cu                  kernel :180-232 with its element helpers :52-90
                                                               (first-generation cudaDMAHalo, "cudaDMA.h"), launch :261-268
+    src/examples/saxpy/saxpy_cudaDMA_kernel.cu                the eight saxpy kernels :54-420 (two of them on
+                                                              cudaDMASequential), launch saxpy_cudaDMA.cu:138
+    src/examples/stencil/*_buffer.h + stencil_math.h          the five buffering styles of the 2-D stencil on
+                                                              CudaDMAStrided, launch cudaDMA_stencil2D.cu:118-185
+    src/examples/sgemv/sgemv_dma.cu                           its seven DMA kernels :141-620 (cudaDMASequential for the
+                                                              vector, cudaDMAStrided for the matrix panel), each under
+                                                              its own -D switch with its own sizes :79-133, launch :845-856
 
 The kernels take their parameters as template arguments named like the macros the reference's Makefiles pass
 (-DALIGNMENT=... and so on); here the template heads are left out and the macros of one parameter set are defined in
@@ -147,6 +154,132 @@ extern "C" int refk_halo(int instance, void* d_in, void* d_out, int dimx, int di
 ''').replace("@C@", str(COMPUTE_THREADS))
 
 
+# saxpy example: the parameters of its params_directed.h in multiples of 64 threads
+SAXPY = dict(CTA_COUNT=96, COMPUTE_THREADS_PER_CTA=256, NUM_ITERS=16, DMA_THREADS_PER_LD=64, BYTES_PER_DMA_THREAD=32)
+SAXPY_KERNELS = ["saxpy_baseline", "saxpy_float4s", "saxpy_shmem", "saxpy_shmem_doublebuffer", "saxpy_float4s_shmem",
+                 "saxpy_float4s_shmem_doublebuffer", "saxpy_cudaDMA", "saxpy_cudaDMA_doublebuffer"]
+
+
+def _compile_saxpy_unit(hipcc, scratch):
+    text = open("/root/reference/src/examples/saxpy/saxpy_cudaDMA_kernel.cu").read()
+    kernels = [text[m.start():_END_OF_FUNCTION.search(text, m.start()).end()] for m in re.finditer(r"^__global__", text, re.M)]
+    defines = "".join(f"#define {k} {v}\n" for k, v in SAXPY.items()) + "#define DMA_SZ (4 * COMPUTE_THREADS_PER_CTA)\n"
+    # threads per workgroup as the reference's THREADS_PER_CTA macro has them: the compute threads, plus two DMA
+    # groups for saxpy_cudaDMA and four for saxpy_cudaDMA_doublebuffer
+    cases = "".join(
+        f"    case {i}: hipLaunchKernelGGL({k}, dim3(CTA_COUNT), dim3(COMPUTE_THREADS_PER_CTA + "
+        f"{ {'saxpy_cudaDMA': 2, 'saxpy_cudaDMA_doublebuffer': 4}.get(k, 0) } * DMA_THREADS_PER_LD), 0, s, d_y, d_x, a, (clock_t*)d_timers); break;\n"
+        for i, k in enumerate(SAXPY_KERNELS))
+    launcher = ('''
+extern "C" int refk_saxpy(int which, float* d_y, float* d_x, float a, void* d_timers, void* stream)
+{
+  hipStream_t s = (hipStream_t)stream;
+  switch (which) {
+''' + cases + '''    default: return -1;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+''')
+    source = ('#include <hip/hip_runtime.h>\n#include <stdio.h>\n#include <stdlib.h>\n#include <time.h>\n#include "cudaDMA.h"\n' + defines +
+              "namespace {\n" + "\n".join(kernels) + "\n}\n" + launcher)
+    src, obj = os.path.join(scratch, "saxpy.hip"), os.path.join(scratch, "saxpy.o")
+    with open(src, "w") as f:
+        f.write(source)
+    cmd = [hipcc, "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-I", os.path.join(ROOT, "include"), "-c", src, "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("saxpy:\n" + "\n".join(l for l in res.stderr.splitlines() if "error" in l)[:3000])
+    return obj
+
+
+# sgemv example: the seven configurations of sgemv_dma.cu:79-133; the matrix is SGEMV_N x SGEMV_N (the reference's 896
+# does not divide by the 1024 vector elements of its own VEC_DOUBLE configuration)
+SGEMV_CONFIGS = ["VEC_SINGLE", "VEC_DOUBLE", "VEC_MANUAL", "BOTH_SINGLE", "BOTH_DOUBLE", "BOTH_MANUAL", "MAT_SINGLE"]
+SGEMV_N = 1024
+
+
+def _compile_sgemv_unit(hipcc, scratch, config):
+    text = open("/root/reference/src/examples/sgemv/sgemv_dma.cu").read()
+    last = "#endif // MAT_SINGLE"
+    body = text[text.index("#define num_threads"):text.index(last) + len(last)]
+    # thread groups in wavefronts of 64; `blockIdx.x**COMPUTE_THREADS_PER_CTA` (:468, :479) is a typing slip for one `*`
+    body = re.sub(r"(#define DMA_THREADS_PER_LD\s+)32", r"\g<1>64", body).replace("blockIdx.x**COMPUTE", "blockIdx.x*COMPUTE")
+    launcher = '''
+extern "C" int refk_sgemv_@CFG@(int n, int m, float alpha, float* d_A, float* d_x, float* d_y, void* stream)
+{
+  const int n1 = (m / COMPUTE_THREADS_PER_CTA) * COMPUTE_THREADS_PER_CTA;
+  const int blocks = (n + COMPUTE_THREADS_PER_CTA - 1) / COMPUTE_THREADS_PER_CTA;
+  hipLaunchKernelGGL(DMA_KERNEL, dim3(blocks), dim3(COMPUTE_THREADS_PER_CTA + DMA_LDS * DMA_THREADS_PER_LD), 0,
+                     (hipStream_t)stream, n, m, n1, alpha, d_A, n, d_x, d_y);
+  return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+'''.replace("@CFG@", config)
+    source = (f"#define {config} 1\n#define SIZE_N {SGEMV_N}\n#define SIZE_M SIZE_N\n"
+              '#include <hip/hip_runtime.h>\n#include <cstdio>\n#include "cudaDMA.h"\nnamespace {\n' + body + "\n}\n" + launcher)
+    src, obj = os.path.join(scratch, f"sgemv_{config}.hip"), os.path.join(scratch, f"sgemv_{config}.o")
+    with open(src, "w") as f:
+        f.write(source)
+    cmd = [hipcc, "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-I", os.path.join(ROOT, "include"), "-c", src, "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"sgemv {config}:\n" + "\n".join(l for l in res.stderr.splitlines() if "error" in l)[:3000])
+    return obj
+
+
+# stencil example: the directed parameters of params_directed.h:20-24 (tiles of 32 x 4 float2 cells, radius 4, 12 x 16
+# bytes per DMA thread), one DMA wavefront of 64 per load in place of one warp
+STENCIL_HEADERS = ["warp_specialized_single_buffer", "warp_specialized_double_buffer", "warp_specialized_manual_buffer",
+                   "non_warp_specialized_single_buffer", "non_warp_specialized_double_buffer"]
+STENCIL = dict(TILE_X=32, TILE_Y=4, RADIUS=4, DMA_THREADS_PER_LD=64)
+
+
+def _compile_stencil_unit(hipcc, scratch):
+    base = "/root/reference/src/examples/stencil"
+
+    def without_includes(path):
+        return "\n".join(l for l in open(path).read().splitlines() if not l.strip().startswith("#include"))
+    body = without_includes(os.path.join(base, "stencil_math.h")) + "\n"
+    for h in STENCIL_HEADERS:
+        # non_warp_specialized_double_buffer.h calls member templates of a dependent type without the `template`
+        # keyword, which nvcc lets pass and clang does not
+        body += re.sub(r"(\w)\.(start_xfer_async|wait_xfer_finish|execute_dma)<", r"\1.template \2<",
+                       without_includes(os.path.join(base, h + ".h"))) + "\n"
+    t = STENCIL
+    ws = f"16, 12 * 16, {t['TILE_X']}, {t['TILE_Y']}, {t['RADIUS']}, {t['DMA_THREADS_PER_LD']}"
+    nws = f"16, 12 * 16, {t['TILE_X']}, {t['TILE_Y']}, {t['RADIUS']}"
+    compute = t["TILE_X"] * t["TILE_Y"]
+    dma_groups = [1, 2, 1, 0, 0]                       # total_warps of cudaDMA_stencil2D.cu:122,135,149,163,176
+    cases = "".join(
+        f"    case {i}: hipLaunchKernelGGL((stencil_2D_{h}<{ws if d else nws}>), grid, dim3({compute} + {d} * {t['DMA_THREADS_PER_LD']}), 0, s, "
+        f"(const float2*)d_src, (float2*)d_dst, offset, row_stride, slice_stride, dimz); break;\n"
+        for i, (h, d) in enumerate(zip(STENCIL_HEADERS, dma_groups)))
+    launcher = ('''
+extern "C" int refk_stencil2d(int which, const void* d_src, void* d_dst, int dimx, int dimy, int dimz, void* stream)
+{
+  const int row_stride = dimx + 2 * @R@, slice_stride = (dimy + 2 * @R@) * row_stride;
+  const int offset = @R@ * slice_stride + @R@ * row_stride + @R@;
+  const dim3 grid(dimx / @TX@, dimy / @TY@);
+  hipStream_t s = (hipStream_t)stream;
+  switch (which) {
+''' + cases + '''    default: return -1;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -2;
+}
+''').replace("@R@", str(t["RADIUS"])).replace("@TX@", str(t["TILE_X"])).replace("@TY@", str(t["TILE_Y"]))
+    source = '#include <hip/hip_runtime.h>\n#include "cudaDMAv2.h"\nnamespace {\n' + body + "\n}\n" + launcher
+    src, obj = os.path.join(scratch, "stencil2d.hip"), os.path.join(scratch, "stencil2d.o")
+    with open(src, "w") as f:
+        f.write(source)
+    cmd = [hipcc, "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-I", os.path.join(ROOT, "include"), "-c", src, "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("stencil2d:\n" + "\n".join(l for l in res.stderr.splitlines() if "error" in l)[:3000])
+    return obj
+
+
 def _compile_halo_unit(hipcc, scratch):
     text = open(os.path.join(REFERENCE_TESTS, "test_halo/cudaDMA_test_halo.cu")).read()
     start = text.index("template<typename TYPE>")                    # initialize<> / get_val<> come before the kernel
@@ -208,11 +341,14 @@ def build(jobs=None):
     units = [(p, s, m) for p in PROGRAMS for s, m in PARAMETER_SETS.items() if has_unit(p, m)]
     with tempfile.TemporaryDirectory() as scratch:        # the reference's text exists only here, and only for the build
         with concurrent.futures.ThreadPoolExecutor(max_workers=jobs or min(16, os.cpu_count() or 8)) as pool:
-            halo = pool.submit(_compile_halo_unit, hipcc, scratch)
-            objs = list(pool.map(lambda u: _compile_unit(hipcc, scratch, *u), units)) + [halo.result()]
+            extra = [pool.submit(_compile_halo_unit, hipcc, scratch), pool.submit(_compile_saxpy_unit, hipcc, scratch)]
+            extra += [pool.submit(_compile_sgemv_unit, hipcc, scratch, c) for c in SGEMV_CONFIGS]
+            extra.append(pool.submit(_compile_stencil_unit, hipcc, scratch))
+            objs = list(pool.map(lambda u: _compile_unit(hipcc, scratch, *u), units)) + [e.result() for e in extra]
         subprocess.check_call([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950"] + objs + ["-o", OUT])
     print(f"built {OUT}: {len(units)} units ({len(PROGRAMS)} programs, {len(PARAMETER_SETS)} parameter sets) + the halo "
-          f"test kernel in {len(HALO_INSTANCES)} instantiations")
+          f"test kernel in {len(HALO_INSTANCES)} instantiations + the {len(SAXPY_KERNELS)} saxpy kernels + "
+          f"the {len(SGEMV_CONFIGS)} sgemv configurations + the {len(STENCIL_HEADERS)} stencil kernels")
     return OUT
 
 

@@ -132,3 +132,94 @@ def test_reference_halo_test_kernel_matches_the_oracle(kernels, device, instance
                 assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
                 ran += 1
     assert ran >= 30
+
+@pytest.mark.parametrize("which", range(len(ref.SAXPY_KERNELS)), ids=ref.SAXPY_KERNELS)
+def test_reference_saxpy_kernels_match_the_oracle(kernels, device, which):
+    """The eight kernels of src/examples/saxpy/saxpy_cudaDMA_kernel.cu:54-420 (saxpy_cudaDMA and
+    saxpy_cudaDMA_doublebuffer stage x and y through cudaDMASequential objects) launched as saxpy_cudaDMA.cu:138 does,
+    on CTA_COUNT x NUM_ITERS x COMPUTE_THREADS_PER_CTA elements.  The reference accepts |host - device| <= 1e-6
+    (saxpy_cudaDMA.cu:167-178); here the result is compared bit for bit with one fused multiply-add per element,
+    which is what the device code does after contraction."""
+    p = ref.SAXPY
+    n = p["CTA_COUNT"] * p["NUM_ITERS"] * p["COMPUTE_THREADS_PER_CTA"]
+    x = ol.uniform(n, 11)
+    y0 = ol.uniform(n, 12)
+    a = np.float32(0.37)
+    want = y0.copy()
+    ol.load().oracle_saxpy(ctypes.c_float(float(a)), ptr(x), ptr(want), n)
+    fn = kernels.refk_saxpy
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p]
+    d_x = torch.from_numpy(x).to(device)
+    d_y = torch.from_numpy(y0).to(device)
+    d_timers = torch.zeros(1024, dtype=torch.int64, device=device)
+    print(f"saxpy kernel {ref.SAXPY_KERNELS[which]}", flush=True)
+    assert fn(which, ctypes.c_void_p(d_y.data_ptr()), ctypes.c_void_p(d_x.data_ptr()), ctypes.c_float(float(a)),
+              ctypes.c_void_p(d_timers.data_ptr()), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    torch.cuda.synchronize()
+    got = d_y.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), float(np.abs(got - want).max())
+
+@pytest.mark.parametrize("config", ref.SGEMV_CONFIGS)
+def test_reference_sgemv_kernels_match_their_own_expectation(kernels, device, config):
+    """The seven DMA kernels of src/examples/sgemv/sgemv_dma.cu:141-620 launched as its main() launches them (:845-856)
+    on the reference's own data (initialize_host, :735-749: A[j][i] = (i * j) % 11, x[i] = i % 11, alpha = 2), whose
+    products and sums are whole numbers below 2^24: the result is exact in any order of summation, and verify()
+    (:752-771) is restated with integers.  The matrix is 1024 x 1024 instead of 896 x 896 so that every
+    configuration's vector length divides it; the buffers carry a margin of zeros."""
+    n = m = ref.SGEMV_N
+    i = np.arange(n, dtype=np.int64)
+    j = np.arange(m, dtype=np.int64)
+    a_int = (j[:, None] * i[None, :]) % 11                              # matA[j * n + i]
+    x_int = j % 11
+    alpha = 2.0
+    want = (alpha * (a_int * x_int[:, None]).sum(axis=0)).astype(np.float32)
+    assert want.max() < 2 ** 24
+    margin = 64
+    d_a = torch.zeros((m + margin) * n, dtype=torch.float32, device=device)
+    d_a[:m * n] = torch.from_numpy(a_int.astype(np.float32).reshape(-1)).to(device)
+    d_x = torch.zeros(m + 2048, dtype=torch.float32, device=device)
+    d_x[:m] = torch.from_numpy(x_int.astype(np.float32)).to(device)
+    d_y = torch.full((n + 256,), float("nan"), dtype=torch.float32, device=device)
+    fn = getattr(kernels, f"refk_sgemv_{config}")
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    print(f"sgemv {config}", flush=True)
+    assert fn(n, m, ctypes.c_float(alpha), ctypes.c_void_p(d_a.data_ptr()), ctypes.c_void_p(d_x.data_ptr()),
+              ctypes.c_void_p(d_y.data_ptr()), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    torch.cuda.synchronize()
+    got = d_y.cpu().numpy()
+    assert np.array_equal(got[:n], want), int(np.argmax(got[:n] != want))
+    assert np.isnan(got[n:]).all()                                     # nothing written past the vector
+
+
+@pytest.mark.parametrize("which", range(len(ref.STENCIL_HEADERS)), ids=ref.STENCIL_HEADERS)
+@pytest.mark.parametrize("dims", [(32, 4, 2), (96, 20, 6), (960, 160, 8)], ids=lambda d: "x".join(map(str, d)))
+def test_reference_stencil_kernels_match_the_oracle(kernels, device, which, dims):
+    """The five kernels of src/examples/stencil/*_buffer.h launched as cudaDMA_stencil2D.cu:118-185 launches them
+    (grid DIM_X/TILE_X x DIM_Y/TILE_Y, TILE_X * TILE_Y compute threads plus one or two DMA groups, the offset and
+    strides of :94-97) on float2 cells in a (dimz + 2R, dimy + 2R, dimx + 2R) volume.  The reference checks nothing
+    here; the oracle's cross (arms of R - 1 cells, as stencil_math.h sums them) is compared bit for bit over the whole
+    destination, the cells no kernel may touch included."""
+    O = ol.load()
+    dimx, dimy, dimz = dims
+    r = ref.STENCIL["RADIUS"]
+    shape = (dimz + 2 * r, dimy + 2 * r, dimx + 2 * r, 2)
+    cells = int(np.prod(shape))
+    src = ol.uniform(cells, 31)
+    want = np.full(cells, -7.0, dtype=np.float32)
+    O.oracle_stencil2d(ptr(src), ptr(want), dimx, dimy, dimz, r, r - 1)
+    margin = 4 * shape[1] * shape[2] * 2                                # four planes beyond either buffer
+    d_src = torch.zeros(cells + margin, dtype=torch.float32, device=device)
+    d_src[:cells] = torch.from_numpy(src).to(device)
+    d_dst = torch.full((cells + margin,), -7.0, dtype=torch.float32, device=device)
+    fn = kernels.refk_stencil2d
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    print(f"stencil2d {ref.STENCIL_HEADERS[which]} {dims}", flush=True)
+    assert fn(which, ctypes.c_void_p(d_src.data_ptr()), ctypes.c_void_p(d_dst.data_ptr()), dimx, dimy, dimz,
+              ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    torch.cuda.synchronize()
+    got = d_dst.cpu().numpy()
+    assert np.array_equal(got[:cells].view(np.uint32), want.view(np.uint32)), int(np.argmax(got[:cells] != want))
+    assert (got[cells:] == -7.0).all()
