@@ -84,6 +84,18 @@ def test_sequential_copy_of_a_gibibyte(device, variant):
     assert np.array_equal(dst[:1 << 16].cpu().numpy().view(np.uint32), head.view(np.uint32))
 
 
+def test_sequential_copy_beyond_four_gibibytes(device):
+    """5 GiB: byte offsets past 2^32 on both sides (327 680 tiles)."""
+    m = 5 * (1 << 28)
+    pool = torch.empty(2 * m, dtype=torch.float32, device=device)
+    src = wl.fill_uniform(pool[:m], 1001)
+    dst = pool[m:]
+    dst.fill_(float("nan"))
+    wl.sequential_copy(src, dst)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.view(torch.int32), src.view(torch.int32))
+
+
 def test_sequential_copy_rejects_ragged_sizes(device):
     src = torch.zeros(5000, dtype=torch.float32, device=device)
     with pytest.raises(cd.CudaDMAError, match="multiple"):
@@ -179,6 +191,18 @@ def test_strided_transpose_full_size(device, variant):
     wl.strided_transpose(dst, back, variant)
     torch.cuda.synchronize()
     assert torch.equal(back.view(torch.int32), src.view(torch.int32))
+
+
+def test_strided_transpose_beyond_four_gibibytes(device):
+    """33 792 x 33 792 floats = 4.25 GiB per matrix: element offsets past 2^30, byte offsets past 2^32."""
+    n = 33792
+    src = wl.fill_uniform(torch.empty(n * n, dtype=torch.float32, device=device), 1002).view(n, n)
+    dst = torch.full((n, n), float("nan"), dtype=torch.float32, device=device)
+    wl.strided_transpose(src, dst)
+    torch.cuda.synchronize()
+    for r0 in range(0, n, 4096):                            # against the source read the other way, in bands
+        r1 = min(r0 + 4096, n)
+        assert torch.equal(dst[r0:r1].view(torch.int32), src[:, r0:r1].t().contiguous().view(torch.int32)), r0
 
 
 # ------------------------------------------------------------------ config 3
@@ -368,6 +392,28 @@ def test_halo_stencil_full_size(device, variant):
         got = d_out[z0:z0 + 3].cpu().numpy()
         assert np.all(np.abs(got - want) <= STENCIL_RTOL * np.maximum(np.abs(want), 1.0))
     # a constant field has zero Laplacian everywhere (catches a wrong tile or plane anywhere in the grid)
+    d_in.fill_(1.0)
+    wl.halo_stencil(d_in, d_out, variant)
+    torch.cuda.synchronize()
+    assert float(d_out.abs().max()) <= 1e-5
+
+
+@pytest.mark.parametrize("variant", [0, 6])
+def test_halo_stencil_beyond_four_gibibytes(device, variant):
+    """1024 x 1024 x 1032 cells: input and output each pass 2^32 bytes; the last planes against the host statement."""
+    nx = ny = 1024
+    nz = 1032
+    p = 2 * wl.STENCIL_RADIUS
+    d_in = wl.fill_uniform(torch.empty((nz + p) * (ny + p) * (nx + p), dtype=torch.float32, device=device), 1004).view(nz + p, ny + p, nx + p)
+    d_out = torch.full((nz, ny, nx), float("nan"), dtype=torch.float32, device=device)
+    wl.halo_stencil(d_in, d_out, variant)
+    torch.cuda.synchronize()
+    for z0 in (0, 517, nz - 3):
+        slab = np.ascontiguousarray(d_in[z0:z0 + 3 + p].cpu().numpy())
+        want = np.empty((3, ny, nx), dtype=np.float32)
+        ol.load().oracle_stencil25(ptr(slab), ptr(want), nx, ny, 3, wl.STENCIL_RADIUS)
+        got = d_out[z0:z0 + 3].cpu().numpy()
+        assert np.all(np.abs(got - want) <= STENCIL_RTOL * np.maximum(np.abs(want), 1.0)), z0
     d_in.fill_(1.0)
     wl.halo_stencil(d_in, d_out, variant)
     torch.cuda.synchronize()
