@@ -12,6 +12,7 @@ one compute wavefront of 64 threads plus DMA_THREADS DMA threads; dynamic LDS of
                                                               cudaDMASequential), launch saxpy_cudaDMA.cu:138
     src/examples/stencil/*_buffer.h + stencil_math.h          the five buffering styles of the 2-D stencil on
                                                               CudaDMAStrided, launch cudaDMA_stencil2D.cu:118-185
+    src/perf/sequential/perf_sequential.cu                    the four kernel shapes of the read-bandwidth probe
     src/examples/sgemv/sgemv_dma.cu                           its seven DMA kernels :141-620 (cudaDMASequential for the
                                                               vector, cudaDMAStrided for the matrix panel), each under
                                                               its own -D switch with its own sizes :79-133, launch :845-856
@@ -280,6 +281,47 @@ extern "C" int refk_stencil2d(int which, const void* d_src, void* d_dst, int dim
     return obj
 
 
+# read-bandwidth probe: the directed parameters of src/perf/sequential/params_directed.h (float, ALIGNMENT 16, elements
+# of 4096 bytes, 32 loops), two DMA wavefronts of 64 in place of two warps, one compute wavefront
+PERF_KERNELS = ["non_specialized", "single_buffer", "double_buffer", "manual_buffer"]
+PERF = dict(ALIGNMENT=16, ELMT_SIZE=4096, DMA_THREADS=128, LOOP_ITERS=32, COMPUTE_THREADS=64)
+
+
+def _compile_perf_unit(hipcc, scratch):
+    text = open("/root/reference/src/perf/sequential/perf_sequential.cu").read()
+    start = text.index("template<typename T, int ALIGNMENT, int BYTES_PER_ELMT, int TOTAL_THREADS, int NUM_LOOPS>")
+    end = _END_OF_FUNCTION.search(text, text.index("void manual_buffer")).end()
+    t = PERF
+    args = f"float, {t['ALIGNMENT']}, {t['ELMT_SIZE']}, {t['DMA_THREADS']}, {t['LOOP_ITERS']}"
+    # threads per workgroup as performance_test() counts them (perf_sequential.cu:229-241): the DMA groups alone when not
+    # specialised, plus one compute group, plus a second set of DMA groups when double-buffered
+    launcher = f'''
+extern "C" int refk_perf_sequential(int which, const float* d_src, float* d_dst, int ctas, int always_false, void* stream)
+{{
+  hipStream_t s = (hipStream_t)stream;
+  const int dma = {t['DMA_THREADS']}, compute = {t['COMPUTE_THREADS']};
+  switch (which) {{
+    case 0: hipLaunchKernelGGL((non_specialized<{args}>), dim3(ctas), dim3(dma), 0, s, d_src, d_dst, always_false != 0); break;
+    case 1: hipLaunchKernelGGL((single_buffer<{args}>), dim3(ctas), dim3(dma + compute), 0, s, d_src, d_dst, compute, always_false != 0); break;
+    case 2: hipLaunchKernelGGL((double_buffer<{args}>), dim3(ctas), dim3(2 * dma + compute), 0, s, d_src, d_dst, compute, always_false != 0); break;
+    case 3: hipLaunchKernelGGL((manual_buffer<{args}>), dim3(ctas), dim3(dma + compute), 0, s, d_src, d_dst, compute, always_false != 0); break;
+    default: return -1;
+  }}
+  return hipGetLastError() == hipSuccess ? 0 : -2;
+}}
+'''
+    source = '#include <hip/hip_runtime.h>\n#include "cudaDMA.h"\nnamespace {\n' + text[start:end] + "\n}\n" + launcher
+    src, obj = os.path.join(scratch, "perf.hip"), os.path.join(scratch, "perf.o")
+    with open(src, "w") as f:
+        f.write(source)
+    cmd = [hipcc, "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-I", os.path.join(ROOT, "include"), "-c", src, "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("perf_sequential:\n" + "\n".join(l for l in res.stderr.splitlines() if "error" in l)[:3000])
+    return obj
+
+
 def _compile_halo_unit(hipcc, scratch):
     text = open(os.path.join(REFERENCE_TESTS, "test_halo/cudaDMA_test_halo.cu")).read()
     start = text.index("template<typename TYPE>")                    # initialize<> / get_val<> come before the kernel
@@ -344,11 +386,12 @@ def build(jobs=None):
             extra = [pool.submit(_compile_halo_unit, hipcc, scratch), pool.submit(_compile_saxpy_unit, hipcc, scratch)]
             extra += [pool.submit(_compile_sgemv_unit, hipcc, scratch, c) for c in SGEMV_CONFIGS]
             extra.append(pool.submit(_compile_stencil_unit, hipcc, scratch))
+            extra.append(pool.submit(_compile_perf_unit, hipcc, scratch))
             objs = list(pool.map(lambda u: _compile_unit(hipcc, scratch, *u), units)) + [e.result() for e in extra]
         subprocess.check_call([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950"] + objs + ["-o", OUT])
     print(f"built {OUT}: {len(units)} units ({len(PROGRAMS)} programs, {len(PARAMETER_SETS)} parameter sets) + the halo "
           f"test kernel in {len(HALO_INSTANCES)} instantiations + the {len(SAXPY_KERNELS)} saxpy kernels + "
-          f"the {len(SGEMV_CONFIGS)} sgemv configurations + the {len(STENCIL_HEADERS)} stencil kernels")
+          f"the {len(SGEMV_CONFIGS)} sgemv configurations + the {len(STENCIL_HEADERS)} stencil kernels + the {len(PERF_KERNELS)} probe kernels")
     return OUT
 
 

@@ -223,3 +223,35 @@ def test_reference_stencil_kernels_match_the_oracle(kernels, device, which, dims
     got = d_dst.cpu().numpy()
     assert np.array_equal(got[:cells].view(np.uint32), want.view(np.uint32)), int(np.argmax(got[:cells] != want))
     assert (got[cells:] == -7.0).all()
+
+
+@pytest.mark.parametrize("which", range(len(ref.PERF_KERNELS)), ids=ref.PERF_KERNELS)
+def test_reference_probe_kernels_move_what_they_should(kernels, device, which):
+    """The four kernel shapes of src/perf/sequential/perf_sequential.cu:52-224 (not specialised; single, double and manual
+    buffering on cudaDMASequential) launched as its performance_test() launches them (:229-241, :311-345).  The probe
+    only times them: its `always_false` argument keeps the buffers from being read.  Here they also run with the
+    argument true, which makes every compute thread add its word of each of the 32 buffers to the output
+    (out[first + t] += buffer[t], :67-70), a sum that pins which bytes reached the LDS buffer in which loop."""
+    t = ref.PERF
+    ctas, loops, per = 96, t["LOOP_ITERS"], t["ELMT_SIZE"] // 4
+    readers = t["DMA_THREADS"] if which == 0 else t["COMPUTE_THREADS"]       # threads that reach the addition
+    rng = np.random.default_rng(12 + which)
+    src = rng.integers(0, 10, size=ctas * loops * per).astype(np.float32)
+    want = np.full(src.size, -3.0, dtype=np.float32)
+    for i in range(loops):                                                    # float32 additions in the kernel's order
+        want.reshape(ctas, loops * per)[:, :readers] += src.reshape(ctas, loops, per)[:, i, :readers]
+    d_src = torch.from_numpy(src).to(device)
+    fn = kernels.refk_perf_sequential
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    for always_false in (0, 1):
+        d_dst = torch.full((src.size,), -3.0, dtype=torch.float32, device=device)
+        print(f"perf_sequential {ref.PERF_KERNELS[which]} always_false={always_false}", flush=True)
+        assert fn(which, ctypes.c_void_p(d_src.data_ptr()), ctypes.c_void_p(d_dst.data_ptr()), ctas, always_false,
+                  ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+        torch.cuda.synchronize()
+        got = d_dst.cpu().numpy()
+        if always_false:
+            assert np.array_equal(got, want), int(np.argmax(got != want))
+        else:
+            assert (got == -3.0).all()                                        # as timed: nothing is written
