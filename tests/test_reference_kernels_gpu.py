@@ -1,11 +1,12 @@
-"""The reference's own test kernels on the GPU.  oracle/build_ref_kernels.py compiles the special_xfer_* / nonspec_xfer_*
-kernels of the reference's v2 test programs (src/tests/test_{sequential,strided,indirect}/cudaDMA_test_*_v2.cu) from the
-reference tree against this repository's cudaDMAv2.h into oracle/_ref/libref_kernels.so (not kept in the repository;
-it travels with the built libraries).  Here they run as the reference's run_experiment() runs them: input float(i)
+"""The reference's own device kernels on the GPU.  oracle/build_ref_kernels.py compiles them from the reference tree against
+this repository's cudaDMAv2.h / cudaDMA.h into oracle/_ref/libref_kernels.so (not kept in the repository; it travels with
+the built libraries): the special_xfer_* / nonspec_xfer_* kernels of the v2 test programs
+(src/tests/test_{sequential,strided,indirect}/cudaDMA_test_*_v2.cu), the halo test kernel, the saxpy, sgemv and stencil
+examples and the read-bandwidth probe.  The test kernels run as the reference's run_experiment() runs them: input float(i)
 (cudaDMA_test_sequential_v2.cu:416-418), one workgroup, the LDS buffer zeroed by the compute threads, filled by the DMA
 threads, copied out; every kernel in its one-phase and two-phase form, with and without the cache qualifiers the kernel
 text names.  The output is compared with the oracle's closed form over the whole buffer (the reference compares the
-moved elements only, :501-512), bit for bit."""
+moved elements only, :501-512), bit for bit.  The examples and the probe run as their own main()s launch them."""
 import ctypes
 import os
 
