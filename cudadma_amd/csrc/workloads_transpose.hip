@@ -8,6 +8,7 @@
 // 17*L + j, so eight consecutive lanes hit eight different units modulo 8 and no
 // banks collide.  The tile column c then leaves as one global_store_dword per
 // wavefront: 64 lanes x 4 B = 256 contiguous bytes of output row c.
+#include <utility>
 #include "workloads.hpp"
 
 namespace {
@@ -422,10 +423,91 @@ transpose_split(const float* __restrict__ in, float* __restrict__ out, const int
   }
 }
 
+// N copies of an object without a default constructor
+template<typename T, int N> struct Copies { T v[N]; };
+template<typename T, int... I>
+__device__ __forceinline__ Copies<T, (int)sizeof...(I)> copies_of(const T& x, std::integer_sequence<int, I...>)
+{ return Copies<T, (int)sizeof...(I)>{{((void)I, x)...}}; }
+
+// transpose_split with the tile requested in K pieces of 64 / K rows, M pieces in flight: between whole numbers of
+// tiles ahead (M / K = 1.25, 1.5, 1.75 tiles outstanding per workgroup).  One CudaDMAStrided object per piece in
+// flight, all on the same DMA wavefronts (manual buffering, src/examples/stencil/warp_specialized_manual_buffer.h:54-71);
+// the LDS tile is handed over whole: the guard is taken before the first piece of a tile lands and released after
+// the last.  The compute side is that of transpose_split.
+template<int DW, int CW, int K, int M>
+__global__ void __launch_bounds__((DW + CW) * 64)
+transpose_pieces(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles, const int band)
+{
+  static_assert(CW == 1 || CW == 2 || CW == 4, "the compute wavefronts share the sixteen 16-byte columns of a tile row evenly");
+  static_assert(kTile % K == 0 && 2 * M >= K && M <= 2 * K, "between half a tile and two tiles in flight");
+  constexpr int kLdsRow = 272;
+  constexpr int kDma = DW * 64, kCompute = CW * 64;
+  constexpr int kRows = kTile / K;
+  constexpr int kChunks = kRows * kRowBytes / 16;
+  constexpr int kBpt = ((kChunks + kDma - 1) / kDma) * 16;
+  __shared__ __attribute__((aligned(16))) char buf[kTile * kLdsRow];
+  cudaDMACustom guard(0, kDma, kCompute, kCompute);
+  typedef CudaDMAStrided<false, 16, kBpt, kRowBytes, kDma, kRows> obj_t;
+  const int tiles_per_side = n / kTile;
+  const int stride = gridDim.x;
+  const int last = num_tiles - 1;
+  if (guard.owns_this_thread()) {
+    // piece q of this workgroup: part q % K of its tile number q / K; past the end the last tile again, so that the
+    // loads stay unconditional
+    auto src_of = [&](const int q) {
+      const int t = blockIdx.x + (q / K) * stride;
+      int ty, tx;
+      tile_coords(t < num_tiles ? t : last, tiles_per_side, band, ty, tx);
+      return (const void*)(in + ((size_t)ty * kTile + (size_t)((q % K) * kRows)) * n + (size_t)tx * kTile);
+    };
+    if ((int)blockIdx.x >= num_tiles) return;
+    Copies<obj_t, M> objs = copies_of(obj_t(n * 4, kLdsRow, kCompute), std::make_integer_sequence<int, M>());
+    obj_t* o = objs.v;
+#pragma unroll
+    for (int i = 0; i < M; ++i) o[i].template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(i));
+    const int pieces = ((num_tiles - 1 - (int)blockIdx.x) / stride + 1) * K;
+    // K * M pieces per turn: object and part of every step are then compile-time constants
+    for (int q0 = 0; q0 < pieces; q0 += K * M) {
+#pragma unroll
+      for (int i = 0; i < K * M; ++i) {
+        if (q0 + i < pieces) {
+          if (i % K == 0) guard.wait_for_dma_start();
+          o[i % M].template wait_xfer_finish<true, LOAD_CACHE_STREAMING, STORE_LDS>(buf + (i % K) * kRows * kLdsRow);
+          if (i % K == K - 1) guard.finish_async_dma();
+        }
+        o[i % M].template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(q0 + i + M));
+      }
+    }
+  } else {
+    constexpr int kUnits = 16 / CW;
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6;
+    guard.start_async_dma();
+    for (int t = blockIdx.x; t < num_tiles; t += stride) {
+      int ty, tx;
+      tile_coords(t, tiles_per_side, band, ty, tx);
+      guard.wait_for_dma_finish();
+      vec4_t v[kUnits];
+      const vec4_t* row = (const vec4_t*)(buf + lane * kLdsRow) + w * kUnits;
+#pragma unroll
+      for (int j = 0; j < kUnits; ++j) v[j] = row[j];
+      guard.start_async_dma();
+      float* o = out + (size_t)(tx * kTile + w * 4 * kUnits + (lane & 3)) * n + (size_t)ty * kTile + (lane & ~3);
+#pragma unroll
+      for (int j = 0; j < kUnits; ++j)
+        __builtin_nontemporal_store(quad_transpose(v[j], lane), (vec4_t*)(o + (size_t)(4 * j) * n));
+    }
+  }
+}
+
 typedef void (*split_kernel_t)(const float*, float*, int, int, int);
 struct SplitEntry { int dw, cw, ahead; split_kernel_t kernel; };
 #define SPLIT(DW, CW) {DW, CW, 1, transpose_split<DW, CW, 1>}, {DW, CW, 2, transpose_split<DW, CW, 2>}
-const SplitEntry kSplits[] = {SPLIT(2, 2), SPLIT(1, 1), SPLIT(1, 2), SPLIT(2, 1), SPLIT(3, 1), SPLIT(4, 1), SPLIT(3, 2), SPLIT(4, 2),
+// "tiles ahead" 3 .. 7 stand for a tile requested in pieces (the fastest split only): 3 = 3 halves in flight (1.5 tiles),
+// 4 = 5 quarters (1.25), 5 = 6 quarters (1.5), 6 = 7 quarters (1.75), 7 = 3 quarters (0.75)
+const SplitEntry kSplits[] = {{3, 1, 3, transpose_pieces<3, 1, 2, 3>}, {3, 1, 4, transpose_pieces<3, 1, 4, 5>},
+                              {3, 1, 5, transpose_pieces<3, 1, 4, 6>}, {3, 1, 6, transpose_pieces<3, 1, 4, 7>},
+                              {3, 1, 7, transpose_pieces<3, 1, 4, 3>}, SPLIT(2, 2), SPLIT(1, 1), SPLIT(1, 2), SPLIT(2, 1), SPLIT(3, 1), SPLIT(4, 1), SPLIT(3, 2), SPLIT(4, 2),
                               SPLIT(1, 4), SPLIT(2, 4), SPLIT(4, 4)};
 #undef SPLIT
 

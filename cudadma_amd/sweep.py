@@ -7,6 +7,7 @@ point; here the variants are compiled in and the occupancy is a run-time knob.
     python -m cudadma_amd.sweep saxpy sgemv stencil2d        # the reference's example programs, every variant
     python -m cudadma_amd.sweep perf_sequential --wg 2,8     # read-bandwidth probe: element size x DMA wavefronts x buffering
     python -m cudadma_amd.sweep transpose_split              # DMA : compute wavefronts x tiles ahead x workgroups per CU
+    python -m cudadma_amd.sweep transpose_walk               # tile order x workgroup count, one-tile and two-tile kernels
     python -m cudadma_amd.sweep placement                    # 1 GiB copies against the distance between source and destination
 """
 import argparse
@@ -123,10 +124,33 @@ def main(argv=None):
                     ms = _time(lambda: wl.strided_transpose(src, dst, wl.TRANSPOSE_SPLIT_VARIANT), args.steps, settle_ms=15.0)
                     cells.append(f"{ms:.4f} ({2 * n * n * 4 / ms / 1e6 / PEAK_GBS * 100:4.1f}%)")
                 wl.set_tuning("transpose_workgroups", 0)
-                print(f"{code // 100} + {code // 10 % 10}, {code % 10} ahead:  " + "   ".join(cells) + ("" if exact else "   WRONG RESULT"),
+                ahead = {3: "1.5 (3 halves)", 4: "1.25 (5 quarters)", 5: "1.5 (6 quarters)", 6: "1.75 (7 quarters)",
+                         7: "0.75 (3 quarters)"}.get(code % 10, str(code % 10))
+                print(f"{code // 100} + {code // 10 % 10}, {ahead} ahead:  " + "   ".join(cells) + ("" if exact else "   WRONG RESULT"),
                       flush=True)
             wl.set_tuning("transpose_split", 0)
             del ref
+        elif name == "transpose_walk":
+            # the order in which the tiles are taken (bands of `band` tile rows; a band as high as the matrix walks down
+            # the columns, so every workgroup stays on its own 64 matrix rows) against the number of workgroups, for the
+            # kernels with one tile per workgroup in flight (variants 0, 1) and with two (variants 11, 3, 5)
+            n = 16384
+            src = wl.fill_uniform(torch.empty(n * n, device=dev), 1002).view(n, n)
+            dst = torch.empty_like(src)
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            counts = (cus // 2, cus * 3 // 4, cus - 8, cus, cus + 8, cus * 2, cus * 4)
+            print("# variant, band: % of 8 TB/s with " + " / ".join(str(c) for c in counts) + " workgroups")
+            for variant in (0, 1, wl.TRANSPOSE_TWO_LDS_TILES_VARIANT, 3, 5):
+                for band in (256, 64, 16, 4, 1):
+                    wl.set_tuning("transpose_band", band)
+                    cells = []
+                    for count in counts:
+                        wl.set_tuning("transpose_workgroups", count)
+                        ms = _time(lambda: wl.strided_transpose(src, dst, variant), args.steps, settle_ms=10.0)
+                        cells.append(f"{2 * n * n * 4 / ms / 1e6 / PEAK_GBS * 100:4.1f}")
+                    print(f"variant {variant:2d}  band {band:3d}:  " + "  ".join(cells), flush=True)
+            wl.set_tuning("transpose_band", 0)
+            wl.set_tuning("transpose_workgroups", 0)
         elif name == "placement":
             # linear copies of 1 GiB inside one allocation, against the distance from source to destination;
             # the transposition of the same bytes beside them
