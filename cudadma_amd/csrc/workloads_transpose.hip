@@ -365,7 +365,7 @@ __global__ void __launch_bounds__((DW + CW) * 64)
 transpose_split(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles, const int band)
 {
   static_assert(CW == 1 || CW == 2 || CW == 4, "the compute wavefronts share the sixteen 16-byte columns of a tile row evenly");
-  static_assert(AHEAD == 1 || AHEAD == 2, "one or two tiles requested ahead");
+  static_assert(AHEAD >= 1 && AHEAD <= 3, "one or two tiles requested ahead, or (3) one in flight with two register sets");
   constexpr int kLdsRow = 272;
   constexpr int kDma = DW * 64, kCompute = CW * 64;
   constexpr int kChunks = kTile * kRowBytes / 16;
@@ -391,6 +391,26 @@ transpose_split(const float* __restrict__ in, float* __restrict__ out, const int
     int t = blockIdx.x;
     if (t >= num_tiles) return;
     a.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t));
+    if constexpr (AHEAD == 3) {
+      // two register sets but one tile in flight: the next tile is requested as soon as the loads of the current one
+      // have returned, before it is stored to LDS, so that the store and the handshake leave the round trip
+      auto returned = [&]() __attribute__((always_inline)) {
+        asm volatile("" ::: "memory");
+        hipdma::detail::wait_lds_direct();                 // s_waitcnt vmcnt(0)
+        asm volatile("" ::: "memory");
+      };
+      for (; t < num_tiles; t += 2 * stride) {
+        returned();
+        b.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t + stride));
+        land(a);
+        if (t + stride < num_tiles) {
+          returned();
+          a.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t + 2 * stride));
+          land(b);
+        }
+      }
+      return;
+    }
     if constexpr (AHEAD == 2) b.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t + stride));
     for (; t < num_tiles; t += AHEAD * stride) {
       land(a);
@@ -507,7 +527,9 @@ struct SplitEntry { int dw, cw, ahead; split_kernel_t kernel; };
 // 4 = 5 quarters (1.25), 5 = 6 quarters (1.5), 6 = 7 quarters (1.75), 7 = 3 quarters (0.75)
 const SplitEntry kSplits[] = {{3, 1, 3, transpose_pieces<3, 1, 2, 3>}, {3, 1, 4, transpose_pieces<3, 1, 4, 5>},
                               {3, 1, 5, transpose_pieces<3, 1, 4, 6>}, {3, 1, 6, transpose_pieces<3, 1, 4, 7>},
-                              {3, 1, 7, transpose_pieces<3, 1, 4, 3>}, SPLIT(2, 2), SPLIT(1, 1), SPLIT(1, 2), SPLIT(2, 1), SPLIT(3, 1), SPLIT(4, 1), SPLIT(3, 2), SPLIT(4, 2),
+                              {3, 1, 7, transpose_pieces<3, 1, 4, 3>},
+                              // 8 = two register sets, one tile in flight without a pause
+                              {3, 1, 8, transpose_split<3, 1, 3>}, {2, 2, 8, transpose_split<2, 2, 3>}, SPLIT(2, 2), SPLIT(1, 1), SPLIT(1, 2), SPLIT(2, 1), SPLIT(3, 1), SPLIT(4, 1), SPLIT(3, 2), SPLIT(4, 2),
                               SPLIT(1, 4), SPLIT(2, 4), SPLIT(4, 4)};
 #undef SPLIT
 

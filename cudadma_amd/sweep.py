@@ -125,7 +125,7 @@ def main(argv=None):
                     cells.append(f"{ms:.4f} ({2 * n * n * 4 / ms / 1e6 / PEAK_GBS * 100:4.1f}%)")
                 wl.set_tuning("transpose_workgroups", 0)
                 ahead = {3: "1.5 (3 halves)", 4: "1.25 (5 quarters)", 5: "1.5 (6 quarters)", 6: "1.75 (7 quarters)",
-                         7: "0.75 (3 quarters)"}.get(code % 10, str(code % 10))
+                         7: "0.75 (3 quarters)", 8: "1, requested on return,"}.get(code % 10, str(code % 10))
                 print(f"{code // 100} + {code // 10 % 10}, {ahead} ahead:  " + "   ".join(cells) + ("" if exact else "   WRONG RESULT"),
                       flush=True)
             wl.set_tuning("transpose_split", 0)

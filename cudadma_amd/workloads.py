@@ -16,9 +16,10 @@ STENCIL_RADIUS = 4
 TRANSPOSE_SPLIT_VARIANT = 10           # cudadma_strided_transpose variant whose wavefront split follows the knob "transpose_split"
 # knob values = 100 x DMA wavefronts + 10 x compute wavefronts + tiles ahead, every compiled combination; with three DMA
 # wavefronts and one compute wavefront "tiles ahead" 3 to 7 stand for a tile requested in pieces: 3 halves (1.5 tiles), 5, 6
-# and 7 quarters (1.25, 1.5, 1.75 tiles) and 3 quarters (0.75) in flight
+# and 7 quarters (1.25, 1.5, 1.75 tiles) and 3 quarters (0.75) in flight; 8 (also with 2 + 2) for one tile in flight
+# without a pause: the next tile is requested when the loads of the current one have returned, before it goes to LDS
 TRANSPOSE_SPLITS = (111, 112, 121, 122, 141, 142, 211, 212, 221, 222, 241, 242, 311, 312, 321, 322, 411, 412, 421, 422, 441, 442,
-                    313, 314, 315, 316, 317)
+                    313, 314, 315, 316, 317, 228, 318)
 TRANSPOSE_TWO_LDS_TILES_VARIANT = 11    # two LDS tiles and two CudaDMAStrided objects (manual double buffering in LDS)
 HALO_WIDE_TILES_VARIANT = 6            # cudadma_halo_stencil variant 0 with tiles of 64 x 16 cells
 GEMM_WARP_SPECIALISED_VARIANT = 7      # the cudadma_gemm_bf16 variant in which DMA wavefronts feed compute wavefronts

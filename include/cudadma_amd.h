@@ -234,7 +234,8 @@ int cudadma_set_workgroups_per_cu(int value);
  *   "transpose_workgroups"  workgroups to launch for config 2, whatever the per-CU knob says
  *   "transpose_split"  config 2, variant 10: 100 x DMA wavefronts + 10 x compute wavefronts + tiles requested ahead
  *                      (1 or 2; with 3 + 1 wavefronts also 3 .. 7: the tile requested in halves or quarters, 1.5, 1.25, 1.5,
- *                      1.75 and 0.75 tiles in flight)
+ *                      1.75 and 0.75 tiles in flight; 8, also with 2 + 2: the next tile requested as soon as the loads of
+ *                      the current one have returned)
  *   "stencil_zchunk"     output planes one workgroup marches through in config 4
  *   "stencil_xcd_remap"  config 4 numbers its workgroups so that each XCD gets a slab of the grid over its whole width;
  *                        4 asks for compact blocks of the tile grid instead (2 x 4 blocks), 2 turns the numbering off
