@@ -74,7 +74,9 @@ static const VariantInfo kStrided[] = {
   {"as variant 8 with the quad transposition and dwordx4 stores of variant 7"},
   {"variant 1 with the split of the workgroup as a knob (\"transpose_split\" = 100 x DMA wavefronts + 10 x compute "
    "wavefronts + tiles requested ahead; default 311: three DMA wavefronts, one compute wavefront, one tile ahead, "
-   "the fastest of the 22 splits compiled): one LDS tile guarded by a sync-only object, one or two CudaDMAStrided "
+   "the fastest of the 22 splits compiled; with 3 + 1 wavefronts the last digit 3 to 7 asks for the tile in halves "
+   "or quarters, 0.75 to 1.75 tiles in flight, and 8 for the next tile requested as soon as the loads of the current "
+   "one have returned): one LDS tile guarded by a sync-only object, one or two CudaDMAStrided "
    "objects without a handshake of their own on the DMA wavefronts; the kernel the benchmark reports"},
   {"manual double buffer in LDS: one DMA group of 2 wavefronts, two CudaDMAStrided objects and two LDS tiles with padded "
    "rows (272 B), four workgroups per compute unit"},
