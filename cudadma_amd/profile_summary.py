@@ -12,7 +12,7 @@ Expected layout, one directory per pattern of bench.py (`--only <pattern>`), one
 FETCH_SIZE and WRITE_SIZE (KiB per dispatch) are scaled by what the same counters read, in the same run, for
 the library's plain copy of 1 GiB (`plain_copy_kernel`: 1 048 576 KiB read and as many written).
 
-    python -m cudadma_amd.profile_summary gpurun_out/prof > /tmp/table.md      # writes profiles/counters.json
+    python -m cudadma_amd.profile_summary <root> > table.md      # writes profiles/counters.json
 """
 import csv
 import glob
