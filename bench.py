@@ -11,9 +11,14 @@ under "patterns" / "gemm".  The sequential copy and the gather are each reported
 configuration names (64 MiB buffer, 512 MiB table: both working sets are helped by the 256 MB Infinity Cache)
 and at a size that is not (1 GiB buffer, 4 GiB table).  "yardsticks" holds what read-only, write-only and
 copy-shaped streams and the vendor's own device-to-device copy reach on the same 1 GiB buffers in the same
-run; roofline.ceiling is the best read + write yardstick of the run.  Counter-derived fields (HBM traffic per
-launch, matrix-core occupancy) come from profiles/counters.json, which `python -m cudadma_amd.profile_summary`
-writes from rocprofv3 output.  One JSON line goes to stdout; progress goes to stderr.
+run; roofline.ceiling is the best read + write yardstick of the run.  Every row of "patterns" also carries a
+"ceiling" of its own: what a kernel without LDS and without a DMA object reaches in the same run on the same buffers with
+the pattern's own addresses (the gather's index list, the scatter's permutation, a plain copy for the sequential and
+strided patterns and, scaled by the stencil's measured traffic, for the halo), and "settle_ms": the wall time of untimed
+launches in front of the timed ones.  The headline row "strided" is timed exactly as the command line says (--warmup
+launches, then --steps timed ones); "strided_settled" is the same kernel under the policy of the other rows.
+Counter-derived fields (HBM traffic per launch, matrix-core occupancy) come from profiles/counters.json, which
+`python -m cudadma_amd.profile_summary` writes from rocprofv3 output.  One JSON line goes to stdout; progress goes to stderr.
 """
 import argparse
 import json
@@ -34,6 +39,8 @@ COUNTERS_JSON = os.path.join(ROOT, "profiles", "counters.json")
 # name -> (kernel the pattern launches, as rocprofv3 names it; used by cudadma_amd.profile_summary)
 PATTERN_KERNELS = {
     "strided": "transpose_split<3, 1, 1>",
+    "strided_settled": "transpose_split<3, 1, 1>",
+    "sequential_read_probe": "perf_manual<2, 4>",
     "strided_even_split": "transpose_single<true, true>",
     "strided_two_lds_tiles": "transpose_manual_double<272, false>",
     "sequential": "copy_manual_double<4>",
@@ -159,6 +166,21 @@ def cpu_baselines(budget_s=15.0):
     out["halo"] = {"GB/s": round(2.0 * g ** 3 * 4 / med / 1e9, 2),
                    "sample": f"oracle_stencil25 on the full {g}^3 float32 grid, median of {reps}"}
 
+    del grid, res
+
+    dim, rows = 4096, 1024                           # config 5, a quarter of the rows of C (the loop nest is the same for every row)
+    ga = np.empty(rows * dim, dtype=np.uint16)
+    gb = np.empty(dim * dim, dtype=np.uint16)
+    gc = np.empty(rows * dim, dtype=np.float32)
+    O.oracle_fill_normal_bf16(ptr(ga), ga.size, 1005)
+    O.oracle_fill_normal_bf16(ptr(gb), gb.size, 2005)
+    t0 = time.perf_counter()
+    O.oracle_gemm_bf16(ptr(ga), ptr(gb), ptr(gc), rows, dim, dim)
+    dt = time.perf_counter() - t0
+    out["gemm"] = {"TFLOP/s": round(2.0 * rows * dim * dim / dt / 1e12, 4),
+                   "sample": f"oracle_gemm_bf16 (fp32 products of the bf16 inputs, ascending k) on the first {rows} of the {dim} rows of C "
+                             f"of the {dim}^3 problem, one repetition of {dt:.1f} s"}
+
     head = {"value": out["strided"]["GB/s"], "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": "OpenMP " + out["strided"]["sample"]}
     return head, out
@@ -193,15 +215,25 @@ def main():
     patterns, yardsticks = {}, {}
     cus = torch.cuda.get_device_properties(0).multi_processor_count
 
-    def report(table, name, ms, nbytes, note, bound="hbm"):
+    def report(table, name, ms, nbytes, note, bound="hbm", settle_ms=SETTLE_MS, launches=None):
         gbs = nbytes / ms / 1e6
         row = {"GB/s": round(gbs, 1), "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4), "ms": round(ms, 4),
-               "algorithmic_bytes": nbytes, "bound": bound, "workload": note}
+               "algorithmic_bytes": nbytes, "bound": bound, "settle_ms": settle_ms,
+               "timed_launches": launches if launches is not None else steps, "workload": note}
         if table is patterns:
             row["kernel"] = PATTERN_KERNELS.get(name)
             row["traffic_bytes_from_counters"] = traffic(name)
         table[name] = row
         log(f"{name:24s} {ms:9.4f} ms  {gbs:8.1f} GB/s  {100 * gbs / HBM_PEAK_GBS:5.1f}% of peak   {note}")
+
+    def best_shape(launch, choices, nbytes, label, note):
+        """The fastest of a few launch shapes of a yardstick; launch(choice) returns the function to time."""
+        best = None
+        for choice in choices:
+            ms, _ = time_launches(launch(choice), max(10, steps // 2), 5, 10.0)
+            if best is None or ms < best[0]:
+                best = (ms, choice)
+        report(yardsticks, label, best[0], nbytes, note.format(best=best[1], tried=len(choices)), settle_ms=10.0, launches=max(10, steps // 2))
 
     # ---- config 2: strided tile transpose (headline) ----
     # One allocation holds the source and, exactly 1 GiB behind it, the destination of every 1 GiB + 1 GiB stream of
@@ -214,10 +246,14 @@ def main():
     dst = pool[n * n:].view(n, n)
     strided_ms, strided_wall_ms = time_launches(lambda: wl.strided_transpose(src, dst, STRIDED_VARIANT), steps, warmup)
     strided_bytes = 2 * n * n * 4
-    report(patterns, "strided", strided_ms, strided_bytes,
-           "CudaDMAStrided 64x256B tiles of a 16384^2 f32 matrix, transposed out: one LDS tile, the next tile in the DMA "
-           "wavefronts' registers (the double buffer is LDS + registers), one workgroup of three DMA wavefronts and one "
-           "compute wavefront per compute unit")
+    strided_note = ("CudaDMAStrided 64x256B tiles of a 16384^2 f32 matrix, transposed out: one LDS tile, the next tile in the DMA "
+                    "wavefronts' registers (the double buffer is LDS + registers), one workgroup of three DMA wavefronts and one "
+                    "compute wavefront per compute unit")
+    report(patterns, "strided", strided_ms, strided_bytes, strided_note + f"; timed as the command line says: {warmup} untimed launches, "
+           f"then {steps} timed ones", settle_ms=0.0)
+    if want("strided_settled"):
+        ms, _ = time_launches(lambda: wl.strided_transpose(src, dst, STRIDED_VARIANT), steps, warmup, SETTLE_MS)
+        report(patterns, "strided_settled", ms, strided_bytes, "the kernel of the strided row under the policy of the rows below")
     if want("strided_even_split"):
         ms, _ = time_launches(lambda: wl.strided_transpose(src, dst, 1), steps, warmup, SETTLE_MS)
         report(patterns, "strided_even_split", ms, strided_bytes, "the same kernel shape with two DMA and two compute wavefronts (128 + 128 threads)")
@@ -236,19 +272,25 @@ def main():
         ms, _ = time_launches(lambda: wl.probe_memory("vendor_copy", flat_src, flat_dst, 1), steps, warmup, SETTLE_MS)
         report(yardsticks, "vendor_copy", ms, strided_bytes, "hipMemcpyDtoDAsync of 1 GiB")
 
-        def best_shape(modes, s_, d_, shapes, nbytes, label):
-            best = None
-            for mode in modes:
-                for wg in shapes:
-                    ms, _ = time_launches(lambda: wl.probe_memory(mode, s_, d_, int(cus * wg)), max(10, steps // 2), 5, 10.0)
-                    if best is None or ms < best[0]:
-                        best = (ms, wg, mode)
-            report(yardsticks, label, best[0], nbytes,
-                   f"{best[2]} stream over 1 GiB, grid-stride dwordx4, best of {len(modes) * len(shapes)} (cache hint, launch shape) "
-                   f"pairs: {best[1]} workgroups per compute unit")
-        best_shape(("read", "read_nontemporal"), flat_src, None, (1, 1.5, 2, 3, 4), strided_bytes // 2, "read_only")
-        best_shape(("write", "write_nontemporal"), None, flat_dst, (0.5, 1, 2, 4), strided_bytes // 2, "write_only")
-        best_shape(("copy", "copy_nontemporal"), flat_src, flat_dst, (1, 2, 4, 8), strided_bytes, "copy_best_shape")
+        def stream_shapes(modes, s_, d_, shapes):
+            return ([(mode, wg) for mode in modes for wg in shapes],
+                    lambda c: (lambda: wl.probe_memory(c[0], s_, d_, int(cus * c[1]))))
+        stream_note = "{best[0]} stream over 1 GiB, grid-stride dwordx4, best of {tried} (cache hint, launch shape) pairs: {best[1]} workgroups per compute unit"
+        choices, launch = stream_shapes(("read", "read_nontemporal"), flat_src, None, (1, 1.5, 2, 3, 4))
+        best_shape(launch, choices, strided_bytes // 2, "read_only", stream_note)
+        choices, launch = stream_shapes(("write", "write_nontemporal"), None, flat_dst, (0.5, 1, 2, 4))
+        best_shape(launch, choices, strided_bytes // 2, "write_only", stream_note)
+        choices, launch = stream_shapes(("copy", "copy_nontemporal"), flat_src, flat_dst, (1, 2, 4, 8))
+        best_shape(launch, choices, strided_bytes, "copy_best_shape", stream_note)
+        # the two halves of the transposition alone, with its own addresses in its own order
+        sink = torch.empty(8 * cus * 4, dtype=torch.float32, device=dev)
+        best_shape(lambda wg: (lambda: wl.probe_pattern("tile_read", src, None, sink, int(cus * wg))), (1, 1.5, 2, 3, 4), strided_bytes // 2,
+                   "strided_reads_alone", "the source tiles of the transposition (64 rows x 256 B, rows 64 KiB apart) read in its tile order, "
+                   "nothing written; best of {tried} launch shapes: {best} workgroups per compute unit")
+        best_shape(lambda wg: (lambda: wl.probe_pattern("tile_write", None, None, dst, int(cus * wg))), (0.5, 1, 1.5, 2, 3), strided_bytes // 2,
+                   "strided_writes_alone", "the destination tiles of the transposition written in its tile order, nothing read; best of "
+                   "{tried} launch shapes: {best} workgroups per compute unit")
+        del sink
     del src, dst, flat_src, flat_dst
 
     # ---- config 1: sequential copy in 16 KiB tiles: the 64 MiB of the configuration, and 1 GiB ----
@@ -259,7 +301,12 @@ def main():
         ms, _ = time_launches(lambda: wl.sequential_copy(s_src, s_dst, 0), max(steps, 50), warmup, SETTLE_MS)
         report(patterns, "sequential", ms, 2 * m * 4, "CudaDMASequential 16 KiB tiles of the configuration's 64 MiB f32 buffer: the "
                "128 MiB working set stays in the 256 MB Infinity Cache from launch to launch, so this is a cache-assisted rate, "
-               "not an HBM rate", bound="infinity cache + hbm")
+               "not an HBM rate", bound="infinity cache + hbm", launches=max(steps, 50))
+        if want("yardsticks"):
+            best_shape(lambda c: (lambda: wl.probe_memory(c[0], s_src, s_dst, int(cus * c[1]))),
+                       [(mode, wg) for mode in ("copy", "copy_nontemporal") for wg in (2, 4, 8)], 2 * m * 4, "copy_best_shape_64MiB",
+                       "{best[0]} stream over the same 64 MiB buffers (cache-assisted like the sequential row), best of {tried} "
+                       "(cache hint, launch shape) pairs: {best[1]} workgroups per compute unit")
         del s_src, s_dst
     if want("sequential_hbm"):
         m = 1024 * 1024 * 1024 // 4
@@ -270,6 +317,19 @@ def main():
                "next tile in the DMA wavefronts' registers, two workgroups per compute unit, streaming loads and non-temporal stores; "
                "destination exactly 1 GiB behind the source")
         del s_src, s_dst
+    if want("sequential_read_probe"):
+        # the reference's own metric (src/perf/sequential/perf_sequential.cu:354-361): bytes read into LDS per second, nothing written
+        m = 1024 * 1024 * 1024 // 4
+        s_src = pool[:m]
+        groups, elmt = 2 * cus, 16 * 1024
+        loops = (m * 4) // (groups * elmt)
+        run = lambda: wl.perf_sequential(s_src, elmt, 4, wl.BUFFERING_MANUAL, loops, groups, None, wl.LOAD_CACHE_STREAMING, wl.STORE_LDS)
+        nbytes = run()
+        ms, _ = time_launches(run, steps, warmup, SETTLE_MS)
+        report(patterns, "sequential_read_probe", ms, nbytes, "the reference's read-bandwidth probe on CudaDMASequential: 1 GiB read into LDS in "
+               "16 KiB elements and dropped, four DMA wavefronts + one compute wavefront per workgroup, two objects on the DMA wavefronts "
+               "(manual double buffering), LOAD_CACHE_STREAMING + STORE_LDS, 64 bytes per thread, two workgroups per compute unit")
+        del s_src
     del pool
 
     # ---- config 3: indirect gather, row-sum consumer: the 512 MiB table of the configuration, and a 4 GiB table ----
@@ -288,6 +348,10 @@ def main():
         sums = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, dtype=torch.float32, device=dev)
         ms, _ = time_launches(lambda: wl.gather_rowsum(table, idx, sums, 0), steps, warmup, SETTLE_MS)
         report(patterns, name, ms, n_idx * 4 + n_idx * 128 + sums.numel() * 4, note, bound=bound)
+        if want("yardsticks"):
+            best_shape(lambda wg: (lambda: wl.probe_pattern("gather_xor", table, idx, sums, int(cus * wg))), (3, 4, 6), n_idx * 132 + sums.numel() * 4,
+                       name + "_reads_alone", "the same index list and table read straight into registers (no LDS, no DMA object, xor instead of "
+                       "the sum), 128 B written per 32 records; best of {tried} launch shapes: {best} workgroups per compute unit")
         del table, idx, sums
 
     # ---- the opposite direction (LDS -> global): scatter of 4 Mi records by a permutation ----
@@ -299,6 +363,10 @@ def main():
         ms, _ = time_launches(lambda: wl.scatter_copy(records, perm, table, 0), steps, warmup, SETTLE_MS)
         report(patterns, "scatter", ms, recs * 4 + 2 * recs * 128,
                "CudaDMAIndirect<false> LDS -> global: 4 Mi records of 128 B placed by a permutation, 32 records per tile")
+        if want("yardsticks"):
+            best_shape(lambda wg: (lambda: wl.probe_pattern("scatter", records, perm, table, int(cus * wg))), (1, 2, 4), recs * 260,
+                       "scatter_writes_alone", "the same records placed by the same permutation straight from registers (no LDS, no DMA "
+                       "object); best of {tried} launch shapes: {best} workgroups per compute unit")
         del records, perm, table
 
     # ---- config 4: halo stencil ----
@@ -313,7 +381,11 @@ def main():
                    "(ring landed without handshake, one s_barrier per plane)")
         if want("halo_handshake"):
             ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 1), steps, warmup, SETTLE_MS)
-            report(patterns, "halo_handshake", ms, 2 * g ** 3 * 4, "same kernel with the empty/full handshake on the LDS planes next to the s_barrier")
+            report(patterns, "halo_handshake", ms, 2 * g ** 3 * 4, "same kernel with the empty/full handshake on the LDS planes next to the s_barrier "
+                   "(the split wait peek_dma_finish + wait_for_dma_finish(seen) keeps the poll off the critical path; the remaining cost is "
+                   "the two LDS words per plane)")
+            if "halo" in patterns:
+                patterns["halo_handshake"]["time_vs_halo"] = round(ms / patterns["halo"]["ms"], 4)
         if want("halo_wide_tiles"):
             ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, wl.HALO_WIDE_TILES_VARIANT), steps, warmup, SETTLE_MS)
             report(patterns, "halo_wide_tiles", ms, 2 * g ** 3 * 4, "the kernel of the halo row with tiles of 64x16 cells (rows of 256 B in memory) "
@@ -356,6 +428,24 @@ def main():
     value = patterns["strided"]["GB/s"]
     copies = [yardsticks[k]["GB/s"] for k in ("plain_copy", "vendor_copy", "copy_best_shape") if k in yardsticks]
     ceiling = max(copies) if copies else None
+    # every pattern against the yardstick of its own shape, measured in this run on the same buffers
+    halo_traffic = None
+    t_halo = traffic("halo")
+    if t_halo:
+        halo_traffic = t_halo / (2 * 512 ** 3 * 4)
+    priced = {"strided": ("copy_best_shape", 1.0), "strided_settled": ("copy_best_shape", 1.0), "strided_even_split": ("copy_best_shape", 1.0),
+              "strided_two_lds_tiles": ("copy_best_shape", 1.0), "sequential": ("copy_best_shape_64MiB", 1.0),
+              "sequential_hbm": ("copy_best_shape", 1.0), "sequential_read_probe": ("read_only", 1.0),
+              "gather": ("gather_reads_alone", 1.0), "gather_hbm": ("gather_hbm_reads_alone", 1.0), "scatter": ("scatter_writes_alone", 1.0),
+              "halo": ("copy_best_shape", halo_traffic), "halo_handshake": ("copy_best_shape", halo_traffic),
+              "halo_wide_tiles": ("copy_best_shape", halo_traffic)}
+    for name, (stick, factor) in priced.items():
+        if name in patterns and stick in yardsticks and factor:
+            c = yardsticks[stick]["GB/s"] / factor
+            patterns[name]["ceiling"] = round(c, 1)
+            patterns[name]["frac_of_ceiling"] = round(patterns[name]["GB/s"] / c, 4)
+            patterns[name]["ceiling_kind"] = f"yardsticks.{stick} of this run" + (
+                "" if factor == 1.0 else f" divided by {factor:.3f}: the kernel's measured HBM traffic per algorithmic byte (ghost cells and padding)")
     roofline = {"bound": "hbm", "achieved": value, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(value / HBM_PEAK_GBS, 4), "traffic": traffic("strided"),
                 "kernel": PATTERN_KERNELS["strided"], "kernel_ms": round(strided_ms, 4),
@@ -400,7 +490,8 @@ def main():
         result["cpu_baseline"], result["cpu_baseline_patterns"] = cpu_baselines()
         log(f"cpu baseline: {result['cpu_baseline']}")
         for name, row in result["cpu_baseline_patterns"].items():
-            log(f"  cpu {name:14s} {row['GB/s']:8.2f} GB/s   {row['sample']}")
+            rate = f"{row['GB/s']:8.2f} GB/s" if "GB/s" in row else f"{row['TFLOP/s']:8.4f} TFLOP/s"
+            log(f"  cpu {name:14s} {rate}   {row['sample']}")
     print(json.dumps(result), flush=True)
 
 

@@ -111,9 +111,13 @@ def lib():
     L.cudadma_variant_name.restype = ctypes.c_char_p
     L.cudadma_variant_name.argtypes = [ci, ci]
     L.cudadma_perf_sequential.restype = ctypes.c_longlong
-    L.cudadma_perf_sequential.argtypes = [vp, cs, vp, ci, ci, ci, ci, ci, vp]
+    L.cudadma_perf_sequential.argtypes = [vp, cs, vp, ci, ci, ci, ci, ci, ci, ci, vp]
     L.cudadma_probe_memory.restype = ctypes.c_longlong
     L.cudadma_probe_memory.argtypes = [ci, vp, vp, cs, ci, vp]
+    L.cudadma_probe_pattern.restype = ctypes.c_longlong
+    L.cudadma_probe_pattern.argtypes = [ci, vp, vp, vp, cs, cs, ci, vp]
+    L.cudadma_transpose_splits.restype = ci
+    L.cudadma_transpose_splits.argtypes = [ctypes.POINTER(ci), ci]
     L.cudadma_v1_get_case.restype = ci
     L.cudadma_v1_get_case.argtypes = [ci, ctypes.POINTER(V1Case)]
     L.cudadma_v1_case_text.restype = ctypes.c_char_p
@@ -174,4 +178,4 @@ def exported_symbols():
     """Every extern "C" symbol include/cudadma_amd.h declares."""
     return ["cudadma_last_error", "cudadma_device_cus", "cudadma_num_cases", "cudadma_get_case",
             "cudadma_run_case", "cudadma_variant_name", "cudadma_example_variant_name",
-            "cudadma_v1_get_case", "cudadma_v1_case_text", "cudadma_perf_sequential", "cudadma_probe_memory", "cudadma_plan_map", "cudadma_plan_extents", "cudadma_diagnose", "cudadma_set_tuning"] + list(_WORKLOAD_SIGNATURES)
+            "cudadma_v1_get_case", "cudadma_v1_case_text", "cudadma_perf_sequential", "cudadma_probe_memory", "cudadma_probe_pattern", "cudadma_transpose_splits", "cudadma_plan_map", "cudadma_plan_extents", "cudadma_diagnose", "cudadma_set_tuning"] + list(_WORKLOAD_SIGNATURES)

@@ -28,7 +28,7 @@ struct Knob {
   const char* name;
   std::atomic<int> value;
 };
-static Knob g_knobs[] = {{"transpose_band", {0}}, {"transpose_workgroups", {0}}, {"transpose_split", {0}}, {"stencil_zchunk", {0}}, {"stencil_xcd_remap", {0}}, {"stencil_ring", {0}}};
+static Knob g_knobs[] = {{"transpose_band", {0}}, {"transpose_workgroups", {0}}, {"transpose_split", {0}}, {"stencil_zchunk", {0}}, {"stencil_xcd_remap", {0}}, {"stencil_ring", {0}}, {"probe_piece_bytes", {0}}, {"probe_xcd_group", {0}}, {"transpose_wide_order", {0}}, {"transpose_wide_dma", {0}}};
 
 static Knob* find_knob(const char* name)
 {
@@ -80,6 +80,14 @@ static const VariantInfo kStrided[] = {
    "objects without a handshake of their own on the DMA wavefronts; the kernel the benchmark reports"},
   {"manual double buffer in LDS: one DMA group of 2 wavefronts, two CudaDMAStrided objects and two LDS tiles with padded "
    "rows (272 B), four workgroups per compute unit"},
+#ifdef HIPDMA_SWEEP_VARIANTS
+  {"output rows written 1 KiB at a time: the DMA side of variant 10 (tiles of 64 rows x 256 B, one LDS tile, one tile of loads "
+   "in flight), the compute wavefront gathers four tiles that lie side by side in the output in a second LDS buffer, "
+   "transposed, and writes 64 rows of 1 KiB with one store instruction per row (knobs transpose_wide_order, transpose_wide_dma)"},
+  {"variant 12 with two LDS tiles on the DMA side (still one tile of loads in flight)"},
+#else
+  {""}, {""},
+#endif
 };
 static const VariantInfo kGather[] = {
   {"the library's choice: variant 6 (two objects, index words requested one transfer ahead)"},
@@ -98,8 +106,16 @@ static const VariantInfo kHalo[] = {
   {"as variant 1 but the compute wavefronts meet in an LDS-counter GroupBarrier and the DMA wavefront runs free"},
   {"not warp-specialised, dwordx4 cells: every thread computes, half of them also carry a ring chunk requested one "
    "plane ahead; one LDS plane, two s_barriers per plane"},
+#ifdef HIPDMA_SWEEP_VARIANTS
   {"warp-specialised, one cell per dword load (first version kept for comparison)"},
+#else
+  {""},
+#endif
+#ifdef HIPDMA_SWEEP_VARIANTS
   {"not warp-specialised, one cell per dword load"},
+#else
+  {""},
+#endif
   {"variant 0 with tiles of 64 x 16 cells (rows of 256 B; nx a multiple of 64, ny of 16): 2 to 8 % faster at 512^3, not "
    "the tile the benchmark configuration names"},
   {"variant 1 with tiles of 64 x 16 cells"},
@@ -113,16 +129,32 @@ static const VariantInfo kGemm[] = {
    "ds_read_b64_tr_b16; 128 x 128 workgroup tile, 64 x 64 per compute wavefront, two workgroups per compute unit"},
   {"same structure, 128 x 256 workgroup tile, 64 x 128 per compute wavefront, one workgroup per compute unit"},
   {"same structure, 256 x 128 workgroup tile, 128 x 64 per compute wavefront, one workgroup per compute unit"},
+#ifdef HIPDMA_SWEEP_VARIANTS
   {"256 x 128 workgroup tile with the tiles brought in by global_load_lds_dwordx4 (STORE_LDS_DIRECT_SWIZZLE): three "
    "unpadded swizzled LDS stages, two transfers in flight per DMA wavefront, no ds_write"},
+#else
+  {""},
+#endif
+#ifdef HIPDMA_SWEEP_VARIANTS
   {"256 x 256 workgroup tile (m and n multiples of 256): eight compute wavefronts of 128 x 64, two per SIMD, next to the "
    "four DMA wavefronts; twelve wavefronts leave 168 registers each"},
+#else
+  {""},
+#endif
+#ifdef HIPDMA_SWEEP_VARIANTS
   {"256 x 256 workgroup tile, K step 32, four unpadded swizzled LDS stages filled by global_load_lds_dwordx4 "
    "(three transfers in flight per DMA wavefront), eight compute wavefronts"},
+#else
+  {""},
+#endif
   {"variant 6 with A transfers of two K steps (256 rows x 128 B, whole cache lines) into two 32 KB buffers with guards "
    "of their own; B keeps four stages of one K step"},
+#ifdef HIPDMA_SWEEP_VARIANTS
   {"not warp-specialised: 256 x 256 tile, four wavefronts that each issue their share of the direct-to-LDS loads and "
    "multiply a 128 x 128 block; one s_barrier per K step"},
+#else
+  {""},
+#endif
   {"variant 8 with A transfers of two K steps (rows of 128 B, whole cache lines) into a ring of three buffers: with the "
    "four B stages all of the 160 KB of LDS"},
 };

@@ -250,6 +250,7 @@ struct Three {
   template<int I> __device__ __forceinline__ T& get() { if constexpr (I == 0) return a0; else if constexpr (I == 1) return a1; else return a2; }
 };
 
+#ifdef HIPDMA_SWEEP_VARIANTS
 __global__ void __launch_bounds__(kComputeThreads + 2 * kDmaWave)
 gemm_bf16_ws_direct(const unsigned short* __restrict__ a, const unsigned short* __restrict__ b, float* __restrict__ c,
                     const int m, const int n, const int k)
@@ -399,6 +400,7 @@ gemm_bf16_ws_direct(const unsigned short* __restrict__ a, const unsigned short* 
         }
   }
 }
+#endif  // HIPDMA_SWEEP_VARIANTS
 
 // ---- 256 x 256 tile, K step 32, four unpadded swizzled stages filled by global_load_lds_dwordx4 ----
 // Eight compute wavefronts (2 x 4, 128 x 64 each, two per SIMD) and four DMA wavefronts.  A stage is
@@ -411,6 +413,7 @@ struct Four4 {
 
 constexpr int kDirect4DmaThreads = 128;    // DMA threads per operand
 constexpr int kDirect4Ahead = 3;           // transfers in flight per DMA wavefront (2: 3 % slower; 4 stages allow no more)
+#ifdef HIPDMA_SWEEP_VARIANTS
 __global__ void __launch_bounds__(512 + 2 * kDirect4DmaThreads)
 gemm_bf16_ws_direct4(const unsigned short* __restrict__ a, const unsigned short* __restrict__ b, float* __restrict__ c,
                      const int m, const int n, const int k)
@@ -554,6 +557,7 @@ gemm_bf16_ws_direct4(const unsigned short* __restrict__ a, const unsigned short*
         }
   }
 }
+#endif  // HIPDMA_SWEEP_VARIANTS
 
 // ---- the same kernel with A rows of 128 B: an A transfer covers two K steps ----
 // A K step of 32 takes 64 B of every A row, half a cache line: the L1 fetches each line of the A
@@ -733,6 +737,7 @@ gemm_bf16_ws_direct4_a64(const unsigned short* __restrict__ a, const unsigned sh
 // and with it its matrix core, for 550 cycles: the address unit takes one 16-byte load of a wavefront per
 // sixteen cycles); the fragments of the next slice, in the second half those of the next stage, are requested
 // under the products of the current one.
+#ifdef HIPDMA_SWEEP_VARIANTS
 __global__ void __launch_bounds__(256)
 gemm_bf16_all_direct(const unsigned short* __restrict__ a, const unsigned short* __restrict__ b, float* __restrict__ c,
                      const int m, const int n, const int k)
@@ -878,6 +883,7 @@ gemm_bf16_all_direct(const unsigned short* __restrict__ a, const unsigned short*
         __builtin_nontemporal_store(acc[i][j][e], &cbase[(size_t)row * n + col]);
       }
 }
+#endif  // HIPDMA_SWEEP_VARIANTS
 
 // ---- the same kernel with A transfers of two K steps (rows of 128 B) ----
 // A K step of 32 takes 64 B of an A row, half a cache line, and the L1 asks the L2 for every line of the A panel
@@ -1092,25 +1098,35 @@ extern "C" int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float
     case 1: return launch_gemm<2, 2>(d_a, d_b, d_c, m, n, k, s);
     case 2: return launch_gemm<2, 4>(d_a, d_b, d_c, m, n, k, s);
     case 3: return launch_gemm<4, 2>(d_a, d_b, d_c, m, n, k, s);
+#ifdef HIPDMA_SWEEP_VARIANTS
     case 5: return launch_gemm<4, 2, 2, 4>(d_a, d_b, d_c, m, n, k, s);
+#endif
     case 6: case 7: case 8: case 9: {
       CUDADMA_REQUIRE((m % 256) == 0 && (n % 256) == 0, "this variant needs m and n multiples of 256 (got %d x %d)", m, n);
       const long long grid = (long long)(m / 256) * (n / 256);
       CUDADMA_REQUIRE(grid <= 0x7fffffffLL, "grid too large");
-      if (variant == 6) hipLaunchKernelGGL(gemm_bf16_ws_direct4, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
-      else if (variant == 7) hipLaunchKernelGGL(gemm_bf16_ws_direct4_a64, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
-      else if (variant == 8) hipLaunchKernelGGL(gemm_bf16_all_direct, dim3((unsigned)grid), dim3(256), 0, s, d_a, d_b, d_c, m, n, k);
-      else hipLaunchKernelGGL(gemm_bf16_all_direct_a64, dim3((unsigned)grid), dim3(256), 0, s, d_a, d_b, d_c, m, n, k);
+      if (variant == 7) hipLaunchKernelGGL(gemm_bf16_ws_direct4_a64, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
+      else if (variant == 9) hipLaunchKernelGGL(gemm_bf16_all_direct_a64, dim3((unsigned)grid), dim3(256), 0, s, d_a, d_b, d_c, m, n, k);
+#ifdef HIPDMA_SWEEP_VARIANTS
+      else if (variant == 6) hipLaunchKernelGGL(gemm_bf16_ws_direct4, dim3((unsigned)grid), dim3(512 + 2 * kDirect4DmaThreads), 0, s, d_a, d_b, d_c, m, n, k);
+      else hipLaunchKernelGGL(gemm_bf16_all_direct, dim3((unsigned)grid), dim3(256), 0, s, d_a, d_b, d_c, m, n, k);
+#else
+      else CUDADMA_REQUIRE(false, "gemm variant %d is a sweep kernel: build the library with make EXTRA=-DHIPDMA_SWEEP_VARIANTS", variant);
+#endif
       CUDADMA_HIP_CHECK(hipGetLastError());
       return CUDADMA_OK;
     }
     default: {
+#ifdef HIPDMA_SWEEP_VARIANTS
       CUDADMA_REQUIRE((m % 256) == 0, "this variant needs m a multiple of 256 (got %d)", m);
       const long long grid = (long long)(m / 256) * (n / 128);
       CUDADMA_REQUIRE(grid <= 0x7fffffffLL, "grid too large");
       hipLaunchKernelGGL(gemm_bf16_ws_direct, dim3((unsigned)grid), dim3(kComputeThreads + 2 * kDmaWave), 0, s, d_a, d_b, d_c, m, n, k);
       CUDADMA_HIP_CHECK(hipGetLastError());
       return CUDADMA_OK;
+#else
+      CUDADMA_REQUIRE(false, "gemm variant %d is a sweep kernel: build the library with make EXTRA=-DHIPDMA_SWEEP_VARIANTS", variant);
+#endif
     }
   }
 }

@@ -108,6 +108,7 @@ __device__ __forceinline__ TileWork tile_work(const float* in, float* out, const
   return w;
 }
 
+#ifdef HIPDMA_SWEEP_VARIANTS
 __global__ void __launch_bounds__(kComputeThreads + kDmaThreads)
 stencil_warp_specialized(const float* __restrict__ in, float* __restrict__ out, const int nx, const int ny,
                          const int nz, const int zchunk, const Coeffs k)
@@ -179,7 +180,9 @@ stencil_warp_specialized(const float* __restrict__ in, float* __restrict__ out, 
     }
   }
 }
+#endif  // HIPDMA_SWEEP_VARIANTS
 
+#ifdef HIPDMA_SWEEP_VARIANTS
 __global__ void __launch_bounds__(kComputeThreads)
 stencil_not_specialized(const float* __restrict__ in, float* __restrict__ out, const int nx, const int ny,
                         const int nz, const int zchunk, const Coeffs k)
@@ -222,6 +225,7 @@ stencil_not_specialized(const float* __restrict__ in, float* __restrict__ out, c
     __syncthreads();
   }
 }
+#endif  // HIPDMA_SWEEP_VARIANTS
 
 // ---------------------------------------------------------------------------
 // dwordx4 version: a compute thread owns four consecutive cells of one tile row
@@ -662,8 +666,12 @@ extern "C" int cudadma_halo_stencil(const float* d_in, float* d_out, int nx, int
       else hipLaunchKernelGGL((stencil_ws_vec4<kHandshakeAndGroupBarrier, 8>), g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k);
       break;
     case 3: hipLaunchKernelGGL(stencil_all_vec4, g, all, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+#ifdef HIPDMA_SWEEP_VARIANTS
     case 4: hipLaunchKernelGGL(stencil_warp_specialized, g, ws, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
     default: hipLaunchKernelGGL(stencil_not_specialized, g, all, 0, s, d_in, d_out, nx, ny, nz, zchunk, k); break;
+#else
+    default: CUDADMA_REQUIRE(false, "halo stencil variant %d is a sweep kernel: build the library with make EXTRA=-DHIPDMA_SWEEP_VARIANTS", variant);
+#endif
   }
   CUDADMA_HIP_CHECK(hipGetLastError());
   return CUDADMA_OK;

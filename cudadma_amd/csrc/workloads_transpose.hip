@@ -364,6 +364,7 @@ template<int DW, int CW, int AHEAD>
 __global__ void __launch_bounds__((DW + CW) * 64)
 transpose_split(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles, const int band)
 {
+  const int first_tile = blockIdx.x;
   static_assert(CW == 1 || CW == 2 || CW == 4, "the compute wavefronts share the sixteen 16-byte columns of a tile row evenly");
   static_assert(AHEAD >= 1 && AHEAD <= 3, "one or two tiles requested ahead, or (3) one in flight with two register sets");
   constexpr int kLdsRow = 272;
@@ -388,7 +389,7 @@ transpose_split(const float* __restrict__ in, float* __restrict__ out, const int
       o.template wait_xfer_finish<true, LOAD_CACHE_STREAMING, STORE_LDS>(buf);
       guard.finish_async_dma();
     };
-    int t = blockIdx.x;
+    int t = first_tile;
     if (t >= num_tiles) return;
     a.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t));
     if constexpr (AHEAD == 3) {
@@ -426,7 +427,7 @@ transpose_split(const float* __restrict__ in, float* __restrict__ out, const int
     const int lane = threadIdx.x & 63;
     const int w = threadIdx.x >> 6;
     guard.start_async_dma();
-    for (int t = blockIdx.x; t < num_tiles; t += stride) {
+    for (int t = first_tile; t < num_tiles; t += stride) {
       int ty, tx;
       tile_coords(t, tiles_per_side, band, ty, tx);
       guard.wait_for_dma_finish();
@@ -439,6 +440,114 @@ transpose_split(const float* __restrict__ in, float* __restrict__ out, const int
 #pragma unroll
       for (int j = 0; j < kUnits; ++j)
         __builtin_nontemporal_store(quad_transpose(v[j], lane), (vec4_t*)(o + (size_t)(4 * j) * n));
+    }
+  }
+}
+
+#ifdef HIPDMA_SWEEP_VARIANTS
+// The transposition with output rows written 1 KiB at a time.  The DMA side is that of transpose_split (tiles of 64
+// rows x 256 B, one tile of loads in flight, NBUF LDS tiles guarded by sync-only objects); the compute wavefront
+// gathers four tiles that lie one below the other in the source (so side by side in the output) in a second LDS
+// buffer, already transposed (four ds_write_b32 per 16-byte unit, 64 lanes on 64 consecutive words: no conflicts),
+// and then writes 64 output rows of 1 KiB, one row per store instruction.  A write-only stream with the
+// transposition's addresses runs at 67 % of peak in pieces of 256 B and at 78 % in pieces of 1 KiB; the reads care
+// less (87 % in pieces of 256 B against 91 % for a linear stream).  Reads and writes together gain nothing from it:
+// 74.0 % against 74.8 % for transpose_split<3, 1, 1> in the same run, which is why this kernel is only built for the
+// sweeps.
+// order 0: the workgroups that run together take neighbouring groups of four tile rows first (they write whole output
+// rows together); order 1: neighbouring tile columns first (they read whole source rows together).
+template<int DW, int NBUF>
+__global__ void __launch_bounds__((DW + 1) * 64)
+transpose_wide_rows(const float* __restrict__ in, float* __restrict__ out, const int n, const int order)
+{
+  static_assert(NBUF == 1 || NBUF == 2, "one or two LDS tiles");
+  constexpr int kLdsRow = 272;
+  constexpr int kDma = DW * 64, kCompute = 64;
+  constexpr int kChunks = kTile * kRowBytes / 16;
+  constexpr int kBpt = ((kChunks + kDma - 1) / kDma) * 16;
+  constexpr int kGroup = 4;                               // tiles gathered per pass: 4 x 256 B = 1 KiB of every output row
+  __shared__ __attribute__((aligned(16))) char buf[NBUF][kTile * kLdsRow];
+  __shared__ __attribute__((aligned(16))) float stage[kTile][kGroup * kTile];
+  cudaDMACustom guard0(0, kDma, kCompute, kCompute);
+  cudaDMACustom guard1(1, kDma, kCompute, kCompute);
+  typedef CudaDMAStrided<false, 16, kBpt, kRowBytes, kDma, kTile> obj_t;
+  const int tiles_per_side = n / kTile;
+  const int groups_per_side = (tiles_per_side + kGroup - 1) / kGroup;
+  const int passes = groups_per_side * tiles_per_side;    // a pass: up to four tiles (group q of tile rows, tile column tx)
+  const int stride = gridDim.x;
+  auto pass_coords = [&](const int p, int& q, int& tx) {
+    if (order == 0) { tx = p / groups_per_side; q = p - tx * groups_per_side; }
+    else { q = p / tiles_per_side; tx = p - q * tiles_per_side; }
+  };
+  auto tiles_in = [&](const int q) { const int left = tiles_per_side - q * kGroup; return left < kGroup ? left : kGroup; };
+  if (guard0.owns_this_thread()) {
+    obj_t a(n * 4, kLdsRow, kCompute);
+    int p = blockIdx.x;
+    if (p >= passes) return;
+    int q, tx, k = 0;
+    pass_coords(p, q, tx);
+    int count = tiles_in(q);
+    auto src_now = [&]() { return (const void*)(in + (size_t)(q * kGroup + k) * kTile * n + (size_t)tx * kTile); };
+    a.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_now());
+    unsigned i = 0;
+    for (;;) {
+      if (NBUF == 2 && (i & 1u)) {
+        guard1.wait_for_dma_start();
+        a.template wait_xfer_finish<true, LOAD_CACHE_STREAMING, STORE_LDS>(buf[NBUF - 1]);
+        guard1.finish_async_dma();
+      } else {
+        guard0.wait_for_dma_start();
+        a.template wait_xfer_finish<true, LOAD_CACHE_STREAMING, STORE_LDS>(buf[0]);
+        guard0.finish_async_dma();
+      }
+      ++i;
+      if (++k == count) {
+        p += stride;
+        if (p >= passes) break;
+        pass_coords(p, q, tx);
+        count = tiles_in(q);
+        k = 0;
+      }
+      a.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_now());
+    }
+  } else {
+    const int lane = threadIdx.x & 63;
+    guard0.start_async_dma();
+    if constexpr (NBUF == 2) guard1.start_async_dma();
+    unsigned i = 0;
+    for (int p = blockIdx.x; p < passes; p += stride) {
+      int q, tx;
+      pass_coords(p, q, tx);
+      const int count = tiles_in(q);
+      for (int k = 0; k < count; ++k, ++i) {
+        const bool second = NBUF == 2 && (i & 1u);
+        if (second) guard1.wait_for_dma_finish(); else guard0.wait_for_dma_finish();
+        // lane = tile row r: its sixteen 16-byte units
+        vec4_t v[16];
+        const vec4_t* row = (const vec4_t*)(buf[second ? NBUF - 1 : 0] + lane * kLdsRow);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) v[j] = row[j];
+        if (second) guard1.start_async_dma(); else guard0.start_async_dma();
+        // element (r, c) of tile k becomes word 64 k + r of output row c
+        float* col = &stage[0][k * kTile + lane];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+#pragma unroll
+          for (int w = 0; w < 4; ++w) col[(4 * j + w) * (kGroup * kTile)] = __uint_as_float(v[j][w]);
+        }
+      }
+      // 64 output rows of count x 256 B: lane l carries the 16 bytes at 16 l of every row
+      float* o = out + (size_t)tx * kTile * n + (size_t)q * (kGroup * kTile) + 4 * lane;
+      if (lane < 16 * count) {
+#pragma unroll
+        for (int batch = 0; batch < 4; ++batch) {
+          vec4_t w[16];
+#pragma unroll
+          for (int m = 0; m < 16; ++m) w[m] = *(const vec4_t*)&stage[16 * batch + m][4 * lane];
+#pragma unroll
+          for (int m = 0; m < 16; ++m) __builtin_nontemporal_store(w[m], (vec4_t*)(o + (size_t)(16 * batch + m) * n));
+        }
+      }
     }
   }
 }
@@ -519,21 +628,38 @@ transpose_pieces(const float* __restrict__ in, float* __restrict__ out, const in
     }
   }
 }
+#endif  // HIPDMA_SWEEP_VARIANTS
 
 typedef void (*split_kernel_t)(const float*, float*, int, int, int);
 struct SplitEntry { int dw, cw, ahead; split_kernel_t kernel; };
 #define SPLIT(DW, CW) {DW, CW, 1, transpose_split<DW, CW, 1>}, {DW, CW, 2, transpose_split<DW, CW, 2>}
-// "tiles ahead" 3 .. 7 stand for a tile requested in pieces (the fastest split only): 3 = 3 halves in flight (1.5 tiles),
-// 4 = 5 quarters (1.25), 5 = 6 quarters (1.5), 6 = 7 quarters (1.75), 7 = 3 quarters (0.75)
-const SplitEntry kSplits[] = {{3, 1, 3, transpose_pieces<3, 1, 2, 3>}, {3, 1, 4, transpose_pieces<3, 1, 4, 5>},
+// The library holds the split it reports (three DMA wavefronts + one compute wavefront), the even split, and both with
+// two tiles ahead.  The other splits, the tile requested in pieces ("tiles ahead" 3 .. 7 with 3 + 1 wavefronts: 3 = 3
+// halves in flight (1.5 tiles), 4 = 5 quarters (1.25), 5 = 6 quarters (1.5), 6 = 7 quarters (1.75), 7 = 3 quarters
+// (0.75)) and the schedule without a pause (8: two register sets, the next tile requested as soon as the loads of the
+// current one have returned) were all measured slower; they are compiled with -DHIPDMA_SWEEP_VARIANTS for the sweeps.
+const SplitEntry kSplits[] = {SPLIT(3, 1), SPLIT(2, 2),
+#ifdef HIPDMA_SWEEP_VARIANTS
+                              {3, 1, 3, transpose_pieces<3, 1, 2, 3>}, {3, 1, 4, transpose_pieces<3, 1, 4, 5>},
                               {3, 1, 5, transpose_pieces<3, 1, 4, 6>}, {3, 1, 6, transpose_pieces<3, 1, 4, 7>},
                               {3, 1, 7, transpose_pieces<3, 1, 4, 3>},
-                              // 8 = two register sets, one tile in flight without a pause
-                              {3, 1, 8, transpose_split<3, 1, 3>}, {2, 2, 8, transpose_split<2, 2, 3>}, SPLIT(2, 2), SPLIT(1, 1), SPLIT(1, 2), SPLIT(2, 1), SPLIT(3, 1), SPLIT(4, 1), SPLIT(3, 2), SPLIT(4, 2),
-                              SPLIT(1, 4), SPLIT(2, 4), SPLIT(4, 4)};
+                              {3, 1, 8, transpose_split<3, 1, 3>}, {2, 2, 8, transpose_split<2, 2, 3>},
+                              SPLIT(1, 1), SPLIT(1, 2), SPLIT(2, 1), SPLIT(4, 1), SPLIT(3, 2), SPLIT(4, 2), SPLIT(1, 4), SPLIT(2, 4), SPLIT(4, 4),
+#endif
+};
 #undef SPLIT
 
 }  // namespace
+
+extern "C" int cudadma_transpose_splits(int* codes, int capacity)
+{
+  int n = 0;
+  for (const SplitEntry& c : kSplits) {
+    if (codes != nullptr && n < capacity) codes[n] = 100 * c.dw + 10 * c.cw + c.ahead;
+    ++n;
+  }
+  return n;
+}
 
 extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n, int variant, void* stream)
 {
@@ -580,10 +706,36 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
       const SplitEntry* e = nullptr;
       for (const SplitEntry& c : kSplits)
         if (100 * c.dw + 10 * c.cw + c.ahead == code) e = &c;
-      CUDADMA_REQUIRE(e != nullptr, "no transposition kernel was compiled for the split %d", code);
+      CUDADMA_REQUIRE(e != nullptr, "this build of the library holds no transposition kernel for the split %d (cudadma_transpose_splits lists "
+                                       "those it holds; the rest are compiled with -DHIPDMA_SWEEP_VARIANTS)", code);
       hipLaunchKernelGGL(e->kernel, grid_for(1), dim3((e->dw + e->cw) * 64), 0, s, d_in, d_out, n, tiles, band);
       break;
     }
+#ifdef HIPDMA_SWEEP_VARIANTS
+    case 12:
+    case 13: {
+      // output rows written 1 KiB at a time; knobs: "transpose_wide_order" 1 = neighbouring tile columns first,
+      // "transpose_wide_dma" = DMA wavefronts (3 by default; 2 or 4)
+      const int order = workloads::tuning("transpose_wide_order", 1) - 1;
+      const int dw = workloads::tuning("transpose_wide_dma", 3);
+      const int passes = ((tiles_per_side + 3) / 4) * tiles_per_side;
+      const dim3 g((unsigned)(forced > 0 ? (forced < passes ? forced : passes) : workloads::persistent_grid(passes, 1)));
+      CUDADMA_REQUIRE(dw >= 2 && dw <= 4, "transpose_wide_dma: 2, 3 or 4 DMA wavefronts");
+      if (variant == 12) {
+        if (dw == 2) hipLaunchKernelGGL((transpose_wide_rows<2, 1>), g, dim3(192), 0, s, d_in, d_out, n, order);
+        else if (dw == 3) hipLaunchKernelGGL((transpose_wide_rows<3, 1>), g, dim3(256), 0, s, d_in, d_out, n, order);
+        else hipLaunchKernelGGL((transpose_wide_rows<4, 1>), g, dim3(320), 0, s, d_in, d_out, n, order);
+      } else {
+        if (dw == 2) hipLaunchKernelGGL((transpose_wide_rows<2, 2>), g, dim3(192), 0, s, d_in, d_out, n, order);
+        else if (dw == 3) hipLaunchKernelGGL((transpose_wide_rows<3, 2>), g, dim3(256), 0, s, d_in, d_out, n, order);
+        else hipLaunchKernelGGL((transpose_wide_rows<4, 2>), g, dim3(320), 0, s, d_in, d_out, n, order);
+      }
+      break;
+    }
+#else
+    case 12:
+    case 13: CUDADMA_REQUIRE(false, "variants 12 and 13 are sweep kernels: build the library with make EXTRA=-DHIPDMA_SWEEP_VARIANTS");
+#endif
     default: hipLaunchKernelGGL(transpose_not_specialized, grid_for(1), block, 0, s, d_in, d_out, n, tiles, band); break;
   }
   CUDADMA_HIP_CHECK(hipGetLastError());

@@ -9,6 +9,8 @@ point; here the variants are compiled in and the occupancy is a run-time knob.
     python -m cudadma_amd.sweep transpose_split              # DMA : compute wavefronts x tiles ahead x workgroups per CU
     python -m cudadma_amd.sweep transpose_walk               # tile order x workgroup count, one-tile and two-tile kernels
     python -m cudadma_amd.sweep placement                    # 1 GiB copies against the distance between source and destination
+    python -m cudadma_amd.sweep queue_depth --config NAME    # one launch shape of QUEUE_CONFIGS, a few launches: the process to put
+                                                             # under rocprofv3 --pmc when asking what more work in flight costs
 """
 import argparse
 import sys
@@ -19,6 +21,20 @@ from . import examples as ex
 from . import workloads as wl
 
 PEAK_GBS = 8000.0
+
+# Launch shapes that differ only in how much work a compute unit has in flight: (what to launch, knobs / workgroups per compute
+# unit).  `python -m cudadma_amd.sweep queue_depth --config NAME` runs one of them on 2 x 1 GiB; cudadma_amd.profile_summary
+# tabulates the counters of such runs.
+QUEUE_CONFIGS = {
+    "transpose_1wg_1tile": ("transpose", {"transpose_split": 311, "transpose_workgroups": 1}),
+    "transpose_2wg_1tile": ("transpose", {"transpose_split": 311, "transpose_workgroups": 2}),
+    "transpose_1wg_2tiles": ("transpose", {"transpose_split": 312, "transpose_workgroups": 1}),
+    "transpose_2wg_2tiles": ("transpose", {"transpose_split": 312, "transpose_workgroups": 2}),
+    "copy_2wg": ("copy_nontemporal", 2), "copy_4wg": ("copy_nontemporal", 4), "copy_8wg": ("copy_nontemporal", 8),
+    "copy_16wg": ("copy_nontemporal", 16),
+    "read_1.5wg": ("read_nontemporal", 1.5), "read_4wg": ("read_nontemporal", 4), "read_8wg": ("read_nontemporal", 8),
+    "write_0.5wg": ("write", 0.5), "write_4wg": ("write", 4), "write_8wg": ("write", 8),
+}
 
 
 def _time(fn, steps, warmup=3, settle_ms=30.0):
@@ -53,6 +69,7 @@ def main(argv=None):
     ap.add_argument("workloads", nargs="*", default=["sequential", "strided", "gather", "halo", "gemm"])
     ap.add_argument("--wg", default="0,2,4,8", help="workgroups per compute unit to try (0 = each kernel's default)")
     ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--config", default="", help="queue_depth: name of the launch shape (see QUEUE_CONFIGS)")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         sys.exit("no GPU visible")
@@ -62,7 +79,7 @@ def main(argv=None):
         if name == "sequential":
             src = wl.fill_uniform(torch.empty(16 << 20, device=dev), 1001)
             dst = torch.empty_like(src)
-            for v in range(wl.num_variants(wl.SEQUENTIAL)):
+            for v in wl.variants(wl.SEQUENTIAL):
                 print(f"# sequential variant {v}: {wl.variant_name(wl.SEQUENTIAL, v)}")
                 for wg in wgs:
                     wl.set_workgroups_per_cu(wg)
@@ -71,7 +88,7 @@ def main(argv=None):
             n = 16384
             src = wl.fill_uniform(torch.empty(n * n, device=dev), 1002).view(n, n)
             dst = torch.empty_like(src)
-            for v in range(wl.num_variants(wl.STRIDED)):
+            for v in wl.variants(wl.STRIDED):
                 print(f"# strided variant {v}: {wl.variant_name(wl.STRIDED, v)}")
                 for wg in wgs:
                     wl.set_workgroups_per_cu(wg)
@@ -82,7 +99,7 @@ def main(argv=None):
             table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1003)
             idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=dev), recs, 1003)
             out = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, device=dev)
-            for v in range(wl.num_variants(wl.GATHER)):
+            for v in wl.variants(wl.GATHER):
                 print(f"# gather (row-sum) variant {v}: {wl.variant_name(wl.GATHER, v)}")
                 for wg in wgs:
                     wl.set_workgroups_per_cu(wg)
@@ -113,7 +130,7 @@ def main(argv=None):
             ref = src.t().contiguous()
             cus = torch.cuda.get_device_properties(0).multi_processor_count
             print("# DMA + compute wavefronts, tiles ahead: ms (% of 8 TB/s) at 1 / 2 / 3 workgroups per compute unit")
-            for code in wl.TRANSPOSE_SPLITS:
+            for code in wl.transpose_splits():
                 wl.set_tuning("transpose_split", code)
                 dst.zero_()
                 wl.strided_transpose(src, dst, wl.TRANSPOSE_SPLIT_VARIANT)
@@ -171,12 +188,34 @@ def main(argv=None):
                     cells.append(f"{ms:.4f} ({2 * m * 4 / ms / 1e6 / PEAK_GBS * 100:4.1f}%)")
                 print(f"+{off:>9d} B:  " + "   ".join(cells), flush=True)
             del pool
+        elif name == "queue_depth":
+            if args.config not in QUEUE_CONFIGS:
+                sys.exit("--config must be one of: " + ", ".join(QUEUE_CONFIGS))
+            what, shape = QUEUE_CONFIGS[args.config]
+            m = (1 << 30) // 4
+            pool = torch.empty(2 * m, device=dev)              # destination exactly 1 GiB behind the source
+            src, dst = wl.fill_uniform(pool[:m], 1002), pool[m:]
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            if what == "transpose":
+                wl.set_tuning("transpose_split", shape["transpose_split"])
+                wl.set_tuning("transpose_workgroups", cus * shape["transpose_workgroups"])
+                fn = lambda: wl.strided_transpose(src.view(16384, 16384), dst.view(16384, 16384), wl.TRANSPOSE_SPLIT_VARIANT)
+                nbytes = 2 * m * 4
+            else:
+                s_, d_ = (None if what.startswith("write") else src), (None if what.startswith("read") else dst)
+                fn = lambda: wl.probe_memory(what, s_, d_, int(cus * shape))
+                nbytes = (m * 4 if s_ is not None else 0) + (m * 4 if d_ is not None else 0)
+            ms = _time(fn, args.steps, warmup=2, settle_ms=0.0)
+            print(f"queue_depth {args.config:22s} {ms:8.4f} ms  {nbytes / ms / 1e6:7.0f} GB/s  {100 * nbytes / ms / 1e6 / PEAK_GBS:5.1f}%", flush=True)
+            wl.set_tuning("transpose_split", 0)
+            wl.set_tuning("transpose_workgroups", 0)
+            del pool
         elif name == "scatter":
             recs = 4 << 20
             records = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1006)
             perm = wl.fill_permutation(torch.empty(recs, dtype=torch.int32, device=dev), 1006)
             table = torch.empty(recs * wl.REC_FLOATS, device=dev)
-            for v in range(wl.num_variants(wl.SCATTER)):
+            for v in wl.variants(wl.SCATTER):
                 print(f"# scatter variant {v}: {wl.variant_name(wl.SCATTER, v)}")
                 for wg in wgs:
                     wl.set_workgroups_per_cu(wg)
@@ -185,7 +224,7 @@ def main(argv=None):
             g = 512
             gi = wl.fill_uniform(torch.empty((g + 8) ** 3, device=dev), 1004).view(g + 8, g + 8, g + 8)
             go = torch.empty(g, g, g, device=dev)
-            for v in range(wl.num_variants(wl.HALO)):
+            for v in wl.variants(wl.HALO):
                 print(f"# halo variant {v}: {wl.variant_name(wl.HALO, v)}")
                 for zc in (0, 128, 256, 512):
                     wl.set_tuning("stencil_zchunk", zc)
@@ -200,7 +239,7 @@ def main(argv=None):
                 a = torch.randn(n, n, device=dev).to(torch.bfloat16)
                 b = torch.randn(n, n, device=dev).to(torch.bfloat16)
                 c = torch.empty(n, n, device=dev)
-                for v in range(1, wl.num_variants(wl.GEMM)):
+                for v in wl.variants(wl.GEMM)[1:]:
                     ms = _time(lambda: wl.gemm_bf16(a, b, c, v), args.steps, settle_ms=10.0)
                     print(f"gemm {n}^3  variant {v}  {ms:9.4f} ms  {2.0 * n ** 3 / ms / 1e9:8.1f} TFLOP/s", flush=True)
                 ms = _time(lambda: torch.matmul(a, b), args.steps, settle_ms=10.0)
@@ -208,22 +247,29 @@ def main(argv=None):
                 del a, b, c
         elif name == "perf_sequential":
             # src/perf/sequential/param_sweep.py:27-58: element size x DMA wavefronts x workgroups per CU x
-            # buffering; a launch reads 1 GiB whatever the point (loop count follows from that)
+            # buffering; a launch reads 1 GiB whatever the point (loop count follows from that).  On top of the
+            # reference's space: the cache qualifier of the loads and how the bytes reach LDS.
             src = wl.fill_uniform(torch.empty(1 << 28, device=dev), 1001)
             cus = torch.cuda.get_device_properties(0).multi_processor_count
-            print("# read bandwidth into LDS, GB/s (1 GiB per launch); columns: buffering none / single / double / manual")
-            for elmt in (32, 128, 512, 2048, 4096, 8192, 16384):
-                for waves in (1, 2, 4):
-                    for wg in wgs if wgs != [0] else [4]:
-                        wg = wg or 4
-                        groups = cus * wg
-                        loops = max(1, (1 << 30) // (groups * elmt))
-                        cells = []
-                        for b in range(4):
-                            nbytes = wl.perf_sequential(src, elmt, waves, b, loops, groups)
-                            ms = _time(lambda: wl.perf_sequential(src, elmt, waves, b, loops, groups), args.steps, settle_ms=5.0)
-                            cells.append(f"{nbytes / ms / 1e6:7.0f}")
-                        print(f"elmt {elmt:6d} B  dma waves {waves}  wg/cu {wg:2d}  loops {loops:6d}  " + " ".join(cells), flush=True)
+            quals = (("LOAD_CACHE_ALL, STORE_WRITE_BACK (the reference's defaults)", wl.LOAD_CACHE_ALL, wl.STORE_WRITE_BACK),
+                     ("LOAD_CACHE_STREAMING, STORE_LDS", wl.LOAD_CACHE_STREAMING, wl.STORE_LDS),
+                     ("LOAD_CACHE_ALL, STORE_LDS_DIRECT", wl.LOAD_CACHE_ALL, wl.STORE_LDS_DIRECT),
+                     ("LOAD_CACHE_STREAMING, STORE_LDS_DIRECT", wl.LOAD_CACHE_STREAMING, wl.STORE_LDS_DIRECT))
+            for label, lq, sq in quals:
+                print(f"# {label}: read bandwidth into LDS, GB/s (1 GiB per launch); columns: buffering none / single / double / manual")
+                for elmt in (32, 128, 512, 2048, 4096, 8192, 16384):
+                    for waves in (1, 2, 4):
+                        for wg in wgs if wgs != [0] else [4]:
+                            wg = wg or 4
+                            groups = cus * wg
+                            loops = max(1, (1 << 30) // (groups * elmt))
+                            cells = []
+                            for b in range(4):
+                                run = lambda: wl.perf_sequential(src, elmt, waves, b, loops, groups, None, lq, sq)
+                                nbytes = run()
+                                ms = _time(run, args.steps, settle_ms=5.0)
+                                cells.append(f"{nbytes / ms / 1e6:7.0f}")
+                            print(f"elmt {elmt:6d} B  dma waves {waves}  wg/cu {wg:2d}  loops {loops:6d}  " + " ".join(cells), flush=True)
         elif name == "saxpy":
             # bytes as the reference's driver counts them: x read, y read, y written (saxpy_cudaDMA.cu:192)
             n = 1 << 28

@@ -14,12 +14,10 @@ RECS_PER_TILE = 32
 SEQ_TILE_BYTES = 16 * 1024
 STENCIL_RADIUS = 4
 TRANSPOSE_SPLIT_VARIANT = 10           # cudadma_strided_transpose variant whose wavefront split follows the knob "transpose_split"
-# knob values = 100 x DMA wavefronts + 10 x compute wavefronts + tiles ahead, every compiled combination; with three DMA
-# wavefronts and one compute wavefront "tiles ahead" 3 to 7 stand for a tile requested in pieces: 3 halves (1.5 tiles), 5, 6
-# and 7 quarters (1.25, 1.5, 1.75 tiles) and 3 quarters (0.75) in flight; 8 (also with 2 + 2) for one tile in flight
-# without a pause: the next tile is requested when the loads of the current one have returned, before it goes to LDS
-TRANSPOSE_SPLITS = (111, 112, 121, 122, 141, 142, 211, 212, 221, 222, 241, 242, 311, 312, 321, 322, 411, 412, 421, 422, 441, 442,
-                    313, 314, 315, 316, 317, 228, 318)
+# knob values = 100 x DMA wavefronts + 10 x compute wavefronts + tiles ahead; transpose_splits() lists those the loaded library
+# holds (311, 312, 221, 222; a library built with -DHIPDMA_SWEEP_VARIANTS also every other split, "tiles ahead" 3 to 7 with three
+# DMA wavefronts and one compute wavefront for a tile requested in pieces: 3 halves (1.5 tiles), 5, 6 and 7 quarters (1.25, 1.5,
+# 1.75 tiles) and 3 quarters (0.75) in flight, and 8 for one tile in flight without a pause)
 TRANSPOSE_TWO_LDS_TILES_VARIANT = 11    # two LDS tiles and two CudaDMAStrided objects (manual double buffering in LDS)
 HALO_WIDE_TILES_VARIANT = 6            # cudadma_halo_stencil variant 0 with tiles of 64 x 16 cells
 GEMM_WARP_SPECIALISED_VARIANT = 7      # the cudadma_gemm_bf16 variant in which DMA wavefronts feed compute wavefronts
@@ -44,6 +42,19 @@ def num_variants(workload):
 
 def variant_name(workload, variant):
     return lib().cudadma_variant_name(workload, variant).decode()
+
+
+def variants(workload):
+    """The variant numbers of `workload` that the loaded library holds."""
+    return [v for v in range(num_variants(workload)) if variant_name(workload, v)]
+
+
+def transpose_splits():
+    """The values of the knob "transpose_split" that the loaded library holds."""
+    n = lib().cudadma_transpose_splits(None, 0)
+    codes = (ctypes.c_int * n)()
+    lib().cudadma_transpose_splits(codes, n)
+    return sorted(codes)
 
 
 def set_workgroups_per_cu(value):
@@ -160,15 +171,22 @@ BUFFERING_NONE, BUFFERING_SINGLE, BUFFERING_DOUBLE, BUFFERING_MANUAL = range(4)
 BUFFERING_NAMES = ("none", "single", "double", "manual")
 
 
-def perf_sequential(src, elmt_bytes, dma_wavefronts, buffering, loop_iters, workgroups, sums=None):
+LOAD_CACHE_ALL, LOAD_CACHE_STREAMING = 0, 2                 # CUDADMA_LOAD_CACHE_* of the C header
+STORE_WRITE_BACK, STORE_LDS, STORE_LDS_DIRECT = 0, 4, 5     # CUDADMA_STORE_*
+
+
+def perf_sequential(src, elmt_bytes, dma_wavefronts, buffering, loop_iters, workgroups, sums=None,
+                    load_qualifier=LOAD_CACHE_ALL, store_qualifier=STORE_WRITE_BACK):
     """The read-bandwidth probe of the sequential object (all parameters at run time).  Returns the
-    bytes one launch reads.  `sums` (uint32/int32, one zeroed word per workgroup) switches the checksum on."""
+    bytes one launch reads.  `sums` (uint32/int32, one zeroed word per workgroup) switches the checksum on.
+    The qualifiers are those of the objects' fully qualified calls; the defaults are the reference's."""
     if not (src.is_cuda and src.is_contiguous()):
         raise ValueError("src must be a contiguous CUDA tensor")
     if sums is not None and not (sums.is_cuda and sums.is_contiguous() and sums.element_size() == 4 and sums.numel() >= workgroups):
         raise ValueError("sums must hold one 32-bit word per workgroup")
     n = lib().cudadma_perf_sequential(_p(src), src.numel() * src.element_size(), _p(sums) if sums is not None else None,
-                                      elmt_bytes, dma_wavefronts, buffering, loop_iters, workgroups, _stream())
+                                      elmt_bytes, dma_wavefronts, buffering, loop_iters, workgroups,
+                                      load_qualifier, store_qualifier, _stream())
     if n < 0:
         check(int(n))
     return int(n)
@@ -192,6 +210,30 @@ def probe_memory(mode, src, dst, workgroups):
     if n < 0:
         check(int(n))
     return int(n)
+
+
+PATTERN_PROBE_MODES = ("gather_xor", "scatter", "tile_read", "tile_write", "tile_copy")
+
+
+def probe_pattern(mode, src, idx, out, workgroups, n_records=0):
+    """One launch of a yardstick with a pattern's own addresses (mode: index into PATTERN_PROBE_MODES or its name).
+    gather_xor: src = table, idx = int32 indices, out = one 128-byte row per 32 indices; scatter: src = records,
+    idx = int32 indices, out = table of n_records records; tile_read: src = n x n float matrix, out = 16 bytes per
+    workgroup; tile_write: out = n x n matrix.  Returns the algorithmic bytes moved."""
+    if isinstance(mode, str):
+        mode = PATTERN_PROBE_MODES.index(mode)
+    if mode in (0, 1):
+        _need(idx, torch.int32, "idx")
+        n = idx.numel()
+        if not n_records:
+            n_records = (src if mode == 0 else out).numel() * (src if mode == 0 else out).element_size() // 128
+    else:
+        n = (src if mode in (2, 4) else out).shape[0]
+    moved = lib().cudadma_probe_pattern(mode, _p(src) if src is not None else None, _p(idx) if idx is not None else None,
+                                        _p(out), n, n_records, int(workgroups), _stream())
+    if moved < 0:
+        check(int(moved))
+    return int(moved)
 
 
 def gemm_bf16(a, b, c, variant=0):

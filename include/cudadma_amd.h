@@ -223,8 +223,12 @@ enum {
   CUDADMA_WORKLOAD_SCATTER    = 5
 };
 int cudadma_num_variants(int workload);
-/* One-line description of a variant ("" when out of range). */
+/* One-line description of a variant ("" when out of range, and for a variant that this build of the library
+ * does not hold: kernels that only serve the parameter sweeps are compiled with make EXTRA=-DHIPDMA_SWEEP_VARIANTS). */
 const char* cudadma_variant_name(int workload, int variant);
+/* The values the knob "transpose_split" accepts in this build: writes up to `capacity` of them to `codes`
+ * (may be NULL) and returns how many there are. */
+int cudadma_transpose_splits(int* codes, int capacity);
 /* Tuning knob: workgroups resident per compute unit for the persistent grids
  * (0 restores each kernel's default).  Returns the previous value. */
 int cudadma_set_workgroups_per_cu(int value);
@@ -323,15 +327,31 @@ int cudadma_gemm_bf16(const uint16_t* d_a, const uint16_t* d_b, float* d_c, int 
  * Returns the bytes read (workgroups * elmt_bytes * loop_iters) or a negative CUDADMA_E*
  * code.  d_sums may be NULL (pure probe, nothing is written, as in the reference); otherwise
  * it holds one zero-initialised word per workgroup, to which the 32-bit words that arrived
- * in LDS are added. */
+ * in LDS are added.
+ * load_qualifier / store_qualifier are the template arguments of the objects' fully qualified calls
+ * (execute_dma<true, LOAD_QUAL, STORE_QUAL>, include/cudaDMAv2.h:1460-1562; the reference's probe uses the
+ * defaults, perf_sequential.cu:67): CUDADMA_LOAD_CACHE_ALL or _STREAMING (non-temporal loads), and how the
+ * bytes reach LDS: CUDADMA_STORE_WRITE_BACK (a generic store, the reference's default), CUDADMA_STORE_LDS
+ * (ds_write_b128) or CUDADMA_STORE_LDS_DIRECT (global_load_lds, no register staging).  Other values are refused
+ * with CUDADMA_ERANGE.  The objects' BYTES_PER_THREAD is 64: four dwordx4 in flight per DMA thread. */
 enum {
   CUDADMA_BUFFERING_NONE   = 0,  /* not warp-specialised, two workgroup barriers per element */
   CUDADMA_BUFFERING_SINGLE = 1,  /* one buffer, one object                                    */
   CUDADMA_BUFFERING_DOUBLE = 2,  /* two buffers, two objects on disjoint DMA wavefronts       */
   CUDADMA_BUFFERING_MANUAL = 3   /* two buffers, two objects on the same DMA wavefronts       */
 };
+/* values of enum CudaDMALoadQualifier / CudaDMAStoreQualifier of the device header (include/cudaDMAv2.h:50-63,
+ * plus the LDS stores this library adds) */
+enum {
+  CUDADMA_LOAD_CACHE_ALL       = 0,
+  CUDADMA_LOAD_CACHE_STREAMING = 2,
+  CUDADMA_STORE_WRITE_BACK     = 0,
+  CUDADMA_STORE_LDS            = 4,
+  CUDADMA_STORE_LDS_DIRECT     = 5
+};
 long long cudadma_perf_sequential(const void* d_src, size_t src_bytes, unsigned* d_sums, int elmt_bytes,
-                                  int dma_wavefronts, int buffering, int loop_iters, int workgroups, void* stream);
+                                  int dma_wavefronts, int buffering, int loop_iters, int workgroups,
+                                  int load_qualifier, int store_qualifier, void* stream);
 
 /* ---- streaming yardsticks ------------------------------------------------------------------
  * Kernels without LDS and without a DMA object (grid-stride dwordx4 accesses) that show what read-only,
@@ -350,6 +370,40 @@ enum {
   CUDADMA_PROBE_MODES                = 7
 };
 long long cudadma_probe_memory(int mode, const void* d_src, void* d_dst, size_t bytes, int workgroups, void* stream);
+
+/* ---- yardsticks with the patterns' own addresses -----------------------------------------------
+ * The memory accesses of the gather, the scatter and the tile transposition with nothing but loads and stores
+ * between them and memory (no LDS, no DMA object, no handshake), on the patterns' own buffers: what each pattern's
+ * figure is read against.  No counterpart in the reference.  `workgroups` workgroups of 256 threads share the work
+ * round-robin.  Returns the algorithmic bytes moved, or a negative CUDADMA_E* code.
+ *   GATHER_XOR  d_in: table of n_records records of 128 B; d_idx: n element indices (n a multiple of 32);
+ *               d_out[t][j] = xor over r < 32 of the 32-bit words table[d_idx[32 t + r]][j]: n / 32 rows of 128 B.
+ *               Moves what cudadma_gather_rowsum moves: n * 132 + n / 32 * 128 bytes.
+ *   SCATTER     d_in: n records of 128 B; d_out: table of n_records records; table[d_idx[i]] = records[i].
+ *               Moves what cudadma_scatter_copy moves: n * 260 bytes.
+ *   TILE_READ   d_in: n x n floats (n a multiple of 64); reads its 64 x 64 tiles in the order in which
+ *               cudadma_strided_transpose takes them (workgroup b: tiles b, b + workgroups, ...; tile t lies in
+ *               tile row t mod (n / 64), tile column t / (n / 64)); d_out receives 16 bytes per workgroup: the xor
+ *               of the 16-byte chunks of its tiles.  n * n * 4 bytes.
+ *   TILE_WRITE  d_out: n x n floats; writes, in the same order, the output tiles of the transposition (source tile
+ *               (row ty, column tx) lands on rows 64 tx.., columns 64 ty..); element (r, c) receives the 32-bit
+ *               pattern r * n + c.  n * n * 4 bytes.  d_in and d_idx are ignored.
+ *   TILE_COPY   both halves together without the transposition inside a tile:
+ *               d_out[64 tx + r][64 ty + c] = d_in[64 ty + r][64 tx + c].  2 * n * n * 4 bytes.
+ * Two knobs of cudadma_set_tuning shape TILE_WRITE and TILE_COPY: "probe_piece_bytes" (256, 512, 1024, 2048 or
+ * 4096; default 256, one tile) is the length of the piece of an output row that a workgroup writes per turn
+ * (TILE_COPY then reads pieces of as many source tiles per turn), "probe_xcd_group" = 1 gives the workgroups of
+ * one XCD neighbouring pieces instead of every eighth one. */
+enum {
+  CUDADMA_PATTERN_PROBE_GATHER_XOR = 0,
+  CUDADMA_PATTERN_PROBE_SCATTER    = 1,
+  CUDADMA_PATTERN_PROBE_TILE_READ  = 2,
+  CUDADMA_PATTERN_PROBE_TILE_WRITE = 3,
+  CUDADMA_PATTERN_PROBE_TILE_COPY  = 4,
+  CUDADMA_PATTERN_PROBE_MODES      = 5
+};
+long long cudadma_probe_pattern(int mode, const void* d_in, const int32_t* d_idx, void* d_out, size_t n,
+                                size_t n_records, int workgroups, void* stream);
 
 /* ---- known-answer cases for the first-generation class names -------------------------
  * One transfer per case by cudaDMASequential / cudaDMAStrided / cudaDMAIndirect as declared in

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Writes tests/golden/vectors.json: known answers for the oracle, produced WITHOUT the oracle.
 
-Every value below comes from pure-Python integer arithmetic, from numpy slicing, or from the
+Every value below comes from pure-Python integer arithmetic, from Python's math module (the Box-Muller draws), from numpy slicing, or from the
 expectation the reference's own test programs state (ramp input and exact comparison,
 cudaDMA_test_strided_v2.cu:561-563,659-677; the halo checker cudaDMA_test_halo.cu:91-164; the
 integer data of the sgemv driver, sgemv_dma.cu:752-771).  The reference itself is neither
@@ -10,6 +10,7 @@ imported nor executed.  tests/test_oracle.py compares oracle/liboracle.so with t
     python tests/golden/make_vectors.py
 """
 import json
+import math
 import os
 
 import numpy as np
@@ -65,6 +66,26 @@ def permutation_head(log2_n, seed, count):
     return out
 
 
+def normal_bf16_bits(seed, count):
+    """(index, bf16 bit pattern) of the first `count` draws of the Box-Muller generator whose value does not lie near
+    a rounding boundary of bf16: u1 = ((h(2i) >> 8) + 1) / 2^24, u2 = (h(2i+1) >> 8) / 2^24,
+    x = sqrt(-2 ln u1) * cos(2 pi u2) with Python's math module in double precision, rounded to binary32 and then to
+    bf16 (nearest even).  A draw is kept when the 16 bits that bf16 drops are at least 2^-8 of a bf16 step away from
+    the half-way point, so that neither the last bit of a library's log / cos nor the double rounding matters."""
+    out = []
+    i = 0
+    while len(out) < count:
+        u1 = ((hash32(seed, 2 * i) >> 8) + 1) / 16777216.0
+        u2 = (hash32(seed, 2 * i + 1) >> 8) / 16777216.0
+        x = math.sqrt(-2.0 * math.log(u1)) * math.cos(2.0 * math.pi * u2)
+        bits = int(np.float32(x).view(np.uint32))
+        dropped = bits & 0xFFFF
+        if abs(dropped - 0x8000) >= 0x100:
+            out.append([i, (bits + 0x7FFF + ((bits >> 16) & 1)) >> 16])
+        i += 1
+    return out
+
+
 def strided_ramp(e_floats, n, src_stride_floats, dst_stride_floats):
     """The reference's strided test: source float(i), every moved element compared exactly."""
     src = np.arange(n * src_stride_floats + e_floats, dtype=np.float32)
@@ -109,6 +130,7 @@ def main():
             {"dimx": dx, "dimy": dy, "radius": r, "corners": c, "pitch": p, "dst": halo_ring(dx, dy, r, c, p)}
             for (dx, dy, r, c, p) in ((8, 6, 2, 0, 16), (8, 6, 2, 1, 16), (32, 32, 4, 0, 48), (5, 3, 1, 1, 9))
         ],
+        "normal_bf16": {str(seed): normal_bf16_bits(seed, 192) for seed in (1005, 2005, 7)},
         "sgemv_reference_driver": {"n": 896, "m": 896, "alpha": 2, "y": sgemv_reference_driver(896, 896, 2)},
     }
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "vectors.json")

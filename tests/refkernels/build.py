@@ -1,4 +1,4 @@
-"""Builds oracle/_ref/libref_kernels.so: the device kernels of the reference's own v2 test programs, compiled from the
+"""Builds tests/refkernels/_build/libref_kernels.so: the device kernels of the reference's own v2 test programs, compiled from the
 reference tree where it lies (never copied into this repository) against this repository's cudaDMAv2.h, each behind
 a small launcher that does what the reference's run_experiment() does (one workgroup; for the warp-specialised kernels
 one compute wavefront of 64 threads plus DMA_THREADS DMA threads; dynamic LDS of the buffer size):
@@ -20,9 +20,10 @@ one compute wavefront of 64 threads plus DMA_THREADS DMA threads; dynamic LDS of
 The kernels take their parameters as template arguments named like the macros the reference's Makefiles pass
 (-DALIGNMENT=... and so on); here the template heads are left out and the macros of one parameter set are defined in
 front of the text, one translation unit per (program, parameter set).  Test infrastructure only: the GPU tests run
-these kernels and compare their output with the oracle's closed forms.
+these kernels (the code under test is this repository's header; the reference supplies the callers) and compare their
+output with the oracle's closed forms.
 
-    python oracle/build_ref_kernels.py          # needs /root/reference and hipcc; writes only into oracle/_ref/
+    python tests/refkernels/build.py          # needs /root/reference and hipcc; writes only into tests/refkernels/_build/
 """
 import concurrent.futures
 import os
@@ -33,9 +34,9 @@ import sys
 import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-ROOT = os.path.dirname(HERE)
+ROOT = os.path.dirname(os.path.dirname(HERE))
 REFERENCE_TESTS = "/root/reference/src/tests"
-OUT_DIR = os.path.join(HERE, "_ref")
+OUT_DIR = os.path.join(HERE, "_build")
 OUT = os.path.join(OUT_DIR, "libref_kernels.so")
 
 PROGRAMS = {

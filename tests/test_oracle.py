@@ -462,6 +462,16 @@ def test_golden_generators(O):
             assert [int(v) for v in got[:len(perm["head"])]] == perm["head"]
 
 
+def test_golden_normal_bf16(O):
+    """Box-Muller draws written by make_vectors.py with Python's math module (draws near a bf16 rounding boundary left
+    out): pins which hash feeds the radius and which the angle, the cosine, and the rounding to bf16."""
+    for seed, pairs in _golden()["normal_bf16"].items():
+        n = pairs[-1][0] + 1
+        got = np.empty(n, dtype=np.uint16)
+        O.oracle_fill_normal_bf16(ptr(got), n, int(seed))
+        assert [[i, int(got[i])] for i, _ in pairs] == pairs
+
+
 def test_golden_strided_ramp_and_halo_ring(O):
     g = _golden()
     for case in g["strided_ramp"]:

@@ -1,5 +1,5 @@
-"""The reference's own device kernels on the GPU.  oracle/build_ref_kernels.py compiles them from the reference tree against
-this repository's cudaDMAv2.h / cudaDMA.h into oracle/_ref/libref_kernels.so (not kept in the repository; it travels with
+"""The reference's own device kernels on the GPU.  tests/refkernels/build.py compiles them from the reference tree against
+this repository's cudaDMAv2.h / cudaDMA.h into tests/refkernels/_build/libref_kernels.so (not kept in the repository; it travels with
 the built libraries): the special_xfer_* / nonspec_xfer_* kernels of the v2 test programs
 (src/tests/test_{sequential,strided,indirect}/cudaDMA_test_*_v2.cu), the halo test kernel, the saxpy, sgemv and stencil
 examples and the read-bandwidth probe.  The test kernels run as the reference's run_experiment() runs them: input float(i)
@@ -14,7 +14,7 @@ import numpy as np
 import pytest
 import torch
 
-from oracle import build_ref_kernels as ref
+from tests.refkernels import build as ref
 from tests import oracle_lib as ol
 from tests.oracle_lib import ptr
 
@@ -26,7 +26,7 @@ _UNITS = [(p, s) for p in ref.PROGRAMS for s, m in ref.PARAMETER_SETS.items() if
 @pytest.fixture(scope="module")
 def kernels():
     if not os.path.exists(ref.OUT):
-        pytest.skip(f"{ref.OUT} has not been built (python oracle/build_ref_kernels.py, where the reference tree is present)")
+        pytest.skip(f"{ref.OUT} has not been built (python tests/refkernels/build.py, where the reference tree is present)")
     return ctypes.CDLL(ref.OUT)
 
 

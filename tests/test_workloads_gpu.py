@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _variants(w):
-    return range(wl.num_variants(w))
+    return wl.variants(w)                # the variant numbers the loaded library holds (no GPU needed)
 
 
 # ------------------------------------------------------------------ generators
@@ -146,7 +146,7 @@ def test_strided_transpose_under_every_tuning(device, variant, band, workgroups)
     assert np.array_equal(dst.cpu().numpy().view(np.uint32), np.ascontiguousarray(host.T).view(np.uint32))
 
 
-_SPLITS = list(wl.TRANSPOSE_SPLITS)
+_SPLITS = wl.transpose_splits()              # loads the library at collection time (no GPU needed)
 
 
 @pytest.mark.parametrize("split", _SPLITS)
@@ -325,12 +325,25 @@ def test_scatter_argument_checks(device):
 STENCIL_RTOL = 1e-5       # benchmark config 4: fp32 within 1e-5 relative of the host reference
 
 
+def _wide_tiles_refuse(device, variant, shape):
+    """Variants 6 and 7 use tiles of 64 x 16 cells: a grid they do not tile is refused on the host, before any launch,
+    and the output buffer stays as it was."""
+    nx, ny, nz = shape
+    p = 2 * wl.STENCIL_RADIUS
+    d_in = torch.zeros((nz + p, ny + p, nx + p), dtype=torch.float32, device=device)
+    d_out = torch.full((nz, ny, nx), 7.0, dtype=torch.float32, device=device)
+    with pytest.raises(cd.CudaDMAError, match="multiple of"):
+        wl.halo_stencil(d_in, d_out, variant)
+    torch.cuda.synchronize()
+    assert bool((d_out == 7.0).all())
+
+
 @pytest.mark.parametrize("variant", _variants(wl.HALO))
 @pytest.mark.parametrize("shape", [(32, 32, 5), (64, 96, 70), (128, 64, 130)])
 def test_halo_stencil_small(device, variant, shape):
     nx, ny, nz = shape
     if variant >= 6 and (nx % 64 or ny % 16):
-        pytest.skip("variants 6 and 7 use tiles of 64 x 16 cells")
+        return _wide_tiles_refuse(device, variant, shape)
     p = 2 * wl.STENCIL_RADIUS
     g = ol.uniform((nx + p) * (ny + p) * (nz + p), 1004).reshape(nz + p, ny + p, nx + p)
     want = np.empty((nz, ny, nx), dtype=np.float32)
@@ -355,7 +368,7 @@ def test_halo_stencil_under_every_tuning(device, variant, ring, remap, shape):
     result does not depend on them."""
     nx, ny, nz = shape
     if variant >= 6 and (nx % 64 or ny % 16):
-        pytest.skip("variants 6 and 7 use tiles of 64 x 16 cells")
+        return _wide_tiles_refuse(device, variant, shape)
     p = 2 * wl.STENCIL_RADIUS
     g = ol.uniform((nx + p) * (ny + p) * (nz + p), 4004).reshape(nz + p, ny + p, nx + p)
     want = np.empty((nz, ny, nx), dtype=np.float32)
@@ -436,6 +449,21 @@ def test_device_normal_bf16_generator_matches_the_host_statement(device):
         assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16), want)
 
 
+def test_device_normal_bf16_generator_matches_the_golden_vectors(device):
+    """The same generator against tests/golden/vectors.json (Box-Muller draws written with Python's math module, without
+    the oracle; draws near a bf16 rounding boundary left out)."""
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "vectors.json")) as f:
+        golden = json.load(f)["normal_bf16"]
+    for seed, pairs in golden.items():
+        n = pairs[-1][0] + 1
+        got = wl.fill_normal_bf16(torch.empty(n, dtype=torch.bfloat16, device=device), int(seed))
+        torch.cuda.synchronize()
+        bits = got.view(torch.int16).cpu().numpy().view(np.uint16)
+        assert [[i, int(bits[i])] for i, _ in pairs] == pairs
+
+
 def _bf16_inputs(m, n, k):
     a = np.empty(m * k, dtype=np.uint16)
     b = np.empty(k * n, dtype=np.uint16)
@@ -445,7 +473,7 @@ def _bf16_inputs(m, n, k):
     return a.reshape(m, k), b.reshape(k, n)
 
 
-@pytest.mark.parametrize("variant", range(10))
+@pytest.mark.parametrize("variant", _variants(wl.GEMM))
 @pytest.mark.parametrize("shape", [(128, 128, 128), (256, 384, 256), (512, 512, 512), (768, 256, 384), (256, 128, 128),
                                    (1024, 256, 896), (256, 256, 128), (256, 512, 640), (768, 1280, 640)])
 def test_gemm_small(device, shape, variant):
@@ -475,7 +503,7 @@ def test_gemm_small(device, shape, variant):
     assert float(np.max(np.abs(got - want))) <= 1e-4 * scale * np.sqrt(k)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("variant", _variants(wl.GEMM))
 def test_gemm_full_size(device, variant):
     m = n = k = 4096
     a, b = _bf16_inputs(m, n, k)
@@ -503,6 +531,33 @@ def test_gemm_rejects_ragged_shapes(device):
         wl.gemm_bf16(a, b, c)
 
 
+def test_variants_the_library_does_not_hold_are_refused(device):
+    """Kernels that only serve the parameter sweeps are left out of the library unless it is built with
+    -DHIPDMA_SWEEP_VARIANTS: their variant numbers stay reserved, have no name and are refused before any launch."""
+    src = torch.zeros((256, 256), dtype=torch.float32, device=device)
+    dst = torch.full_like(src, 7.0)
+    for v in set(range(wl.num_variants(wl.STRIDED))) - set(wl.variants(wl.STRIDED)):
+        with pytest.raises(cd.CudaDMAError, match="HIPDMA_SWEEP_VARIANTS"):
+            wl.strided_transpose(src, dst, v)
+    for v in set(range(wl.num_variants(wl.HALO))) - set(wl.variants(wl.HALO)):
+        with pytest.raises(cd.CudaDMAError, match="HIPDMA_SWEEP_VARIANTS"):
+            wl.halo_stencil(torch.zeros((40, 40, 40), dtype=torch.float32, device=device),
+                            torch.zeros((32, 32, 32), dtype=torch.float32, device=device), v)
+    a = torch.zeros((256, 256), dtype=torch.bfloat16, device=device)
+    for v in set(range(wl.num_variants(wl.GEMM))) - set(wl.variants(wl.GEMM)):
+        with pytest.raises(cd.CudaDMAError, match="HIPDMA_SWEEP_VARIANTS"):
+            wl.gemm_bf16(a, a, torch.zeros((256, 256), dtype=torch.float32, device=device), v)
+    torch.cuda.synchronize()
+    assert bool((dst == 7.0).all())
+    for split in {311, 312, 221, 222, 313, 228, 411} - set(wl.transpose_splits()):
+        wl.set_tuning("transpose_split", split)
+        try:
+            with pytest.raises(cd.CudaDMAError, match="HIPDMA_SWEEP_VARIANTS"):
+                wl.strided_transpose(src, dst, wl.TRANSPOSE_SPLIT_VARIANT)
+        finally:
+            wl.set_tuning("transpose_split", 0)
+
+
 # ------------------------------------------------------------------ streaming yardsticks
 @pytest.mark.parametrize("workgroups", [1, 7, 512])
 def test_yardsticks_move_what_they_say(device, workgroups):
@@ -522,7 +577,69 @@ def test_yardsticks_move_what_they_say(device, workgroups):
             assert torch.equal(dst.view(torch.int32), src.view(torch.int32))
 
 
+@pytest.mark.parametrize("workgroups", [1, 5, 300])
+def test_pattern_yardsticks_move_what_they_say(device, workgroups):
+    """The yardsticks with the patterns' own addresses, bit for bit against numpy: the xor of the gathered records per tile
+    of 32 indices, the scatter by a permutation, the per-workgroup xor of the transposition's source tiles and the
+    transposition's destination tiles written in its order."""
+    recs, n_idx = 4096, 32 * 96
+    table = ol.uniform(recs * 32, 1003)
+    idx = ol.indices(n_idx, recs, 1003)
+    d_out = torch.zeros(n_idx // 32 * 32, dtype=torch.int32, device=device)
+    print(f"pattern yardstick gather_xor workgroups {workgroups}", flush=True)
+    moved = wl.probe_pattern("gather_xor", torch.from_numpy(table).to(device), torch.from_numpy(idx).to(device), d_out, workgroups)
+    torch.cuda.synchronize()
+    assert moved == n_idx * 132 + n_idx // 32 * 128
+    want = np.bitwise_xor.reduce(table.view(np.uint32).reshape(recs, 32)[idx].reshape(-1, 32, 32), axis=1)
+    assert np.array_equal(d_out.cpu().numpy().view(np.uint32).reshape(-1, 32), want)
+
+    log2 = 12
+    records = ol.uniform((1 << log2) * 32, 1006)
+    perm = ol.permutation(log2, 1006)
+    d_table = torch.full(((1 << log2) * 32,), float("nan"), dtype=torch.float32, device=device)
+    print(f"pattern yardstick scatter workgroups {workgroups}", flush=True)
+    moved = wl.probe_pattern("scatter", torch.from_numpy(records).to(device), torch.from_numpy(perm).to(device), d_table, workgroups)
+    torch.cuda.synchronize()
+    assert moved == (1 << log2) * 260
+    want = np.empty_like(records).reshape(-1, 32)
+    want[perm] = records.reshape(-1, 32)
+    assert np.array_equal(d_table.cpu().numpy().view(np.uint32), want.reshape(-1).view(np.uint32))
+
+    n = 320                                                       # 5 x 5 tiles
+    host = ol.uniform(n * n, 1002).reshape(n, n)
+    d_x = torch.zeros(workgroups * 4, dtype=torch.int32, device=device)
+    print(f"pattern yardstick tile_read workgroups {workgroups}", flush=True)
+    moved = wl.probe_pattern("tile_read", torch.from_numpy(host).to(device), None, d_x, workgroups)
+    torch.cuda.synchronize()
+    assert moved == n * n * 4
+    tps = n // 64
+    want = np.zeros((workgroups, 4), dtype=np.uint32)
+    words = host.view(np.uint32)
+    for t in range(tps * tps):
+        tx, ty = t // tps, t % tps
+        tile = words[ty * 64:(ty + 1) * 64, tx * 64:(tx + 1) * 64].reshape(-1, 4)
+        want[t % workgroups] ^= np.bitwise_xor.reduce(tile, axis=0)
+    assert np.array_equal(d_x.cpu().numpy().view(np.uint32).reshape(-1, 4), want)
+
+    d_m = torch.zeros((n, n), dtype=torch.int32, device=device)
+    print(f"pattern yardstick tile_write workgroups {workgroups}", flush=True)
+    moved = wl.probe_pattern("tile_write", None, None, d_m, workgroups)
+    torch.cuda.synchronize()
+    assert moved == n * n * 4
+    assert np.array_equal(d_m.cpu().numpy().reshape(-1), np.arange(n * n, dtype=np.int32))
+
+
 def test_yardstick_argument_checks(device):
+    t = torch.zeros(64 * 64, dtype=torch.float32, device=device)
+    i = torch.zeros(64, dtype=torch.int32, device=device)
+    with pytest.raises(cd.CudaDMAError, match="multiple of 32"):
+        wl.probe_pattern("gather_xor", t, i[:40], t.clone(), 4)
+    with pytest.raises(cd.CudaDMAError, match="multiple of 64"):
+        wl.probe_pattern("tile_write", None, None, torch.zeros((40, 40), dtype=torch.float32, device=device), 4)
+    with pytest.raises(cd.CudaDMAError, match="workgroups"):
+        wl.probe_pattern("scatter", t, i, t.clone(), 0)
+    with pytest.raises(cd.CudaDMAError):
+        wl.probe_pattern(len(wl.PATTERN_PROBE_MODES), t, i, t.clone(), 4)
     t = torch.zeros(64 * 64, dtype=torch.float32, device=device)
     with pytest.raises(cd.CudaDMAError):
         wl.probe_memory(len(wl.PROBE_MODES), t, t.clone(), 4)
@@ -533,18 +650,27 @@ def test_yardstick_argument_checks(device):
 
 
 # ------------------------------------------------------------------ read-bandwidth probe (perf_sequential)
+_PROBE_QUALIFIERS = [(wl.LOAD_CACHE_ALL, wl.STORE_WRITE_BACK), (wl.LOAD_CACHE_STREAMING, wl.STORE_LDS), (wl.LOAD_CACHE_ALL, wl.STORE_LDS),
+                     (wl.LOAD_CACHE_ALL, wl.STORE_LDS_DIRECT), (wl.LOAD_CACHE_STREAMING, wl.STORE_LDS_DIRECT),
+                     (wl.LOAD_CACHE_STREAMING, wl.STORE_WRITE_BACK)]
+
+
+@pytest.mark.parametrize("qualifiers", _PROBE_QUALIFIERS, ids=lambda q: f"load{q[0]}-store{q[1]}")
 @pytest.mark.parametrize("buffering", range(4))
 @pytest.mark.parametrize("elmt,waves,loops,groups", [(32, 1, 1, 3), (48, 2, 5, 7), (4096, 2, 8, 64), (16384, 4, 3, 33),
                                                      (2064, 7, 2, 5), (16, 1, 9, 2)])
-def test_perf_sequential_checksum(device, buffering, elmt, waves, loops, groups):
-    """Every byte of every element reaches LDS: per-workgroup sum of the 32-bit words, modulo 2^32."""
+def test_perf_sequential_checksum(device, buffering, elmt, waves, loops, groups, qualifiers):
+    """Every byte of every element reaches LDS: per-workgroup sum of the 32-bit words, modulo 2^32, for every
+    compiled pair of load and store qualifier (the reference's defaults, non-temporal loads, ds_write_b128,
+    global_load_lds)."""
+    lq, sq = qualifiers
     total = groups * elmt * loops
     rng = np.random.default_rng(elmt + waves)
     words = rng.integers(0, 2 ** 32, size=total // 4 + 64, dtype=np.uint64).astype(np.uint32)
     src = torch.from_numpy(words.view(np.int32)).to(device)
     sums = torch.zeros(groups, dtype=torch.int32, device=device)
-    print(f"perf_sequential elmt {elmt} waves {waves} loops {loops} groups {groups} buffering {buffering}", flush=True)
-    n = wl.perf_sequential(src, elmt, waves, buffering, loops, groups, sums)
+    print(f"perf_sequential elmt {elmt} waves {waves} loops {loops} groups {groups} buffering {buffering} qualifiers {qualifiers}", flush=True)
+    n = wl.perf_sequential(src, elmt, waves, buffering, loops, groups, sums, lq, sq)
     torch.cuda.synchronize()
     assert n == total
     want = words[:total // 4].reshape(groups, -1).astype(np.uint64).sum(axis=1).astype(np.uint32)
@@ -559,3 +685,7 @@ def test_perf_sequential_argument_checks(device):
         wl.perf_sequential(src, 4096, 1, 1, 2, 1)
     with pytest.raises(cd.CudaDMAError, match="unknown buffering"):
         wl.perf_sequential(src, 64, 1, 4, 1, 1)
+    with pytest.raises(cd.CudaDMAError, match="the probe is compiled for"):
+        wl.perf_sequential(src, 64, 1, 1, 1, 1, None, 1, wl.STORE_LDS)        # LOAD_CACHE_GLOBAL is not among them
+    with pytest.raises(cd.CudaDMAError, match="the probe is compiled for"):
+        wl.perf_sequential(src, 64, 1, 1, 1, 1, None, wl.LOAD_CACHE_ALL, 2)       # nor a store to global memory
