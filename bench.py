@@ -38,8 +38,8 @@ COUNTERS_JSON = os.path.join(ROOT, "profiles", "counters.json")
 
 # name -> (kernel the pattern launches, as rocprofv3 names it; used by cudadma_amd.profile_summary)
 PATTERN_KERNELS = {
-    "strided": "transpose_split<3, 1, 1>",
-    "strided_settled": "transpose_split<3, 1, 1>",
+    "strided": "transpose_split<3, 1, 1, false>",
+    "strided_settled": "transpose_split<3, 1, 1, false>",
     "sequential_read_probe": "perf_manual<2, 4>",
     "strided_even_split": "transpose_single<true, true>",
     "strided_two_lds_tiles": "transpose_manual_double<272, false>",

@@ -146,6 +146,7 @@ _WORKLOAD_SIGNATURES = {
     "cudadma_gather_rowsum": [_vp, _vp, _vp, _cs, _cs, _ci, _vp],
     "cudadma_halo_stencil": [_vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cudadma_gemm_bf16": [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
+    "cudadma_probe_clock": [_vp, _ci, _vp],
     "cudadma_selftest_bounded_wait": [_vp, _vp],
     "cudadma_selftest_split_wait": [_vp, _ci, _vp],
     "cudadma_selftest_global_handoff": [_vp, _vp, _ci, _vp],

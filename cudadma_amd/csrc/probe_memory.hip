@@ -53,7 +53,32 @@ probe_copy(const vec4_t* __restrict__ in, vec4_t* __restrict__ out, const size_t
   }
 }
 
+__global__ void __launch_bounds__(64)
+probe_clock(unsigned long long* __restrict__ ticks, const int iterations)
+{
+  float x = 1.0f + 1e-7f * threadIdx.x;
+  const unsigned long long t0 = __builtin_readcyclecounter();           // s_memtime: shader clock
+  const unsigned long long r0 = __builtin_amdgcn_s_memrealtime();       // constant 100 MHz
+  for (int i = 0; i < iterations; ++i) x = __builtin_fmaf(x, 1.0000001f, 1e-9f);
+  asm volatile("" :: "v"(x));                                           // the chain has to be finished before the second reading
+  const unsigned long long t1 = __builtin_readcyclecounter();
+  const unsigned long long r1 = __builtin_amdgcn_s_memrealtime();
+  if (threadIdx.x == 0) {
+    ticks[0] = t1 - t0;
+    ticks[1] = r1 - r0;
+  }
+}
+
 }  // namespace
+
+extern "C" int cudadma_probe_clock(uint64_t* d_ticks, int iterations, void* stream)
+{
+  CUDADMA_REQUIRE(d_ticks != nullptr && cudadma_host::aligned_to(d_ticks, 8), "d_ticks must be an 8-byte aligned device pointer");
+  CUDADMA_REQUIRE(iterations > 0, "iterations must be positive");
+  hipLaunchKernelGGL(probe_clock, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)d_ticks, iterations);
+  CUDADMA_HIP_CHECK(hipGetLastError());
+  return CUDADMA_OK;
+}
 
 extern "C" long long cudadma_probe_memory(int mode, const void* d_src, void* d_dst, size_t bytes, int workgroups,
                                           void* stream)

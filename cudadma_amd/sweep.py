@@ -9,6 +9,9 @@ point; here the variants are compiled in and the occupancy is a run-time knob.
     python -m cudadma_amd.sweep transpose_split              # DMA : compute wavefronts x tiles ahead x workgroups per CU
     python -m cudadma_amd.sweep transpose_walk               # tile order x workgroup count, one-tile and two-tile kernels
     python -m cudadma_amd.sweep placement                    # 1 GiB copies against the distance between source and destination
+    python -m cudadma_amd.sweep placement_fine               # the copy yardstick alone against 51 distances from 0 to 256 MiB
+    python -m cudadma_amd.sweep pattern_yardsticks           # the patterns' own addresses without LDS or objects, next to the patterns
+    python -m cudadma_amd.sweep settle                       # the first 80 launches after an idle second, one by one, with the shader clock
     python -m cudadma_amd.sweep queue_depth --config NAME    # one launch shape of QUEUE_CONFIGS, a few launches: the process to put
                                                              # under rocprofv3 --pmc when asking what more work in flight costs
 """
@@ -187,6 +190,107 @@ def main(argv=None):
                     ms = _time(fn, args.steps, settle_ms=15.0)
                     cells.append(f"{ms:.4f} ({2 * m * 4 / ms / 1e6 / PEAK_GBS * 100:4.1f}%)")
                 print(f"+{off:>9d} B:  " + "   ".join(cells), flush=True)
+            del pool
+        elif name == "placement_fine":
+            m = (1 << 30) // 4
+            pool = torch.empty(2 * m + (256 << 20) // 4, device=dev)
+            src = wl.fill_uniform(pool[:m], 1001)
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            K, M = 1 << 10, 1 << 20
+            offs = [0, 256, 512, 1 * K, 2 * K, 3 * K, 4 * K, 6 * K, 8 * K, 12 * K, 16 * K, 20 * K, 24 * K, 28 * K, 32 * K, 40 * K, 48 * K, 56 * K,
+                    64 * K, 80 * K, 96 * K, 128 * K, 192 * K, 256 * K, 384 * K, 512 * K, 768 * K, 1 * M, 1536 * K, 2 * M, 3 * M, 4 * M, 5 * M, 6 * M,
+                    8 * M, 10 * M, 12 * M, 14 * M, 16 * M, 20 * M, 24 * M, 28 * M, 32 * M, 40 * M, 48 * M, 56 * M, 64 * M, 96 * M, 128 * M, 192 * M,
+                    256 * M]
+            print("# copy_nontemporal yardstick, destination - source = 1 GiB + offset: % of 8 TB/s at 3 / 4 / 6 workgroups per compute unit")
+            for off in offs:
+                dst = pool[m + off // 4: 2 * m + off // 4]
+                cells = []
+                for wg in (3, 4, 6):
+                    ms = _time(lambda: wl.probe_memory("copy_nontemporal", src, dst, cus * wg), args.steps, settle_ms=8.0)
+                    cells.append(f"{2 * m * 4 / ms / 1e6 / PEAK_GBS * 100:5.1f}")
+                print(f"+{off:>10d} B ({off / K:10.2f} KiB):  " + "  ".join(cells), flush=True)
+            del pool
+        elif name == "pattern_yardsticks":
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            pct = lambda nb, ms: f"{nb / ms / 1e6 / PEAK_GBS * 100:5.1f}"
+            n_idx = 32 << 20
+            for recs in (4 << 20, 32 << 20):
+                table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1003)
+                idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=dev), recs, 1003)
+                out = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, device=dev)
+                shapes = (2, 3, 4, 6, 8)
+                nb = n_idx * 132 + out.numel() * 4
+                cells = [pct(nb, _time(lambda: wl.probe_pattern("gather_xor", table, idx, out, cus * wg), args.steps, settle_ms=10.0)) for wg in shapes]
+                dma = pct(nb, _time(lambda: wl.gather_rowsum(table, idx, out, 0), args.steps, settle_ms=10.0))
+                print(f"gather, table of {recs >> 20} Mi records: records read straight into registers " + " / ".join(cells) +
+                      f" % of 8 TB/s at {shapes} workgroups per CU; cudadma_gather_rowsum {dma} %", flush=True)
+                del table, idx, out
+            recs = 4 << 20
+            records = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1006)
+            perm = wl.fill_permutation(torch.empty(recs, dtype=torch.int32, device=dev), 1006)
+            table = torch.empty(recs * wl.REC_FLOATS, device=dev)
+            shapes = (1, 2, 3, 4, 6, 8)
+            cells = [pct(recs * 260, _time(lambda: wl.probe_pattern("scatter", records, perm, table, cus * wg), args.steps, settle_ms=10.0)) for wg in shapes]
+            dma = pct(recs * 260, _time(lambda: wl.scatter_copy(records, perm, table, 0), args.steps, settle_ms=10.0))
+            print(f"scatter of {recs >> 20} Mi records: records written straight from registers " + " / ".join(cells) +
+                  f" % at {shapes} workgroups per CU; cudadma_scatter_copy {dma} %", flush=True)
+            del records, perm, table
+            n = 16384
+            pool = torch.empty(2 * n * n, device=dev)
+            src = wl.fill_uniform(pool[:n * n], 1002).view(n, n)
+            dst = pool[n * n:].view(n, n)
+            sink = torch.empty(8 * cus * 4, device=dev)
+            shapes = (0.5, 1, 1.5, 2, 3, 4)
+            cells = [pct(n * n * 4, _time(lambda: wl.probe_pattern("tile_read", src, None, sink, int(cus * wg)), args.steps, settle_ms=10.0)) for wg in shapes]
+            print("transposition, its source tiles read alone: " + " / ".join(cells) + f" % at {shapes} workgroups per CU", flush=True)
+            for mode, shapes in (("tile_write", (0.5, 1, 1.5, 2, 3, 4)), ("tile_copy", (1, 2, 3, 4, 6, 8))):
+                for xg in (0, 1):
+                    wl.set_tuning("probe_xcd_group", xg)
+                    for piece in (256, 512, 1024, 2048, 4096):
+                        wl.set_tuning("probe_piece_bytes", piece)
+                        nb = n * n * 4 * (2 if mode == "tile_copy" else 1)
+                        s_ = src if mode == "tile_copy" else None
+                        cells = [pct(nb, _time(lambda: wl.probe_pattern(mode, s_, None, dst, int(cus * wg)), args.steps, settle_ms=10.0)) for wg in shapes]
+                        print(f"transposition, {mode} in pieces of {piece:4d} B, XCD grouping {xg}: " + " / ".join(cells) +
+                              f" % at {shapes} workgroups per CU", flush=True)
+            wl.set_tuning("probe_piece_bytes", 0)
+            wl.set_tuning("probe_xcd_group", 0)
+            ms = _time(lambda: wl.strided_transpose(src, dst, 0), args.steps, settle_ms=20.0)
+            print(f"cudadma_strided_transpose variant 0: {pct(2 * n * n * 4, ms)} %", flush=True)
+            del pool
+        elif name == "settle":
+            # what the first launches after an idle phase cost, and whether the shader clock has anything to do with it: after a
+            # second without GPU work, launches of one kernel back to back, each between two events, a clock probe after each
+            import time
+            n = 16384
+            pool = torch.empty(2 * n * n, device=dev)
+            src = wl.fill_uniform(pool[:n * n], 1002).view(n, n)
+            dst = pool[n * n:].view(n, n)
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            kernels = (("transposition (variant 0)", lambda: wl.strided_transpose(src, dst, 0), 2 * n * n * 4),
+                       ("copy_nontemporal yardstick, 4 workgroups per CU", lambda: wl.probe_memory("copy_nontemporal", src.view(-1), dst.view(-1), cus * 4), 2 * n * n * 4),
+                       ("read_nontemporal yardstick, 1.5 workgroups per CU", lambda: wl.probe_memory("read_nontemporal", src.view(-1), None, int(cus * 1.5)), n * n * 4))
+            launches = 80
+            for label, fn, nbytes in kernels:
+                ticks = torch.zeros((launches, 2), dtype=torch.int64, device=dev)
+                events = [torch.cuda.Event(enable_timing=True) for _ in range(launches + 1)]
+                torch.cuda.synchronize()
+                time.sleep(1.0)
+                events[0].record()
+                for i in range(launches):
+                    fn()
+                    events[i + 1].record()
+                    wl.probe_clock(ticks[i], 2048)          # a few microseconds
+                torch.cuda.synchronize()
+                t = ticks.cpu()
+                print(f"# {label}: launch, ms since the first launch, ms of the launch (incl. the clock probe behind it), % of 8 TB/s, shader clock in MHz")
+                at = 0.0
+                for i in range(launches):
+                    ms = events[i].elapsed_time(events[i + 1])
+                    mhz = 100.0 * t[i, 0].item() / max(1, t[i, 1].item())
+                    if i < 12 or i % 4 == 0:
+                        print(f"{i:3d}  {at:8.3f}  {ms:.4f}  {nbytes / ms / 1e6 / PEAK_GBS * 100:5.1f}  {mhz:7.0f}", flush=True)
+                    at += ms
             del pool
         elif name == "queue_depth":
             if args.config not in QUEUE_CONFIGS:

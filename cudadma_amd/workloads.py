@@ -212,6 +212,13 @@ def probe_memory(mode, src, dst, workgroups):
     return int(n)
 
 
+def probe_clock(ticks, iterations=1 << 16):
+    """One launch of the clock probe; `ticks`: int64 CUDA tensor of two elements (shader-clock ticks, 100 MHz ticks)."""
+    _need(ticks, torch.int64, "ticks")
+    check(lib().cudadma_probe_clock(_p(ticks), int(iterations), _stream()))
+    return ticks
+
+
 PATTERN_PROBE_MODES = ("gather_xor", "scatter", "tile_read", "tile_write", "tile_copy")
 
 

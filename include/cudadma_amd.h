@@ -371,6 +371,13 @@ enum {
 };
 long long cudadma_probe_memory(int mode, const void* d_src, void* d_dst, size_t bytes, int workgroups, void* stream);
 
+/* Clock probe: one wavefront runs `iterations` dependent fused multiply-adds between two readings of the shader clock
+ * counter (s_memtime) and of the constant 100 MHz counter (s_memrealtime).  d_ticks[0] and d_ticks[1] receive the two
+ * differences: d_ticks[0] / d_ticks[1] x 100 MHz is the shader clock during the launch, and d_ticks[0] / iterations
+ * the cycles per dependent instruction (a constant of the chip).  Used to tell a clock ramp from a memory-side effect
+ * when the first launches after an idle phase run slow.  No counterpart in the reference. */
+int cudadma_probe_clock(uint64_t* d_ticks, int iterations, void* stream);
+
 /* ---- yardsticks with the patterns' own addresses -----------------------------------------------
  * The memory accesses of the gather, the scatter and the tile transposition with nothing but loads and stores
  * between them and memory (no LDS, no DMA object, no handshake), on the patterns' own buffers: what each pattern's

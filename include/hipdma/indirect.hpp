@@ -199,6 +199,10 @@ private:
     HIPDMA_ASSERT((alt % ALIGNMENT) == 0);
     m_grid.init(ALIGNMENT, MAX_LDS, e, n, t, int(threadIdx.x) - start);
     m_dense_stride = (alt > e) ? alt : e;
+    // a *_prefetched() call that was not preceded by prefetch_index() then addresses record 0 instead of whatever
+    // the registers held (the stores vanish from kernels that never use the prefetched calls)
+#pragma unroll
+    for (int k = 0; k < MAX_LDS; ++k) m_idx_next[k] = 0;
   }
 
   template<int STORE_QUAL>

@@ -228,13 +228,18 @@ def test_global_memory_crosses_the_handshake(device, entry):
     """Global memory written before a signal is seen after the matching wait, in both directions: the compute
     wavefront produces the source in global memory, the DMA wavefronts move it global -> global, the compute
     wavefront reads the destination (bar.sync / bar.arrive order all memory, include/cudaDMAv2.h:65-75).
-    Both builds of the fences must pass on this chip: they wait the same way."""
+    The default build (fences over all address spaces) is the contract and must deliver every word.  The build with
+    fences over LDS only promises nothing about global memory (its fences leave the compiler free to move the global
+    accesses across the hand-off, although on this chip both builds wait the same way): for it the test only asks that
+    the kernel ends with an empty failure record."""
     import ctypes
     scratch = torch.zeros(4096, dtype=torch.int32, device=device)
     wrong = torch.zeros(1, dtype=torch.int32, device=device)
     cd._lib.check(getattr(cd.lib(), entry)(ctypes.c_void_p(scratch.data_ptr()), ctypes.c_void_p(wrong.data_ptr()), 300, None))
     torch.cuda.synchronize()
-    assert wrong.item() == 0
+    assert cd.device_status(clear=False) == (0, 0)
+    if not entry.endswith("_lds_only"):
+        assert wrong.item() == 0
 
 
 def test_split_wait_sees_every_phase(device):
