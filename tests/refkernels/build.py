@@ -24,6 +24,7 @@ these kernels (the code under test is this repository's header; the reference su
 output with the oracle's closed forms.
 
     python tests/refkernels/build.py          # needs /root/reference and hipcc; writes only into tests/refkernels/_build/
+    CUDADMA_REFKERNEL_DRAWS=84 python tests/refkernels/build.py      # plus 84 seeded draws from the reference's random sweep
 """
 import concurrent.futures
 import os
@@ -54,6 +55,47 @@ PARAMETER_SETS = {
     "a16_e6000_t64_n2": dict(ALIGNMENT=16, ALIGN_OFFSET=0, BYTES_PER_THREAD=16, BYTES_PER_ELMT=6000, DMA_THREADS=64, NUM_ELMTS=2),
 }
 COMPUTE_THREADS = 64          # one compute wavefront, where the reference launches one warp
+MANIFEST = os.path.join(OUT_DIR, "parameter_sets.json")       # the sets the library on disk was built with
+LDS_BUDGET = 60 * 1024        # bytes of dynamic LDS a drawn set may ask for (64 KB is what a launch gets without more ado)
+
+
+def drawn_parameter_sets(count, seed=20240517):
+    """`count` further parameter sets drawn the way the reference's own random sweep draws them
+    (src/tests/test_strided/param_sweep_v2.py:50-71): ALIGNMENT from {4, 8, 16}, an offset in floats that keeps it,
+    BYTES_PER_THREAD = ALIGNMENT x 1..8, an element of |N(256, 256)| floats, 1..32 elements, DMA thread groups of 1..8
+    wavefronts of 64 (the reference: 1..16 warps of 32).  Draws whose buffer would not fit the LDS budget are drawn
+    again.  Seeded: the same count gives the same sets."""
+    import math
+    import random
+    rng = random.Random(seed)
+    sets = {}
+    while len(sets) < count:
+        alignment = rng.choice([4, 8, 16])
+        offset = {4: rng.choice([0, 1, 2, 3]), 8: rng.choice([0, 2]), 16: 0}[alignment]
+        bpt = alignment * rng.randint(1, 8)
+        floats = abs(int(math.ceil(rng.gauss(256, 256))))
+        elmts = rng.randint(1, 32)
+        waves = rng.randint(1, 8)
+        if floats == 0:
+            continue
+        per = alignment // 4
+        padded = (floats + per - 1) // per * per
+        if (elmts * padded + offset) * 4 > LDS_BUDGET:
+            continue
+        name = f"draw_a{alignment}_o{offset}_b{bpt}_e{floats * 4}_t{waves * 64}_n{elmts}"
+        sets[name] = dict(ALIGNMENT=alignment, ALIGN_OFFSET=offset, BYTES_PER_THREAD=bpt, BYTES_PER_ELMT=floats * 4,
+                          DMA_THREADS=waves * 64, NUM_ELMTS=elmts)
+    return sets
+
+
+def built_parameter_sets():
+    """The parameter sets of the library on disk (its manifest), or the standard ones when there is none."""
+    import json
+    try:
+        with open(MANIFEST) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return dict(PARAMETER_SETS)
 
 # kernel numbers of a launcher: 0-3 warp-specialised with four / three / two / one compile-time parameters (the
 # sequential program has no "four"), 4-7 the same not warp-specialised
@@ -381,7 +423,11 @@ def build(jobs=None):
         return None
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     os.makedirs(OUT_DIR, exist_ok=True)
-    units = [(p, s, m) for p in PROGRAMS for s, m in PARAMETER_SETS.items() if has_unit(p, m)]
+    # CUDADMA_REFKERNEL_DRAWS=N adds N seeded draws from the distribution of the reference's random sweep to the five
+    # directed sets (about 40 s of one core per program and set); the manifest tells the tests what was built
+    sets = dict(PARAMETER_SETS)
+    sets.update(drawn_parameter_sets(int(os.environ.get("CUDADMA_REFKERNEL_DRAWS", "0") or 0)))
+    units = [(p, s, m) for p in PROGRAMS for s, m in sets.items() if has_unit(p, m)]
     with tempfile.TemporaryDirectory() as scratch:        # the reference's text exists only here, and only for the build
         with concurrent.futures.ThreadPoolExecutor(max_workers=jobs or min(16, os.cpu_count() or 8)) as pool:
             extra = [pool.submit(_compile_halo_unit, hipcc, scratch), pool.submit(_compile_saxpy_unit, hipcc, scratch)]
@@ -390,7 +436,10 @@ def build(jobs=None):
             extra.append(pool.submit(_compile_perf_unit, hipcc, scratch))
             objs = list(pool.map(lambda u: _compile_unit(hipcc, scratch, *u), units)) + [e.result() for e in extra]
         subprocess.check_call([hipcc, "-shared", "-fPIC", "--offload-arch=gfx950"] + objs + ["-o", OUT])
-    print(f"built {OUT}: {len(units)} units ({len(PROGRAMS)} programs, {len(PARAMETER_SETS)} parameter sets) + the halo "
+    import json
+    with open(MANIFEST, "w") as f:
+        json.dump(sets, f, indent=1)
+    print(f"built {OUT}: {len(units)} units ({len(PROGRAMS)} programs, {len(sets)} parameter sets) + the halo "
           f"test kernel in {len(HALO_INSTANCES)} instantiations + the {len(SAXPY_KERNELS)} saxpy kernels + "
           f"the {len(SGEMV_CONFIGS)} sgemv configurations + the {len(STENCIL_HEADERS)} stencil kernels + the {len(PERF_KERNELS)} probe kernels")
     return OUT
