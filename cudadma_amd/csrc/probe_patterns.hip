@@ -128,6 +128,40 @@ probe_tile_write(vec4_t* __restrict__ out, const int n, const size_t blocks, con
   }
 }
 
+// Reads half of a buffer: the 256-byte granules whose index has even parity under `mask`, four loads in flight per
+// lane, and writes one xor of the chunks per workgroup.  When the parity of those address bits picks half of the
+// memory channels the rate halves; when the bits play no part in the choice of the channel it stays.
+__global__ void __launch_bounds__(kThreads)
+probe_masked_read(const vec4_t* __restrict__ in, vec4_t* __restrict__ out, const unsigned long long half_granules, const unsigned mask,
+                  const int top_bit)
+{
+  __shared__ vec4_t part[kThreads / 64];
+  const unsigned long long lanes = (unsigned long long)gridDim.x * kThreads, total = half_granules * 16;
+  // the k-th granule of even parity: k with a bit inserted at the mask's top bit that makes the parity even
+  auto chunk_of = [&](const unsigned long long t) {
+    const unsigned long long k = t >> 4, low = k & ((1ull << top_bit) - 1), high = k >> top_bit;
+    unsigned long long g = (high << (top_bit + 1)) | low;
+    g |= (unsigned long long)(__popcll(g & mask) & 1) << top_bit;
+    return in + g * 16 + (t & 15);
+  };
+  vec4_t acc = {0u, 0u, 0u, 0u};
+  unsigned long long t = (unsigned long long)blockIdx.x * kThreads + threadIdx.x;
+  for (; t + 3 * lanes < total; t += 4 * lanes) {
+    const vec4_t a = __builtin_nontemporal_load(chunk_of(t)), b = __builtin_nontemporal_load(chunk_of(t + lanes));
+    const vec4_t c = __builtin_nontemporal_load(chunk_of(t + 2 * lanes)), d = __builtin_nontemporal_load(chunk_of(t + 3 * lanes));
+    acc ^= a ^ b ^ c ^ d;
+  }
+  for (; t < total; t += lanes) acc ^= __builtin_nontemporal_load(chunk_of(t));
+#pragma unroll
+  for (int shift = 1; shift < 64; shift <<= 1) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w) acc[w] ^= (unsigned)__shfl_xor((int)acc[w], shift, 64);
+  }
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) out[blockIdx.x] = part[0] ^ part[1] ^ part[2] ^ part[3];
+}
+
 // Reads and writes together with the addresses of the transposition but without transposing inside a tile:
 // out[64 tx + r][64 ty + c] = in[64 ty + r][64 tx + c].  A workgroup turn moves 16 KB: ROWS = 16 KB / PIECE rows of
 // PIECE / 256 tiles that lie side by side in the output (one below the other in the source), so a wavefront's store
@@ -193,6 +227,15 @@ extern "C" long long cudadma_probe_pattern(int mode, const void* d_in, const int
       hipLaunchKernelGGL(probe_scatter, grid, block, 0, s, (const vec4_t*)d_in, d_idx, (vec4_t*)d_out, n_tiles);
       moved = (long long)(n * (4 + 2 * kRecBytes));
     }
+  } else if (mode == CUDADMA_PATTERN_PROBE_MASKED_READ) {
+    // n: bytes of the buffer (a power of two, at least 64 KiB); n_records: the mask over the index of the 256-byte granules
+    CUDADMA_REQUIRE(n >= 65536 && (n & (n - 1)) == 0, "n (the bytes of the buffer) must be a power of two, at least 64 KiB");
+    CUDADMA_REQUIRE(n_records > 0 && n_records < n / 256, "n_records (the mask over the granule index) must name bits inside the buffer");
+    CUDADMA_REQUIRE(d_in != nullptr && cudadma_host::aligned_to(d_in, 256), "d_in must be a 256-byte aligned device pointer");
+    const unsigned mask = (unsigned)n_records;
+    hipLaunchKernelGGL(probe_masked_read, grid, block, 0, s, (const vec4_t*)d_in, (vec4_t*)d_out, (unsigned long long)(n / 512), mask,
+                       31 - __builtin_clz(mask));
+    moved = (long long)(n / 2);
   } else {
     CUDADMA_REQUIRE(n > 0 && (n % kTile) == 0 && n * 4 <= 0x7fffffffu, "n (the matrix side) must be a positive multiple of 64 with rows below 2 GiB");
     const size_t tiles = (n / kTile) * (n / kTile);

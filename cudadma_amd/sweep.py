@@ -11,6 +11,7 @@ point; here the variants are compiled in and the occupancy is a run-time knob.
     python -m cudadma_amd.sweep placement                    # 1 GiB copies against the distance between source and destination
     python -m cudadma_amd.sweep placement_fine               # the copy yardstick alone against 51 distances from 0 to 256 MiB
     python -m cudadma_amd.sweep pattern_yardsticks           # the patterns' own addresses without LDS or objects, next to the patterns
+    python -m cudadma_amd.sweep channel_hash                 # which address bits choose the memory channel: half of a 1 GiB buffer by the parity of 1-3 bits
     python -m cudadma_amd.sweep settle                       # the first 80 launches after an idle second, one by one, with the shader clock
     python -m cudadma_amd.sweep queue_depth --config NAME    # one launch shape of QUEUE_CONFIGS, a few launches: the process to put
                                                              # under rocprofv3 --pmc when asking what more work in flight costs
@@ -258,6 +259,36 @@ def main(argv=None):
             ms = _time(lambda: wl.strided_transpose(src, dst, 0), args.steps, settle_ms=20.0)
             print(f"cudadma_strided_transpose variant 0: {pct(2 * n * n * 4, ms)} %", flush=True)
             del pool
+        elif name == "channel_hash":
+            # reads the half of a 1 GiB buffer whose 256-byte granules have even parity under one, two or three address bits:
+            # a parity that picks half of the memory channels halves the rate
+            import itertools
+            buf = wl.fill_uniform(torch.empty(1 << 28, device=dev), 9)
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            groups = int(cus * 1.5)
+            sink = torch.empty(groups * 4, device=dev)
+            bits = range(22)                                    # granule-index bits 0..21 = address bits 8..29
+            def rate(mask):
+                # the better of two measurements: one launch in a few thousand is held up by something else on the machine
+                ms = min(_time(lambda: wl.probe_pattern("masked_read", buf, None, sink, groups, n_records=mask), 5, warmup=2, settle_ms=0.0)
+                         for _ in range(2))
+                return (1 << 29) / ms / 1e6
+            for _ in range(20):
+                rate(1 << 21)
+            print("# GB/s of the half of 1 GiB chosen by the parity of the address bits named")
+            for b in bits:
+                print(f"bit {b + 8:2d}: {rate(1 << b):6.0f}", flush=True)
+            found = []
+            for k in (2, 3):
+                for combo in itertools.combinations(bits, k):
+                    mask = sum(1 << b for b in combo)
+                    found.append((rate(mask), combo))
+            found.sort()
+            print("# the 24 slowest of the 1771 pairs and triples, and the median")
+            for r, combo in found[:24]:
+                print(f"bits {' ^ '.join(str(b + 8) for b in combo):14s}: {r:6.0f}", flush=True)
+            print(f"median: {found[len(found) // 2][0]:6.0f}")
+            del buf
         elif name == "settle":
             # what the first launches after an idle phase cost, and whether the shader clock has anything to do with it: after a
             # second without GPU work, launches of one kernel back to back, each between two events, a clock probe after each

@@ -219,14 +219,16 @@ def probe_clock(ticks, iterations=1 << 16):
     return ticks
 
 
-PATTERN_PROBE_MODES = ("gather_xor", "scatter", "tile_read", "tile_write", "tile_copy")
+PATTERN_PROBE_MODES = ("gather_xor", "scatter", "tile_read", "tile_write", "tile_copy", "masked_read")
 
 
 def probe_pattern(mode, src, idx, out, workgroups, n_records=0):
     """One launch of a yardstick with a pattern's own addresses (mode: index into PATTERN_PROBE_MODES or its name).
     gather_xor: src = table, idx = int32 indices, out = one 128-byte row per 32 indices; scatter: src = records,
     idx = int32 indices, out = table of n_records records; tile_read: src = n x n float matrix, out = 16 bytes per
-    workgroup; tile_write: out = n x n matrix.  Returns the algorithmic bytes moved."""
+    workgroup; tile_write: out = n x n matrix; tile_copy: src and out n x n matrices; masked_read: src = buffer of a power of
+    two of bytes, n_records = the bit mask over the index of its 256-byte granules, out = 16 bytes per workgroup.  Returns the
+    algorithmic bytes moved."""
     if isinstance(mode, str):
         mode = PATTERN_PROBE_MODES.index(mode)
     if mode in (0, 1):
@@ -234,6 +236,8 @@ def probe_pattern(mode, src, idx, out, workgroups, n_records=0):
         n = idx.numel()
         if not n_records:
             n_records = (src if mode == 0 else out).numel() * (src if mode == 0 else out).element_size() // 128
+    elif mode == 5:
+        n = src.numel() * src.element_size()
     else:
         n = (src if mode in (2, 4) else out).shape[0]
     moved = lib().cudadma_probe_pattern(mode, _p(src) if src is not None else None, _p(idx) if idx is not None else None,

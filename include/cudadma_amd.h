@@ -397,6 +397,11 @@ int cudadma_probe_clock(uint64_t* d_ticks, int iterations, void* stream);
  *               pattern r * n + c.  n * n * 4 bytes.  d_in and d_idx are ignored.
  *   TILE_COPY   both halves together without the transposition inside a tile:
  *               d_out[64 tx + r][64 ty + c] = d_in[64 ty + r][64 tx + c].  2 * n * n * 4 bytes.
+ *   MASKED_READ d_in: a buffer of n bytes (a power of two, 256-byte aligned); n_records: a bit mask over the index of
+ *               its 256-byte granules.  Reads the granules whose index has even parity under the mask (half of the
+ *               buffer: n / 2 bytes); d_out receives 16 bytes per workgroup, the xor of the 16-byte chunks it read.
+ *               When the parity of those address bits picks half of the memory channels, the rate halves: a probe
+ *               for the address hash of the part.  d_idx is ignored.
  * Two knobs of cudadma_set_tuning shape TILE_WRITE and TILE_COPY: "probe_piece_bytes" (256, 512, 1024, 2048 or
  * 4096; default 256, one tile) is the length of the piece of an output row that a workgroup writes per turn
  * (TILE_COPY then reads pieces of as many source tiles per turn), "probe_xcd_group" = 1 gives the workgroups of
@@ -407,7 +412,8 @@ enum {
   CUDADMA_PATTERN_PROBE_TILE_READ  = 2,
   CUDADMA_PATTERN_PROBE_TILE_WRITE = 3,
   CUDADMA_PATTERN_PROBE_TILE_COPY  = 4,
-  CUDADMA_PATTERN_PROBE_MODES      = 5
+  CUDADMA_PATTERN_PROBE_MASKED_READ = 5,
+  CUDADMA_PATTERN_PROBE_MODES      = 6
 };
 long long cudadma_probe_pattern(int mode, const void* d_in, const int32_t* d_idx, void* d_out, size_t n,
                                 size_t n_records, int workgroups, void* stream);

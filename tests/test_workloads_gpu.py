@@ -621,6 +621,39 @@ def test_pattern_yardsticks_move_what_they_say(device, workgroups):
         want[t % workgroups] ^= np.bitwise_xor.reduce(tile, axis=0)
     assert np.array_equal(d_x.cpu().numpy().view(np.uint32).reshape(-1, 4), want)
 
+    print(f"pattern yardstick tile_copy workgroups {workgroups}", flush=True)
+    for side, piece in ((320, 256), (512, 1024), (512, 2048), (320, 1024)):
+        mat = ol.uniform(side * side, 1002).reshape(side, side)
+        d_h = torch.from_numpy(mat).to(device)
+        d_c = torch.zeros((side, side), dtype=torch.float32, device=device)
+        wl.set_tuning("probe_piece_bytes", piece)
+        try:
+            if (side * 4) % piece:
+                with pytest.raises(cd.CudaDMAError, match="multiple of the piece"):
+                    wl.probe_pattern("tile_copy", d_h, None, d_c, workgroups)
+                continue
+            moved = wl.probe_pattern("tile_copy", d_h, None, d_c, workgroups)
+        finally:
+            wl.set_tuning("probe_piece_bytes", 0)
+        torch.cuda.synchronize()
+        assert moved == 2 * side * side * 4
+        t = side // 64
+        want = mat.reshape(t, 64, t, 64).transpose(2, 1, 0, 3).reshape(side, side)          # tiles swapped, not transposed inside
+        assert np.array_equal(d_c.cpu().numpy().view(np.uint32), np.ascontiguousarray(want).view(np.uint32))
+
+    buf = ol.uniform(1 << 16, 3)                                   # 256 KiB: 1024 granules of 256 B
+    d_x = torch.zeros(workgroups * 4, dtype=torch.int32, device=device)
+    for mask in (1, 0b1000000001, 0b101010):
+        print(f"pattern yardstick masked_read mask {mask} workgroups {workgroups}", flush=True)
+        moved = wl.probe_pattern("masked_read", torch.from_numpy(buf).to(device), None, d_x, workgroups, n_records=mask)
+        torch.cuda.synchronize()
+        assert moved == buf.nbytes // 2
+        granules = buf.view(np.uint32).reshape(-1, 16, 4)
+        even = np.array([bin(g & mask).count("1") % 2 == 0 for g in range(granules.shape[0])])
+        want = np.bitwise_xor.reduce(granules[even].reshape(-1, 4), axis=0)
+        got = np.bitwise_xor.reduce(d_x.cpu().numpy().view(np.uint32).reshape(-1, 4), axis=0)    # over the workgroups
+        assert np.array_equal(got, want)
+
     d_m = torch.zeros((n, n), dtype=torch.int32, device=device)
     print(f"pattern yardstick tile_write workgroups {workgroups}", flush=True)
     moved = wl.probe_pattern("tile_write", None, None, d_m, workgroups)
