@@ -332,3 +332,18 @@ def test_plan_extents_are_the_footprint_of_the_closed_form():
         assert (dst_origin + ext[2], dst_origin + ext[3]) == (touched[0], touched[-1] + 1), case
         src_bytes = want[touched]
         assert (src_origin + ext[0], src_origin + ext[1]) == (src_bytes.min(), src_bytes.max() + 1), case
+
+
+def test_the_top_level_holds_only_what_belongs_there():
+    """A stray file at the repository root (a shell redirect gone wrong, a result left behind) travels to every GPU run and
+    into history: the tracked top-level entries are the ones named here and the records the round driver writes."""
+    import subprocess
+    if not os.path.isdir(os.path.join(ROOT, ".git")):
+        pytest.skip("not a git checkout")
+    tracked = subprocess.check_output(["git", "-C", ROOT, "ls-files"], text=True).splitlines()
+    top = sorted({path.split("/")[0] for path in tracked})
+    expected = {".gitignore", ".gpurunignore", "README.md", "DESIGN.md", "INTEGRATION.md", "SURVEY.md", "BASELINE.md", "BASELINE.json",
+                "VERDICT.md", "ADVICE.md", "__graft_entry__.py", "bench.py", "cudadma_amd", "include", "oracle", "profiles", "tests"}
+    records = re.compile(r"^(BENCH|GPUTEST|MULTICHIP|SCALE|COPYCHECK|PROGRESS)(_r\d+)?\.(json|jsonl)$")
+    strays = [name for name in top if name not in expected and not records.match(name)]
+    assert not strays, f"unexpected entries at the repository root: {strays}"
