@@ -42,6 +42,7 @@ PATTERN_KERNELS = {
     "strided_settled": "transpose_split<3, 1, 1, false>",
     "sequential_read_probe": "perf_manual<2, 4>",
     "strided_even_split": "transpose_single<true, true>",
+    "strided_double_buffered_lds": "transpose_double_lds<3, 1>",
     "strided_two_lds_tiles": "transpose_manual_double<272, false>",
     "sequential": "copy_manual_double<4>",
     "sequential_hbm": "copy_single<true, false>",
@@ -257,10 +258,17 @@ def main():
     if want("strided_even_split"):
         ms, _ = time_launches(lambda: wl.strided_transpose(src, dst, 1), steps, warmup, SETTLE_MS)
         report(patterns, "strided_even_split", ms, strided_bytes, "the same kernel shape with two DMA and two compute wavefronts (128 + 128 threads)")
+    if want("strided_double_buffered_lds"):
+        ms, _ = time_launches(lambda: wl.strided_transpose(src, dst, wl.TRANSPOSE_DOUBLE_LDS_VARIANT), steps, warmup, SETTLE_MS)
+        report(patterns, "strided_double_buffered_lds", ms, strided_bytes,
+               "the double buffer in LDS: two LDS tiles with a guard each, filled in turn by one CudaDMAStrided object, the next tile in "
+               "the DMA wavefronts' registers (one tile of loads in flight), three DMA wavefronts + one compute wavefront, one workgroup "
+               "per compute unit")
     if want("strided_two_lds_tiles"):
         ms, _ = time_launches(lambda: wl.strided_transpose(src, dst, wl.TRANSPOSE_TWO_LDS_TILES_VARIANT), steps, warmup, SETTLE_MS)
         report(patterns, "strided_two_lds_tiles", ms, strided_bytes,
-               "the same transposition with two LDS tiles and two CudaDMAStrided objects (manual double buffering in LDS)")
+               "the same transposition with two LDS tiles and two CudaDMAStrided objects (manual double buffering in LDS: two tiles "
+               "of loads in flight, four workgroups per compute unit)")
     # ---- yardsticks on the same two 1 GiB buffers: the plain copy used to calibrate the counters, the vendor's
     # copy, and read-only / write-only / copy streams each at the best of a few launch shapes ----
     flat_src, flat_dst = src.view(-1), dst.view(-1)
@@ -434,7 +442,8 @@ def main():
     if t_halo:
         halo_traffic = t_halo / (2 * 512 ** 3 * 4)
     priced = {"strided": ("copy_best_shape", 1.0), "strided_settled": ("copy_best_shape", 1.0), "strided_even_split": ("copy_best_shape", 1.0),
-              "strided_two_lds_tiles": ("copy_best_shape", 1.0), "sequential": ("copy_best_shape_64MiB", 1.0),
+              "strided_two_lds_tiles": ("copy_best_shape", 1.0),
+              "strided_double_buffered_lds": ("copy_best_shape", 1.0), "sequential": ("copy_best_shape_64MiB", 1.0),
               "sequential_hbm": ("copy_best_shape", 1.0), "sequential_read_probe": ("read_only", 1.0),
               "gather": ("gather_reads_alone", 1.0), "gather_hbm": ("gather_hbm_reads_alone", 1.0), "scatter": ("scatter_writes_alone", 1.0),
               "halo": ("copy_best_shape", halo_traffic), "halo_handshake": ("copy_best_shape", halo_traffic),
@@ -471,8 +480,9 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "CudaDMAStrided 2D tile extraction: 16384x16384 f32, 64 rows x 256 B tiles at 65536 B stride, "
-                               "double-buffered as one tile in LDS plus the next in the DMA wavefronts' registers (the form with "
-                               "two LDS tiles is patterns.strided_two_lds_tiles), transposed to output (benchmark config 2 of 5)",
+                               "double-buffered as one tile in LDS plus the next in the DMA wavefronts' registers (the forms with "
+                               "two LDS tiles are patterns.strided_double_buffered_lds, one object, and patterns.strided_two_lds_tiles, "
+                               "two objects), transposed to output (benchmark config 2 of 5)",
                    "tile_rows": 64, "tile_row_bytes": 256, "src_stride_bytes": 65536,
                    "workgroup": "192 DMA + 64 compute threads", "workgroups": "one per compute unit"},
         "roofline": roofline,

@@ -88,6 +88,9 @@ static const VariantInfo kStrided[] = {
 #else
   {""}, {""},
 #endif
+  {"double buffer in LDS with one object: two LDS tiles with a guard each, filled in turn by one CudaDMAStrided object on "
+   "three DMA wavefronts, the next tile in their registers (one tile of loads in flight), one compute wavefront, one "
+   "workgroup per compute unit"},
 };
 static const VariantInfo kGather[] = {
   {"the library's choice: variant 6 (two objects, index words requested one transfer ahead)"},

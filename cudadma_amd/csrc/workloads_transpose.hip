@@ -470,6 +470,78 @@ transpose_split(const float* __restrict__ in, float* __restrict__ out, const int
   }
 }
 
+// The double buffer in LDS with one object: two LDS tiles, each with a sync-only guard, filled in turn by one
+// CudaDMAStrided object on the DMA wavefronts; the tile after the one that is landing waits in their registers, so one
+// tile of loads is in flight (the amount this pattern runs best with) while up to two tiles sit in LDS.  The compute
+// side is that of transpose_split.  src/perf/sequential/perf_sequential.cu:116-173 is the reference's double buffering
+// (two objects on two DMA groups); with the two-phase calls one object serves both buffers.
+template<int DW, int CW>
+__global__ void __launch_bounds__((DW + CW) * 64)
+transpose_double_lds(const float* __restrict__ in, float* __restrict__ out, const int n, const int num_tiles, const int band)
+{
+  static_assert(CW == 1 || CW == 2 || CW == 4, "the compute wavefronts share the sixteen 16-byte columns of a tile row evenly");
+  constexpr int kLdsRow = 272;
+  constexpr int kDma = DW * 64, kCompute = CW * 64;
+  constexpr int kChunks = kTile * kRowBytes / 16;
+  constexpr int kBpt = ((kChunks + kDma - 1) / kDma) * 16;
+  __shared__ __attribute__((aligned(16))) char buf0[kTile * kLdsRow];
+  __shared__ __attribute__((aligned(16))) char buf1[kTile * kLdsRow];
+  cudaDMACustom guard0(0, kDma, kCompute, kCompute);
+  cudaDMACustom guard1(1, kDma, kCompute, kCompute);
+  typedef CudaDMAStrided<false, 16, kBpt, kRowBytes, kDma, kTile> obj_t;
+  const int tiles_per_side = n / kTile;
+  const int stride = gridDim.x;
+  const int last = num_tiles - 1;
+  auto src_of = [&](const int t) {
+    int ty, tx;
+    tile_coords(t < num_tiles ? t : last, tiles_per_side, band, ty, tx);     // past the end: the last tile again, loads stay unconditional
+    return (const void*)(in + (size_t)ty * kTile * n + (size_t)tx * kTile);
+  };
+  if (guard0.owns_this_thread()) {
+    obj_t a(n * 4, kLdsRow, kCompute);
+    int t = blockIdx.x;
+    if (t >= num_tiles) return;
+    a.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t));
+    for (;;) {
+      guard0.wait_for_dma_start();
+      a.template wait_xfer_finish<true, LOAD_CACHE_STREAMING, STORE_LDS>(buf0);
+      guard0.finish_async_dma();
+      a.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t + stride));
+      if (t + stride >= num_tiles) break;
+      guard1.wait_for_dma_start();
+      a.template wait_xfer_finish<true, LOAD_CACHE_STREAMING, STORE_LDS>(buf1);
+      guard1.finish_async_dma();
+      a.template start_xfer_async<true, LOAD_CACHE_STREAMING, STORE_LDS>(src_of(t + 2 * stride));
+      t += 2 * stride;
+      if (t >= num_tiles) break;
+    }
+  } else {
+    constexpr int kUnits = 16 / CW;
+    const int lane = threadIdx.x & 63;
+    const int w = threadIdx.x >> 6;
+    auto write_out = [&](const char* tile, const cudaDMACustom& guard, const int t) __attribute__((always_inline)) {
+      int ty, tx;
+      tile_coords(t, tiles_per_side, band, ty, tx);
+      guard.wait_for_dma_finish();
+      vec4_t v[kUnits];
+      const vec4_t* row = (const vec4_t*)(tile + lane * kLdsRow) + w * kUnits;
+#pragma unroll
+      for (int j = 0; j < kUnits; ++j) v[j] = row[j];
+      guard.start_async_dma();
+      float* o = out + (size_t)(tx * kTile + w * 4 * kUnits + (lane & 3)) * n + (size_t)ty * kTile + (lane & ~3);
+#pragma unroll
+      for (int j = 0; j < kUnits; ++j)
+        __builtin_nontemporal_store(quad_transpose(v[j], lane), (vec4_t*)(o + (size_t)(4 * j) * n));
+    };
+    guard0.start_async_dma();
+    guard1.start_async_dma();
+    for (int t = blockIdx.x; t < num_tiles; t += 2 * stride) {
+      write_out(buf0, guard0, t);
+      if (t + stride < num_tiles) write_out(buf1, guard1, t + stride);
+    }
+  }
+}
+
 #ifdef HIPDMA_SWEEP_VARIANTS
 // The transposition with output rows written 1 KiB at a time.  The DMA side is that of transpose_split (tiles of 64
 // rows x 256 B, one tile of loads in flight, NBUF LDS tiles guarded by sync-only objects); the compute wavefront
@@ -707,7 +779,7 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
   // The kernels with one LDS tile (variants 1 and 4) run best with exactly one workgroup per compute unit, i.e. one
   // 16 KB tile of loads in flight per compute unit, and with the tiles walked down the columns (the workgroups that
   // run together then write whole output rows); the others with four workgroups and bands of 16 tile rows.
-  const bool one_tile = variant == 0 || variant == 1 || variant == 4 || variant == 10;
+  const bool one_tile = variant == 0 || variant == 1 || variant == 4 || variant == 10 || variant == 14;
   int band = workloads::tuning("transpose_band", one_tile ? tiles_per_side : kDefaultBand);
   if (band > tiles_per_side) band = tiles_per_side;
   while (band > 1 && tiles_per_side % band != 0) band /= 2;      // bands must tile the matrix
@@ -741,6 +813,7 @@ extern "C" int cudadma_strided_transpose(const float* d_in, float* d_out, int n,
       hipLaunchKernelGGL(e->kernel, grid_for(1), dim3((e->dw + e->cw) * 64), 0, s, d_in, d_out, n, tiles, band);
       break;
     }
+    case 14: hipLaunchKernelGGL((transpose_double_lds<3, 1>), grid_for(1), dim3(256), 0, s, d_in, d_out, n, tiles, band); break;
 #ifdef HIPDMA_SWEEP_VARIANTS
     case 12:
     case 13: {

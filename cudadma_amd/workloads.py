@@ -19,6 +19,7 @@ TRANSPOSE_SPLIT_VARIANT = 10           # cudadma_strided_transpose variant whose
 # DMA wavefronts and one compute wavefront for a tile requested in pieces: 3 halves (1.5 tiles), 5, 6 and 7 quarters (1.25, 1.5,
 # 1.75 tiles) and 3 quarters (0.75) in flight, and 8 for one tile in flight without a pause)
 TRANSPOSE_TWO_LDS_TILES_VARIANT = 11    # two LDS tiles and two CudaDMAStrided objects (manual double buffering in LDS)
+TRANSPOSE_DOUBLE_LDS_VARIANT = 14       # two LDS tiles filled in turn by one object, one tile of loads in flight
 HALO_WIDE_TILES_VARIANT = 6            # cudadma_halo_stencil variant 0 with tiles of 64 x 16 cells
 GEMM_WARP_SPECIALISED_VARIANT = 7      # the cudadma_gemm_bf16 variant in which DMA wavefronts feed compute wavefronts
 

@@ -127,7 +127,7 @@ def test_strided_transpose_small(device, variant, n):
     assert np.array_equal(dst.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("variant", [0, 10, 1, 4, 11])
+@pytest.mark.parametrize("variant", [0, 10, 1, 4, 11, 14])
 @pytest.mark.parametrize("band,workgroups", [(0, 0), (1, 0), (3, 7), (5, 300), (256, 255), (1000, 100000)])
 def test_strided_transpose_under_every_tuning(device, variant, band, workgroups):
     """The tile order and the number of workgroups are tuning knobs: the result does not depend on them."""
@@ -175,7 +175,7 @@ def test_strided_transpose_under_every_split(device, split, n, workgroups):
             wl.set_tuning("transpose_split", 0)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 11])                   # the reported kernel, its even split and the one with two LDS tiles
+@pytest.mark.parametrize("variant", [0, 1, 11, 14])               # the reported kernel, its even split and the two forms with two LDS tiles
 def test_strided_transpose_full_size(device, variant):
     n = 16384
     src = wl.fill_uniform(torch.empty(n * n, dtype=torch.float32, device=device), 1002).view(n, n)
