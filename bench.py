@@ -4,8 +4,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only NAME[,NAME...]] [--no-cpu-baseline]
 
 A step is one launch of the CudaDMAStrided tile-transpose kernel over the whole 16384 x 16384 float32
-matrix (benchmark config 2, the configuration the metric is quoted on); inputs are resident in HBM before
-the timed region.  The other HBM-bound patterns (sequential copy, indirect gather, halo stencil), the scatter
+matrix (benchmark config 2, the configuration the metric is quoted on).  The inputs of every pattern of the run
+are generated on the device first, so every timed region starts with its inputs resident in HBM; the headline is
+then timed exactly as the command line says (--warmup launches, then --steps timed ones).  The other HBM-bound patterns (sequential copy, indirect gather, halo stencil), the scatter
 in the opposite direction and the GEMM are timed the same way (HIP events on the launch stream) and reported
 under "patterns" / "gemm".  The sequential copy and the gather are each reported twice: at the size the
 configuration names (64 MiB buffer, 512 MiB table: both working sets are helped by the 256 MB Infinity Cache)
@@ -242,16 +243,51 @@ def main():
     # same kernel as the distance varies modulo 64 MiB; the transposition does not care), and two separate
     # allocations land wherever the allocator, or a profiler loaded into the process, leaves room.
     n = 16384
+    setup_start, setup_stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    setup_start.record()
     pool = torch.empty(2 * n * n, dtype=torch.float32, device=dev)
     src = wl.fill_uniform(pool[:n * n], 1002).view(n, n)
     dst = pool[n * n:].view(n, n)
+    # The inputs of every other pattern of the run are generated here as well, before anything is timed: every timed
+    # region then starts with its inputs resident in HBM, and the device has left its idle state (the shader clock dips
+    # from 2.42 to 2.13-2.25 GHz between 1.5 and 8 ms after work begins on an idle device) by the time the first one starts.
+    inputs = {}
+    if want("sequential"):
+        m = 64 * 1024 * 1024 // 4
+        s_src = wl.fill_uniform(torch.empty(m, dtype=torch.float32, device=dev), 1001)
+        inputs["sequential"] = (s_src, torch.empty_like(s_src))
+    n_idx = 32 * 1024 * 1024
+    for name, recs in (("gather", 4 * 1024 * 1024), ("gather_hbm", 32 * 1024 * 1024)):
+        if want(name):
+            inputs[name] = (wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev), 1003),
+                            wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=dev), recs, 1003),
+                            torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, dtype=torch.float32, device=dev))
+    if want("scatter"):
+        recs = 4 * 1024 * 1024
+        inputs["scatter"] = (wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev), 1006),
+                             wl.fill_permutation(torch.empty(recs, dtype=torch.int32, device=dev), 1006),
+                             torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev))
+    if want("halo") or want("halo_handshake") or want("halo_wide_tiles"):
+        g, p = 512, 2 * wl.STENCIL_RADIUS
+        inputs["halo"] = (wl.fill_uniform(torch.empty((g + p) ** 3, dtype=torch.float32, device=dev), 1004).view(g + p, g + p, g + p),
+                          torch.empty((g, g, g), dtype=torch.float32, device=dev))
+    if want("gemm") or want("gemm_warp_specialised"):
+        dim = 4096
+        inputs["gemm"] = (wl.fill_normal_bf16(torch.empty((dim, dim), device=dev, dtype=torch.bfloat16), 1005),
+                          wl.fill_normal_bf16(torch.empty((dim, dim), device=dev, dtype=torch.bfloat16), 2005),
+                          torch.empty((dim, dim), device=dev, dtype=torch.float32))
+    setup_stop.record()
+    torch.cuda.synchronize()
+    setup_ms = setup_start.elapsed_time(setup_stop)
+    log(f"inputs generated in {setup_ms:.1f} ms of device time")
     strided_ms, strided_wall_ms = time_launches(lambda: wl.strided_transpose(src, dst, STRIDED_VARIANT), steps, warmup)
     strided_bytes = 2 * n * n * 4
     strided_note = ("CudaDMAStrided 64x256B tiles of a 16384^2 f32 matrix, transposed out: one LDS tile, the next tile in the DMA "
                     "wavefronts' registers (the double buffer is LDS + registers), one workgroup of three DMA wavefronts and one "
                     "compute wavefront per compute unit")
     report(patterns, "strided", strided_ms, strided_bytes, strided_note + f"; timed as the command line says: {warmup} untimed launches, "
-           f"then {steps} timed ones", settle_ms=0.0)
+           f"then {steps} timed ones, right after the inputs of the whole run were generated ({setup_ms:.0f} ms of device time)", settle_ms=0.0)
+    patterns["strided"]["device_ms_of_input_generation_before"] = round(setup_ms, 1)
     if want("strided_settled"):
         ms, _ = time_launches(lambda: wl.strided_transpose(src, dst, STRIDED_VARIANT), steps, warmup, SETTLE_MS)
         report(patterns, "strided_settled", ms, strided_bytes, "the kernel of the strided row under the policy of the rows below")
@@ -304,8 +340,7 @@ def main():
     # ---- config 1: sequential copy in 16 KiB tiles: the 64 MiB of the configuration, and 1 GiB ----
     if want("sequential"):
         m = 64 * 1024 * 1024 // 4
-        s_src = wl.fill_uniform(torch.empty(m, dtype=torch.float32, device=dev), 1001)
-        s_dst = torch.empty_like(s_src)
+        s_src, s_dst = inputs.pop("sequential")
         ms, _ = time_launches(lambda: wl.sequential_copy(s_src, s_dst, 0), max(steps, 50), warmup, SETTLE_MS)
         report(patterns, "sequential", ms, 2 * m * 4, "CudaDMASequential 16 KiB tiles of the configuration's 64 MiB f32 buffer: the "
                "128 MiB working set stays in the 256 MB Infinity Cache from launch to launch, so this is a cache-assisted rate, "
@@ -341,7 +376,6 @@ def main():
     del pool
 
     # ---- config 3: indirect gather, row-sum consumer: the 512 MiB table of the configuration, and a 4 GiB table ----
-    n_idx = 32 * 1024 * 1024
     for name, recs, note, bound in (
             ("gather", 4 * 1024 * 1024, "CudaDMAIndirect 32 x 128 B records per tile from the configuration's 512 MiB table (4 Mi records, "
              "each read 8 times over per launch: most reads are served by L2 and the 256 MB Infinity Cache), two objects per DMA "
@@ -351,9 +385,7 @@ def main():
              "average; sixteen times the Infinity Cache), four workgroups per compute unit, row-sum consumer", "hbm")):
         if not want(name):
             continue
-        table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev), 1003)
-        idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=dev), recs, 1003)
-        sums = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, dtype=torch.float32, device=dev)
+        table, idx, sums = inputs.pop(name)
         ms, _ = time_launches(lambda: wl.gather_rowsum(table, idx, sums, 0), steps, warmup, SETTLE_MS)
         report(patterns, name, ms, n_idx * 4 + n_idx * 128 + sums.numel() * 4, note, bound=bound)
         if want("yardsticks"):
@@ -365,9 +397,7 @@ def main():
     # ---- the opposite direction (LDS -> global): scatter of 4 Mi records by a permutation ----
     if want("scatter"):
         recs = 4 * 1024 * 1024
-        records = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev), 1006)
-        perm = wl.fill_permutation(torch.empty(recs, dtype=torch.int32, device=dev), 1006)
-        table = torch.empty(recs * wl.REC_FLOATS, dtype=torch.float32, device=dev)
+        records, perm, table = inputs.pop("scatter")
         ms, _ = time_launches(lambda: wl.scatter_copy(records, perm, table, 0), steps, warmup, SETTLE_MS)
         report(patterns, "scatter", ms, recs * 4 + 2 * recs * 128,
                "CudaDMAIndirect<false> LDS -> global: 4 Mi records of 128 B placed by a permutation, 32 records per tile")
@@ -380,9 +410,7 @@ def main():
     # ---- config 4: halo stencil ----
     if want("halo") or want("halo_handshake") or want("halo_wide_tiles"):
         g = 512
-        p = 2 * wl.STENCIL_RADIUS
-        grid_in = wl.fill_uniform(torch.empty((g + p) ** 3, dtype=torch.float32, device=dev), 1004).view(g + p, g + p, g + p)
-        grid_out = torch.empty((g, g, g), dtype=torch.float32, device=dev)
+        grid_in, grid_out = inputs.pop("halo")
         if want("halo"):
             ms, _ = time_launches(lambda: wl.halo_stencil(grid_in, grid_out, 0), steps, warmup, SETTLE_MS)
             report(patterns, "halo", ms, 2 * g ** 3 * 4, "CudaDMAHalo radius-4 ring of 32x32 tiles, 25-point stencil on a 512^3 f32 grid "
@@ -404,9 +432,7 @@ def main():
     gemm = None
     if want("gemm") or want("gemm_warp_specialised"):
         dim = 4096
-        ga = wl.fill_normal_bf16(torch.empty((dim, dim), device=dev, dtype=torch.bfloat16), 1005)
-        gb = wl.fill_normal_bf16(torch.empty((dim, dim), device=dev, dtype=torch.bfloat16), 2005)
-        gc = torch.empty((dim, dim), device=dev, dtype=torch.float32)
+        ga, gb, gc = inputs.pop("gemm")
         flops = 2.0 * dim ** 3
         mfma_busy = lambda name: (counters.get("patterns", {}).get(name) or {}).get("mfma_busy")
 
