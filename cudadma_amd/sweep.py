@@ -38,6 +38,10 @@ QUEUE_CONFIGS = {
     "copy_16wg": ("copy_nontemporal", 16),
     "read_1.5wg": ("read_nontemporal", 1.5), "read_4wg": ("read_nontemporal", 4), "read_8wg": ("read_nontemporal", 8),
     "write_0.5wg": ("write", 0.5), "write_4wg": ("write", 4), "write_8wg": ("write", 8),
+    # cached against non-temporal loads: the plain read stream, and the read-bandwidth probe on CudaDMASequential
+    # (16 KiB elements, four DMA wavefronts, manual double buffering, two workgroups per compute unit)
+    "read_cached_1.5wg": ("read", 1.5),
+    "probe_cached": ("perf_sequential", "LOAD_CACHE_ALL"), "probe_streaming": ("perf_sequential", "LOAD_CACHE_STREAMING"),
 }
 
 
@@ -336,6 +340,11 @@ def main(argv=None):
                 wl.set_tuning("transpose_workgroups", cus * shape["transpose_workgroups"])
                 fn = lambda: wl.strided_transpose(src.view(16384, 16384), dst.view(16384, 16384), wl.TRANSPOSE_SPLIT_VARIANT)
                 nbytes = 2 * m * 4
+            elif what == "perf_sequential":
+                groups, elmt = 2 * cus, 16 * 1024
+                lq = wl.LOAD_CACHE_STREAMING if shape == "LOAD_CACHE_STREAMING" else wl.LOAD_CACHE_ALL
+                fn = lambda: wl.perf_sequential(src, elmt, 4, wl.BUFFERING_MANUAL, (m * 4) // (groups * elmt), groups, None, lq, wl.STORE_LDS)
+                nbytes = m * 4
             else:
                 s_, d_ = (None if what.startswith("write") else src), (None if what.startswith("read") else dst)
                 fn = lambda: wl.probe_memory(what, s_, d_, int(cus * shape))
