@@ -13,6 +13,7 @@ point; here the variants are compiled in and the occupancy is a run-time knob.
     python -m cudadma_amd.sweep pattern_yardsticks           # the patterns' own addresses without LDS or objects, next to the patterns
     python -m cudadma_amd.sweep channel_hash                 # which address bits choose the memory channel: half of a 1 GiB buffer by the parity of 1-3 bits
     python -m cudadma_amd.sweep settle                       # the first 80 launches after an idle second, one by one, with the shader clock
+    python -m cudadma_amd.sweep two_streams                  # a read-only kernel and a write-only kernel side by side against one copy kernel
     python -m cudadma_amd.sweep queue_depth --config NAME    # one launch shape of QUEUE_CONFIGS, a few launches: the process to put
                                                              # under rocprofv3 --pmc when asking what more work in flight costs
 """
@@ -353,6 +354,44 @@ def main(argv=None):
             print(f"queue_depth {args.config:22s} {ms:8.4f} ms  {nbytes / ms / 1e6:7.0f} GB/s  {100 * nbytes / ms / 1e6 / PEAK_GBS:5.1f}%", flush=True)
             wl.set_tuning("transpose_split", 0)
             wl.set_tuning("transpose_workgroups", 0)
+            del pool
+        elif name == "two_streams":
+            # a read-only and a write-only kernel, 1 GiB each, side by side on two streams: do two kernels that each issue one
+            # kind of request pass the copy, whose every wavefront issues both?
+            m = (1 << 30) // 4
+            pool = torch.empty(2 * m, device=dev)
+            src, dst = wl.fill_uniform(pool[:m], 1002), pool[m:]
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+
+            def pair(read_wg, write_wg, reps):
+                torch.cuda.synchronize()
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                s1.wait_event(a)
+                s2.wait_event(a)
+                for _ in range(reps):
+                    with torch.cuda.stream(s1):
+                        wl.probe_memory("read_nontemporal", src, None, int(cus * read_wg))
+                    with torch.cuda.stream(s2):
+                        wl.probe_memory("write", None, dst, int(cus * write_wg))
+                e1, e2 = torch.cuda.Event(), torch.cuda.Event()
+                e1.record(s1)
+                e2.record(s2)
+                torch.cuda.current_stream().wait_event(e1)
+                torch.cuda.current_stream().wait_event(e2)
+                b.record()
+                torch.cuda.synchronize()
+                return a.elapsed_time(b) / reps
+
+            pair(1.5, 0.5, 40)
+            ms = _time(lambda: wl.probe_memory("copy_nontemporal", src, dst, 4 * cus), args.steps)
+            print(f"two_streams  one copy kernel, 4 wg/cu                        {ms:8.4f} ms  {100 * 2 * m * 4 / ms / 1e6 / PEAK_GBS:5.1f}%")
+            for read_wg in (0.5, 0.75, 1, 1.5, 2):
+                for write_wg in (0.25, 0.5, 1, 2):
+                    ms = pair(read_wg, write_wg, args.steps)
+                    print(f"two_streams  read {read_wg:4} wg/cu beside write {write_wg:4} wg/cu, per pair  {ms:8.4f} ms  "
+                          f"{100 * 2 * m * 4 / ms / 1e6 / PEAK_GBS:5.1f}%", flush=True)
             del pool
         elif name == "scatter":
             recs = 4 << 20
