@@ -1,7 +1,7 @@
-"""cudadma_amd: Python side of the hipDMA host drivers (libcudadma_amd.so).
+"""cudadma_amd: Python side of the hipDMA host drivers (libcudadma_amd.so, libcudadma_amd_harness.so).
 
 The device library itself is header-only C++ (include/hipDMA.h).  This package
-only loads the C ABI declared in include/cudadma_amd.h with ctypes and wraps it
+only loads the C ABI declared in include/cudadma_amd.h and include/cudadma_amd_harness.h with ctypes and wraps it
 for tests and benchmarks; PyTorch is used by callers for device memory and
 streams, never for compute.  Loading fails loudly when the shared library has
 not been built: there is no CPU fallback.
@@ -30,6 +30,8 @@ from ._lib import (  # noqa: F401
     STATUS_WAIT_GAVE_UP,
     V1Case,
     device_status,
+    harness_lib,
+    harness_lib_path,
     lib,
     lib_path,
 )

@@ -1,4 +1,4 @@
-"""ctypes binding of include/cudadma_amd.h."""
+"""ctypes binding of include/cudadma_amd.h (lib()) and include/cudadma_amd_harness.h (harness_lib())."""
 import ctypes
 import os
 
@@ -72,33 +72,40 @@ def lib_path():
     return os.path.join(_HERE, "libcudadma_amd.so")
 
 
+def harness_lib_path():
+    return os.path.join(_HERE, "libcudadma_amd_harness.so")
+
+
 _lib = None
+_harness_lib = None
 
 
-def lib():
-    """The loaded shared library; raises when it has not been built."""
-    global _lib
-    if _lib is not None:
-        return _lib
-    path = lib_path()
+def _load(path):
     if not os.path.exists(path):
         raise CudaDMAError(
             f"{path} is missing: build it with `make -C cudadma_amd/csrc` "
             "(or python -c 'import __graft_entry__ as g; g.build()'); there is no fallback path")
-    L = ctypes.CDLL(path)
+    return ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+
+
+def _declare(L, signatures):
+    for name, argtypes in signatures.items():
+        fn = getattr(L, name)
+        fn.restype = ctypes.c_int
+        fn.argtypes = argtypes
+
+
+def lib():
+    """The workloads, probes, examples and planner; raises when the library has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    L = _load(lib_path())
     vp, ci, cs = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
     L.cudadma_last_error.restype = ctypes.c_char_p
     L.cudadma_last_error.argtypes = []
     L.cudadma_device_cus.restype = ci
-    L.cudadma_num_cases.restype = ci
-    L.cudadma_get_case.restype = ci
-    L.cudadma_get_case.argtypes = [ci, ctypes.POINTER(Case)]
-    L.cudadma_run_case.restype = ci
-    L.cudadma_run_case.argtypes = [ci, ctypes.POINTER(RunArgs), vp]
-    for name, argtypes in _WORKLOAD_SIGNATURES.items():
-        fn = getattr(L, name)
-        fn.restype = ci
-        fn.argtypes = argtypes
+    _declare(L, _WORKLOAD_SIGNATURES)
     L.cudadma_plan_map.restype = ci
     L.cudadma_plan_map.argtypes = [ctypes.POINTER(PlanQuery), ctypes.c_longlong, ctypes.c_longlong, vp, cs,
                                    ctypes.POINTER(ci)]
@@ -118,13 +125,32 @@ def lib():
     L.cudadma_probe_pattern.argtypes = [ci, vp, vp, vp, cs, cs, ci, vp]
     L.cudadma_transpose_splits.restype = ci
     L.cudadma_transpose_splits.argtypes = [ctypes.POINTER(ci), ci]
+    L.cudadma_example_variant_name.restype = ctypes.c_char_p
+    L.cudadma_example_variant_name.argtypes = [ci, ci]
+    _lib = L
+    return L
+
+
+def harness_lib():
+    """The known-answer cases and self-tests of the DMA objects: a library of its own that needs the main one
+    (error text, failure record), which is therefore loaded first; raises when either has not been built."""
+    global _harness_lib
+    if _harness_lib is not None:
+        return _harness_lib
+    lib()
+    L = _load(harness_lib_path())
+    ci = ctypes.c_int
+    L.cudadma_num_cases.restype = ci
+    L.cudadma_get_case.restype = ci
+    L.cudadma_get_case.argtypes = [ci, ctypes.POINTER(Case)]
+    L.cudadma_run_case.restype = ci
+    L.cudadma_run_case.argtypes = [ci, ctypes.POINTER(RunArgs), ctypes.c_void_p]
+    _declare(L, _HARNESS_SIGNATURES)
     L.cudadma_v1_get_case.restype = ci
     L.cudadma_v1_get_case.argtypes = [ci, ctypes.POINTER(V1Case)]
     L.cudadma_v1_case_text.restype = ctypes.c_char_p
     L.cudadma_v1_case_text.argtypes = [ci]
-    L.cudadma_example_variant_name.restype = ctypes.c_char_p
-    L.cudadma_example_variant_name.argtypes = [ci, ci]
-    _lib = L
+    _harness_lib = L
     return L
 
 
@@ -147,19 +173,23 @@ _WORKLOAD_SIGNATURES = {
     "cudadma_halo_stencil": [_vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cudadma_gemm_bf16": [_vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cudadma_probe_clock": [_vp, _ci, _vp],
-    "cudadma_selftest_bounded_wait": [_vp, _vp],
-    "cudadma_selftest_split_wait": [_vp, _ci, _vp],
-    "cudadma_selftest_global_handoff": [_vp, _vp, _ci, _vp],
-    "cudadma_selftest_global_handoff_lds_only": [_vp, _vp, _ci, _vp],
     "cudadma_device_status": [ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_uint), _ci, _vp],
     "cudadma_device_status_sources": [],
-    "cudadma_selftest_all_ids": [_vp, _ci, _vp],
-    "cudadma_v1_num_cases": [],
-    "cudadma_v1_run_case": [_ci, _vp, _vp, _vp, _vp],
     "cudadma_example_num_variants": [_ci],
     "cudadma_example_saxpy": [_ci, ctypes.c_float, _vp, _vp, ctypes.c_longlong, _vp],
     "cudadma_example_sgemv": [_ci, _ci, _ci, ctypes.c_float, _vp, _ci, _vp, _vp, _vp],
     "cudadma_example_stencil2d": [_ci, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
+}
+
+# name -> argtypes of the harness library's entry points that return int and take only plain words
+_HARNESS_SIGNATURES = {
+    "cudadma_selftest_bounded_wait": [_vp, _vp],
+    "cudadma_selftest_split_wait": [_vp, _ci, _vp],
+    "cudadma_selftest_global_handoff": [_vp, _vp, _ci, _vp],
+    "cudadma_selftest_global_handoff_lds_only": [_vp, _vp, _ci, _vp],
+    "cudadma_selftest_all_ids": [_vp, _ci, _vp],
+    "cudadma_v1_num_cases": [],
+    "cudadma_v1_run_case": [_ci, _vp, _vp, _vp, _vp],
 }
 
 
@@ -177,6 +207,12 @@ def device_status(clear=True, stream=None):
 
 def exported_symbols():
     """Every extern "C" symbol include/cudadma_amd.h declares."""
-    return ["cudadma_last_error", "cudadma_device_cus", "cudadma_num_cases", "cudadma_get_case",
-            "cudadma_run_case", "cudadma_variant_name", "cudadma_example_variant_name",
-            "cudadma_v1_get_case", "cudadma_v1_case_text", "cudadma_perf_sequential", "cudadma_probe_memory", "cudadma_probe_pattern", "cudadma_transpose_splits", "cudadma_plan_map", "cudadma_plan_extents", "cudadma_diagnose", "cudadma_set_tuning"] + list(_WORKLOAD_SIGNATURES)
+    return ["cudadma_last_error", "cudadma_device_cus", "cudadma_variant_name", "cudadma_example_variant_name",
+            "cudadma_perf_sequential", "cudadma_probe_memory", "cudadma_probe_pattern", "cudadma_transpose_splits",
+            "cudadma_plan_map", "cudadma_plan_extents", "cudadma_diagnose", "cudadma_set_tuning"] + list(_WORKLOAD_SIGNATURES)
+
+
+def harness_exported_symbols():
+    """Every extern "C" symbol include/cudadma_amd_harness.h declares."""
+    return ["cudadma_num_cases", "cudadma_get_case", "cudadma_run_case", "cudadma_v1_get_case",
+            "cudadma_v1_case_text"] + list(_HARNESS_SIGNATURES)

@@ -9,6 +9,7 @@
 #pragma once
 
 #include "common.hpp"
+#include "../../include/cudadma_amd_harness.h"
 #include "../../include/hipDMA.h"
 #include "status_word.hpp"
 

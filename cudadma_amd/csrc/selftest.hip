@@ -3,6 +3,7 @@
 // host side and every wavefront still exits normally.
 #define HIPDMA_SPIN_LIMIT 256
 #include "common.hpp"
+#include "../../include/cudadma_amd_harness.h"
 #include "../../include/hipDMA.h"
 #include "status_word.hpp"
 

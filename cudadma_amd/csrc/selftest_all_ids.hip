@@ -3,6 +3,7 @@
 // slot must hold exactly the token of its phase when the compute side gets to it.  A word shared
 // between two ids, or a lost count, shows up as a wrong token (the bounded wait turns a hang into one).
 #include "common.hpp"
+#include "../../include/cudadma_amd_harness.h"
 #include "../../include/hipDMA.h"
 #include "status_word.hpp"
 

@@ -1,6 +1,7 @@
 // Self-test of the split wait (peek_dma_finish + wait_for_dma_finish(peeked)); kept apart from
 // the bounded-wait test, which lowers the poll limit for its whole translation unit.
 #include "common.hpp"
+#include "../../include/cudadma_amd_harness.h"
 #include "../../include/hipDMA.h"
 #include "status_word.hpp"
 

@@ -3,6 +3,7 @@
 // form of the adapters in hipdma/v1.hpp moves one transfer into an LDS window that
 // was filled with a sentinel, and the whole window is copied out for comparison.
 #include "common.hpp"
+#include "../../include/cudadma_amd_harness.h"
 #include "../../include/cudaDMA.h"
 #include "status_word.hpp"
 

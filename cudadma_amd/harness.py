@@ -3,7 +3,8 @@ cudadma_run_case).  Device memory comes from the caller as torch tensors."""
 import ctypes
 
 from . import _lib
-from ._lib import Case, RunArgs, check, lib
+from ._lib import Case, RunArgs, check
+from ._lib import harness_lib as lib
 
 
 def num_cases():

@@ -210,7 +210,7 @@ def test_unmatched_waits_end_and_are_reported(device):
     import ctypes
     assert cd.device_status(clear=True) == (0, 0)
     flags = torch.zeros(2, dtype=torch.int32, device=device)
-    cd._lib.check(cd.lib().cudadma_selftest_bounded_wait(ctypes.c_void_p(flags.data_ptr()), None))
+    cd._lib.check(cd.harness_lib().cudadma_selftest_bounded_wait(ctypes.c_void_p(flags.data_ptr()), None))
     torch.cuda.synchronize()
     assert flags.tolist() == [1, 1]
     bits, waves = cd.device_status(clear=False)
@@ -235,7 +235,7 @@ def test_global_memory_crosses_the_handshake(device, entry):
     import ctypes
     scratch = torch.zeros(4096, dtype=torch.int32, device=device)
     wrong = torch.zeros(1, dtype=torch.int32, device=device)
-    cd._lib.check(getattr(cd.lib(), entry)(ctypes.c_void_p(scratch.data_ptr()), ctypes.c_void_p(wrong.data_ptr()), 300, None))
+    cd._lib.check(getattr(cd.harness_lib(), entry)(ctypes.c_void_p(scratch.data_ptr()), ctypes.c_void_p(wrong.data_ptr()), 300, None))
     torch.cuda.synchronize()
     assert cd.device_status(clear=False) == (0, 0)
     if not entry.endswith("_lds_only"):
@@ -248,7 +248,7 @@ def test_split_wait_sees_every_phase(device):
     import ctypes
     out = torch.zeros(2, dtype=torch.int32, device=device)
     phases = 200
-    cd._lib.check(cd.lib().cudadma_selftest_split_wait(ctypes.c_void_p(out.data_ptr()), phases, None))
+    cd._lib.check(cd.harness_lib().cudadma_selftest_split_wait(ctypes.c_void_p(out.data_ptr()), phases, None))
     torch.cuda.synchronize()
     wrong, early = out.tolist()
     assert wrong == 0
@@ -261,6 +261,6 @@ def test_all_sixteen_ids_keep_their_own_counts(device, phases):
     ahead: no id may see another id's signals."""
     import ctypes
     out = torch.zeros(1, dtype=torch.int32, device=device)
-    cd._lib.check(cd.lib().cudadma_selftest_all_ids(ctypes.c_void_p(out.data_ptr()), phases, None))
+    cd._lib.check(cd.harness_lib().cudadma_selftest_all_ids(ctypes.c_void_p(out.data_ptr()), phases, None))
     torch.cuda.synchronize()
     assert out.item() == 0

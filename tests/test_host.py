@@ -1,9 +1,10 @@
-"""CPU-side tests of libcudadma_amd.so: it loads, exports what include/cudadma_amd.h declares,
+"""CPU-side tests of libcudadma_amd.so and libcudadma_amd_harness.so: they load, export what their headers declare,
 validates arguments before touching a GPU, and its host replay of the device objects' index
 arithmetic agrees with the oracle's closed forms for every compiled case."""
 import ctypes
 import os
 import re
+import subprocess
 
 import numpy as np
 import pytest
@@ -14,14 +15,28 @@ from tests.cases import CaseIO, case_id_str
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def test_library_exports_every_declared_symbol():
-    header = open(os.path.join(ROOT, "include", "cudadma_amd.h")).read()
-    declared = set(re.findall(r"\b(cudadma_[a-z0-9_]+)\s*\(", header))
+@pytest.mark.parametrize("header_name, load, path, bound", [
+    ("cudadma_amd.h", cd.lib, cd.lib_path, cd._lib.exported_symbols),
+    ("cudadma_amd_harness.h", cd.harness_lib, cd.harness_lib_path, cd._lib.harness_exported_symbols)])
+def test_library_exports_every_declared_symbol(header_name, load, path, bound):
+    header = open(os.path.join(ROOT, "include", header_name)).read()
+    declared = set(re.findall(r"^(?:const\s+)?[a-z_][a-z_ ]*\**\s+(cudadma_[a-z0-9_]+)\s*\(", header, flags=re.M))
     assert declared, "no declarations found"
-    L = ctypes.CDLL(cd.lib_path())
+    load()
+    # the symbol is looked up in this library's own file: its table of dynamic symbols, not what the loader
+    # would also find in a library it depends on
+    own = subprocess.run(["nm", "-D", "--defined-only", path()], capture_output=True, text=True, check=True).stdout
+    exported = {line.split()[-1] for line in own.splitlines() if line.strip()}
     for name in sorted(declared):
-        assert hasattr(L, name), f"{name} is declared in cudadma_amd.h but not exported"
-    assert declared == set(cd._lib.exported_symbols())
+        assert name in exported, f"{name} is declared in {header_name} but not exported by {os.path.basename(path())}"
+    assert declared == set(bound())
+
+
+def test_the_harness_stays_out_of_the_product_library():
+    """The several hundred instantiations of the known-answer cases are test equipment: the library a user
+    links holds the workloads, probes, examples and the planner and stays an order of magnitude smaller."""
+    assert os.path.getsize(cd.lib_path()) < 4 << 20
+    assert os.path.getsize(cd.harness_lib_path()) > os.path.getsize(cd.lib_path())
 
 
 def test_missing_library_fails_loudly(monkeypatch):
@@ -56,12 +71,12 @@ def test_case_table_is_sane():
 
 def test_run_case_validates_before_launching():
     r = cd.RunArgs(d_in=0, d_out=0, lds_bytes=1024, reps=1)
-    L = cd.lib()
+    L = cd.harness_lib()
     assert L.cudadma_run_case(0, ctypes.byref(r), None) == -1
-    assert b"d_in" in L.cudadma_last_error()
+    assert b"d_in" in cd.lib().cudadma_last_error()
     r = cd.RunArgs(d_in=4096, d_out=8192, lds_bytes=1000, reps=1)
     assert L.cudadma_run_case(0, ctypes.byref(r), None) == -1
-    assert b"lds_bytes" in L.cudadma_last_error()
+    assert b"lds_bytes" in cd.lib().cudadma_last_error()
     r = cd.RunArgs(d_in=4096, d_out=8192, lds_bytes=1024, reps=1, src_offset_bytes=2)
     assert L.cudadma_run_case(0, ctypes.byref(r), None) == -1
     assert L.cudadma_run_case(10 ** 6, ctypes.byref(r), None) == -3
@@ -71,13 +86,13 @@ def test_run_case_validates_before_launching():
     for field in ("rt_bytes_per_elmt", "rt_dma_threads", "rt_num_elmts", "rt_dimx"):
         r = cd.RunArgs(d_in=4096, d_out=8192, lds_bytes=1024, reps=1, **{field: 64})
         assert L.cudadma_run_case(full, ctypes.byref(r), None) == -1, field
-        assert b"case" in L.cudadma_last_error()
+        assert b"case" in cd.lib().cudadma_last_error()
     loose = next(i for i, c in enumerate(cases) if c.pattern == cd.PATTERN_STRIDED and c.level == 1)
     for field, value in (("rt_bytes_per_elmt", 6), ("rt_dma_threads", 100), ("rt_dma_threads", 2048), ("rt_num_elmts", -1)):
         r = cd.RunArgs(d_in=4096, d_out=8192, lds_bytes=1024, reps=1, **{field: value})
         assert L.cudadma_run_case(loose, ctypes.byref(r), None) == -1, (field, value)
-    assert L.cudadma_scatter_copy(4096, 4096, 8192, 16, 33, 0, None) == -1
-    assert L.cudadma_probe_memory(3, 4096, 8192, 100, 8, None) == -1           # bytes not a multiple of 16
+    assert cd.lib().cudadma_scatter_copy(4096, 4096, 8192, 16, 33, 0, None) == -1
+    assert cd.lib().cudadma_probe_memory(3, 4096, 8192, 100, 8, None) == -1           # bytes not a multiple of 16
     assert L.cudadma_probe_memory(99, 4096, 8192, 1024, 8, None) == -3
     assert L.cudadma_fill_permutation(4096, 0, 1, None) == -1
     # workloads: sizes and variants are checked first
@@ -255,7 +270,7 @@ def _fake_run(case_id, case, io, **over):
               in_bytes=io.input.size, out_capacity=io.reps * io.lds_bytes, index_elmts=0)
     kw.update(over)
     r = RunArgs(**kw)
-    return cd.lib().cudadma_run_case(case_id, ctypes.byref(r), None), cd.lib().cudadma_last_error().decode()
+    return cd.harness_lib().cudadma_run_case(case_id, ctypes.byref(r), None), cd.lib().cudadma_last_error().decode()
 
 
 @pytest.mark.parametrize("pattern", [cd.PATTERN_SEQUENTIAL, cd.PATTERN_STRIDED, cd.PATTERN_HALO])

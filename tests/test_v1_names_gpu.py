@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 def _cases():
     try:
-        L = cd.lib()
+        L = cd.harness_lib()
     except cd.CudaDMAError:
         return []
     out = []
@@ -57,7 +57,7 @@ def test_v1_case(case_id):
     d_idx = torch.from_numpy(index).to(dev) if index is not None else None
     d_out = torch.zeros(c.window_bytes, dtype=torch.uint8, device=dev)
     print(f"v1 case {case_id}: {text}", flush=True)
-    cd._lib.check(cd.lib().cudadma_v1_run_case(case_id, ctypes.c_void_p(d_src.data_ptr()),
+    cd._lib.check(cd.harness_lib().cudadma_v1_run_case(case_id, ctypes.c_void_p(d_src.data_ptr()),
                                                ctypes.c_void_p(d_idx.data_ptr()) if d_idx is not None else None,
                                                ctypes.c_void_p(d_out.data_ptr()), None))
     torch.cuda.synchronize()
@@ -69,4 +69,4 @@ def test_v1_case(case_id):
 def test_v1_case_table():
     assert len(_CASES) >= 20
     assert {c.pattern for _, c, _ in _CASES} == {0, 1, 2, 3}
-    assert cd.lib().cudadma_v1_case_text(len(_CASES)) is None
+    assert cd.harness_lib().cudadma_v1_case_text(len(_CASES)) is None
