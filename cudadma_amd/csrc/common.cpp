@@ -27,13 +27,16 @@ static std::vector<StatusSource>& status_sources()
   static std::vector<StatusSource> v;
   return v;
 }
-static std::mutex g_status_mutex;
+static std::mutex g_status_mutex;   // constant-initialised: usable by registrars that run before this unit's own initialisers
 
+// Called from static initialisers: of this library at load time, and of any library loaded later that instantiates
+// DMA objects (the harness), possibly while another thread is inside cudadma_device_status().
 void register_status_source(status_address_fn fn, const char* file)
 {
   StatusSource s{};
   s.address = fn;
   s.file = file;
+  std::lock_guard<std::mutex> lock(g_status_mutex);
   status_sources().push_back(s);
 }
 
@@ -66,6 +69,7 @@ extern "C" int cudadma_device_status(unsigned* status_bits, unsigned* waits_give
 
 extern "C" int cudadma_device_status_sources(void)
 {
+  std::lock_guard<std::mutex> lock(cudadma_host::g_status_mutex);
   return (int)cudadma_host::status_sources().size();
 }
 
