@@ -362,3 +362,21 @@ def test_the_top_level_holds_only_what_belongs_there():
     records = re.compile(r"^(BENCH|GPUTEST|MULTICHIP|SCALE|COPYCHECK|PROGRESS)(_r\d+)?\.(json|jsonl)$")
     strays = [name for name in top if name not in expected and not records.match(name)]
     assert not strays, f"unexpected entries at the repository root: {strays}"
+
+
+def _bench(*args):
+    import sys
+    return subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), *args], capture_output=True, text=True, timeout=300)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The build is for one GPU: asking for more ends with a message that says so, before anything touches a device."""
+    r = _bench("--gpus", "2")
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+@pytest.mark.skipif(__import__("torch").cuda.is_available(), reason="this is the behaviour without a GPU")
+def test_bench_has_no_cpu_path():
+    """Without a GPU the benchmark prints no line and fails: the measured path never falls back to host code."""
+    r = _bench("--gpus", "1", "--steps", "1", "--warmup", "0")
+    assert r.returncode != 0 and "no GPU" in r.stderr and r.stdout.strip() == ""
