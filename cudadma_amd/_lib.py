@@ -11,6 +11,7 @@ PATTERN_SEQUENTIAL, PATTERN_STRIDED, PATTERN_GATHER, PATTERN_SCATTER, PATTERN_HA
  CALL_LDS_DIRECT_SC1, CALL_LDS_DIRECT_NT, CALL_INDEX_AHEAD) = range(17)
 # the qualifier matrix: source known to be global / generic source (the latter also run LDS -> global)
 STATUS_WAIT_GAVE_UP = 1
+NOALLOC_MAX_PHASES = 1 << 20
 CALL_MATRIX_GLOBAL = (CALL_Q_GLOBAL_CG, CALL_Q_LASTUSE_CS, CALL_Q_VOLATILE_WT, CALL_Q_STREAMING_WB)
 CALL_MATRIX_GENERIC = (CALL_QG_GLOBAL_CS, CALL_QG_STREAMING_WT, CALL_QG_LASTUSE_CG, CALL_QG_VOLATILE_WB)
 
@@ -187,6 +188,7 @@ _HARNESS_SIGNATURES = {
     "cudadma_selftest_split_wait": [_vp, _ci, _vp],
     "cudadma_selftest_global_handoff": [_vp, _vp, _ci, _vp],
     "cudadma_selftest_global_handoff_lds_only": [_vp, _vp, _ci, _vp],
+    "cudadma_selftest_global_handoff_noalloc": [_vp, _ci, _vp],
     "cudadma_selftest_all_ids": [_vp, _ci, _vp],
     "cudadma_v1_num_cases": [],
     "cudadma_v1_run_case": [_ci, _vp, _vp, _vp, _vp],

@@ -134,6 +134,18 @@ int cudadma_selftest_bounded_wait(int* d_flags, void* stream);
 int cudadma_selftest_global_handoff(unsigned* d_scratch, int* d_wrong, int phases, void* stream);
 int cudadma_selftest_global_handoff_lds_only(unsigned* d_scratch, int* d_wrong, int phases, void* stream);
 
+/* No counterpart in the reference.  cudadma_selftest_global_handoff() for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the same kernel with
+ * its 16 KiB of staging memory in a device array of the library instead of d_scratch, so the caller passes only the
+ * (zeroed) word for the result.  Calls no hipMalloc, hipFree or other allocating routine.  The need for staging memory
+ * is those 16 KiB whatever the arguments; what bounds the call is `phases`, refused beyond CUDADMA_NOALLOC_MAX_PHASES
+ * with CUDADMA_EINVAL.  The array exists once per device (16 KiB held until the process ends) and keeps the last
+ * call's contents, which no call depends on; two calls that overlap on one device (different streams, or threads)
+ * share it and race: run them one after the other.  The first call on a device looks the array's address up
+ * (hipGetSymbolAddress) and should therefore happen outside a graph capture. */
+#define CUDADMA_NOALLOC_MAX_PHASES (1 << 20)
+int cudadma_selftest_global_handoff_noalloc(int* d_wrong, int phases, void* stream);
+
 /* The split wait that only exists here (peek_dma_finish() + wait_for_dma_finish(peeked),
  * include/hipdma/base.hpp): one workgroup hands a 64-word buffer from a DMA wavefront to a
  * compute wavefront `phases` times, the DMA side early on even and late on odd phases.
