@@ -204,7 +204,7 @@ _QUEUE_DERIVED = (
     ("L1 write latency, cycles (TCP_TCC_WRITE_REQ_LATENCY / WRITE_REQ)", _ratio("TCP_TCC_WRITE_REQ_LATENCY_sum", "TCP_TCC_WRITE_REQ_sum")),
     ("address unit stalled by the L1, share of its busy time (TA_ADDR_STALLED_BY_TC / (256 x GRBM_TA_BUSY / 8))",
      lambda c: c["TA_ADDR_STALLED_BY_TC_CYCLES_sum"] / (32.0 * c["GRBM_TA_BUSY"]) if c.get("GRBM_TA_BUSY") and "TA_ADDR_STALLED_BY_TC_CYCLES_sum" in c else None),
-    ("L1 stalled by the return path from L2, million cycles (TCP_TCR_TCP_STALL)", lambda c: c["TCP_TCR_TCP_STALL_CYCLES_sum"] / 1e6 if "TCP_TCR_TCP_STALL_CYCLES_sum" in c else None),
+    ("L1 stalled by the router between it and the L2, million cycles (TCP_TCR_TCP_STALL)", lambda c: c["TCP_TCR_TCP_STALL_CYCLES_sum"] / 1e6 if "TCP_TCR_TCP_STALL_CYCLES_sum" in c else None),
     ("translation misses in the L1 TLB (UTCL1_TRANSLATION_MISS)", lambda c: c.get("TCP_UTCL1_TRANSLATION_MISS_sum")),
     ("translation requests per memory instruction (UTCL1_REQUEST / (VMEM_RD + VMEM_WR))",
      lambda c: c["TCP_UTCL1_REQUEST_sum"] / (c.get("SQ_INSTS_VMEM_RD", 0) + c.get("SQ_INSTS_VMEM_WR", 0)) if c.get("TCP_UTCL1_REQUEST_sum") and (c.get("SQ_INSTS_VMEM_RD", 0) + c.get("SQ_INSTS_VMEM_WR", 0)) else None),

@@ -11,6 +11,8 @@ point; here the variants are compiled in and the occupancy is a run-time knob.
     python -m cudadma_amd.sweep placement                    # 1 GiB copies against the distance between source and destination
     python -m cudadma_amd.sweep placement_fine               # the copy yardstick alone against 51 distances from 0 to 256 MiB
     python -m cudadma_amd.sweep pattern_yardsticks           # the patterns' own addresses without LDS or objects, next to the patterns
+    python -m cudadma_amd.sweep gather_reach                 # the gather against the size of its table, 128 MiB to 16 GiB
+    python -m cudadma_amd.sweep pattern_pitch                # the tile-shaped reads and writes alone, and the kernel, on matrices whose row pitch is not a power of two
     python -m cudadma_amd.sweep channel_hash                 # which address bits choose the memory channel: half of a 1 GiB buffer by the parity of 1-3 bits
     python -m cudadma_amd.sweep settle                       # the first 80 launches after an idle second, one by one, with the shader clock
     python -m cudadma_amd.sweep two_streams                  # a read-only kernel and a write-only kernel side by side against one copy kernel
@@ -43,6 +45,18 @@ QUEUE_CONFIGS = {
     # (16 KiB elements, four DMA wavefronts, manual double buffering, two workgroups per compute unit)
     "read_cached_1.5wg": ("read", 1.5),
     "probe_cached": ("perf_sequential", "LOAD_CACHE_ALL"), "probe_streaming": ("perf_sequential", "LOAD_CACHE_STREAMING"),
+    # the patterns' own addresses through bare loads or stores (cudadma_probe_pattern): (mode, piece bytes, workgroups per
+    # compute unit, XCD grouping) -- the transposition's destination tiles written in pieces of 256 B (its own shape), 1 KiB and
+    # 4 KiB, its source tiles read, the scatter's permutation written, the gather's index list read from a 4 GiB table
+    "tile_write_256": ("pattern", ("tile_write", 256, 1, 0)), "tile_write_1024": ("pattern", ("tile_write", 1024, 0.5, 0)),
+    "tile_write_4096_grouped": ("pattern", ("tile_write", 4096, 0.5, 1)), "tile_read_256": ("pattern", ("tile_read", 256, 1.5, 0)),
+    "scatter_writes": ("pattern", ("scatter", 0, 1, 0)), "gather_hbm_reads": ("pattern", ("gather_xor", 0, 4, 0)),
+    # the gather of 32 Mi random 128-byte records from a table of 512 MiB and of 4 GiB: bare loads (3 and 4 workgroups per
+    # compute unit) and the reported CudaDMAIndirect kernel
+    "gather_reads": ("pattern", ("gather_xor_small", 0, 3, 0)),
+    "gather_reads_1GiB": ("pattern", ("gather_xor_8Mi", 0, 4, 0)), "gather_reads_2GiB": ("pattern", ("gather_xor_16Mi", 0, 4, 0)),
+    "gather_reads_16GiB": ("pattern", ("gather_xor_128Mi", 0, 4, 0)),
+    "gather_dma": ("pattern", ("gather_dma_small", 0, 0, 0)), "gather_hbm_dma": ("pattern", ("gather_dma", 0, 0, 0)),
 }
 
 
@@ -264,6 +278,43 @@ def main(argv=None):
             ms = _time(lambda: wl.strided_transpose(src, dst, 0), args.steps, settle_ms=20.0)
             print(f"cudadma_strided_transpose variant 0: {pct(2 * n * n * 4, ms)} %", flush=True)
             del pool
+        elif name == "gather_reach":
+            # the gather of 32 Mi random 128-byte records against the size of the table they come from: where the rate leaves
+            # the cache-assisted figure, and where address translation starts to miss (counters: queue_depth gather_*)
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            n_idx = 32 << 20
+            out = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, device=dev)
+            nb = n_idx * 132 + out.numel() * 4
+            for mib in (128, 256, 512, 768, 1024, 1536, 2048, 3072, 4096, 8192, 16384):
+                recs = mib << 13
+                table = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1003)
+                idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=dev), recs, 1003)
+                bare = [nb / _time(lambda: wl.probe_pattern("gather_xor", table, idx, out, cus * wg), args.steps, settle_ms=10.0) / 1e6 / PEAK_GBS * 100
+                        for wg in (3, 4)]
+                dma = nb / _time(lambda: wl.gather_rowsum(table, idx, out, 0), args.steps, settle_ms=10.0) / 1e6 / PEAK_GBS * 100
+                print(f"gather_reach  table {mib:6d} MiB: records read into registers {bare[0]:5.1f} / {bare[1]:5.1f} % at 3 / 4 workgroups per CU; "
+                      f"cudadma_gather_rowsum {dma:5.1f} %", flush=True)
+                del table, idx
+        elif name == "pattern_pitch":
+            # is the transposition's write side held back by the power-of-two row pitch (every row of a tile on the same
+            # low address bits: the same cache channel and set)?  The tile-shaped reads and writes alone and the kernel,
+            # on square matrices of other sizes
+            cus = torch.cuda.get_device_properties(0).multi_processor_count
+            pct = lambda nb, ms: f"{nb / ms / 1e6 / PEAK_GBS * 100:5.1f}"
+            for n in (16384, 16384 + 64, 16384 + 128, 16384 + 512, 16384 + 1024, 16384 - 64, 12288, 8192 + 64, 8192):
+                pool = torch.empty(2 * n * n, device=dev)
+                src = wl.fill_uniform(pool[:n * n], 1002).view(n, n)
+                dst = pool[n * n:].view(n, n)
+                sink = torch.empty(8 * cus * 4, device=dev)
+                nb = n * n * 4
+                reads = [pct(nb, _time(lambda: wl.probe_pattern("tile_read", src, None, sink, int(cus * wg)), args.steps, settle_ms=10.0)) for wg in (1, 1.5, 2)]
+                writes = [pct(nb, _time(lambda: wl.probe_pattern("tile_write", None, None, dst, int(cus * wg)), args.steps, settle_ms=10.0)) for wg in (0.5, 1, 1.5)]
+                kernel = pct(2 * nb, _time(lambda: wl.strided_transpose(src, dst, 0), args.steps, settle_ms=20.0))
+                if not torch.equal(dst, src.t()):
+                    sys.exit(f"transposition of {n} x {n} is wrong")
+                print(f"n = {n:5d} (row pitch {4 * n} B): tile reads alone {' / '.join(reads)} % at (1, 1.5, 2) workgroups per CU; tile writes alone "
+                      f"{' / '.join(writes)} % at (0.5, 1, 1.5); cudadma_strided_transpose variant 0 {kernel} %", flush=True)
+                del pool, src, dst
         elif name == "channel_hash":
             # reads the half of a 1 GiB buffer whose 256-byte granules have even parity under one, two or three address bits:
             # a parity that picks half of the memory channels halves the rate
@@ -341,6 +392,37 @@ def main(argv=None):
                 wl.set_tuning("transpose_workgroups", cus * shape["transpose_workgroups"])
                 fn = lambda: wl.strided_transpose(src.view(16384, 16384), dst.view(16384, 16384), wl.TRANSPOSE_SPLIT_VARIANT)
                 nbytes = 2 * m * 4
+            elif what == "pattern":
+                mode, piece, wg, grouped = shape
+                wl.set_tuning("probe_piece_bytes", piece)
+                wl.set_tuning("probe_xcd_group", grouped)
+                if mode == "scatter":
+                    recs = 4 << 20
+                    records = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1006)
+                    perm = wl.fill_permutation(torch.empty(recs, dtype=torch.int32, device=dev), 1006)
+                    table = torch.empty(recs * wl.REC_FLOATS, device=dev)
+                    fn = lambda: wl.probe_pattern("scatter", records, perm, table, int(cus * wg))
+                    nbytes = recs * 260
+                elif mode.startswith("gather"):
+                    del pool
+                    size = mode.rsplit("_", 1)[-1]                      # records in the table: _small = 4 Mi, _<k>Mi, else 32 Mi
+                    recs = (4 << 20) if size == "small" else (int(size[:-2]) << 20) if size.endswith("Mi") else (32 << 20)
+                    n_idx = 32 << 20
+                    pool = wl.fill_uniform(torch.empty(recs * wl.REC_FLOATS, device=dev), 1003)
+                    idx = wl.fill_indices(torch.empty(n_idx, dtype=torch.int32, device=dev), recs, 1003)
+                    out = torch.empty(n_idx // wl.RECS_PER_TILE * wl.REC_FLOATS, device=dev)
+                    if mode.startswith("gather_dma"):
+                        fn = lambda: wl.gather_rowsum(pool, idx, out, 0)
+                    else:
+                        fn = lambda: wl.probe_pattern("gather_xor", pool, idx, out, int(cus * wg))
+                    nbytes = n_idx * 132 + out.numel() * 4
+                elif mode == "tile_read":
+                    sink = torch.empty(8 * cus * 4, device=dev)
+                    fn = lambda: wl.probe_pattern("tile_read", src.view(16384, 16384), None, sink, int(cus * wg))
+                    nbytes = m * 4
+                else:
+                    fn = lambda: wl.probe_pattern(mode, None, None, dst.view(16384, 16384), int(cus * wg))
+                    nbytes = m * 4
             elif what == "perf_sequential":
                 groups, elmt = 2 * cus, 16 * 1024
                 lq = wl.LOAD_CACHE_STREAMING if shape == "LOAD_CACHE_STREAMING" else wl.LOAD_CACHE_ALL
@@ -354,6 +436,8 @@ def main(argv=None):
             print(f"queue_depth {args.config:22s} {ms:8.4f} ms  {nbytes / ms / 1e6:7.0f} GB/s  {100 * nbytes / ms / 1e6 / PEAK_GBS:5.1f}%", flush=True)
             wl.set_tuning("transpose_split", 0)
             wl.set_tuning("transpose_workgroups", 0)
+            wl.set_tuning("probe_piece_bytes", 0)
+            wl.set_tuning("probe_xcd_group", 0)
             del pool
         elif name == "two_streams":
             # a read-only and a write-only kernel, 1 GiB each, side by side on two streams: do two kernels that each issue one
